@@ -1,0 +1,253 @@
+// Row-wise and element-wise kernels: embedding gather, RMSNorm (with optional row
+// gather), SwiGLU, rotation table, rotation fused with the cache write, type conversion,
+// seeded normal fill.  Formulas follow yusiwen/minfer's CPU path; each kernel names its
+// source.  Statistics, angles and the residual stream are 32-bit.
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+// h[t][:] = table[ids[t]][:], no scaling (src/graph/cpu_backend.rs:269-285).  The host
+// checks ids before upload; an id outside the table gives a row of NaN so that it shows.
+template <typename TT>
+__global__ __launch_bounds__(256) void embed_kernel(const TT* __restrict__ table,
+                                                    const int* __restrict__ ids,
+                                                    float* __restrict__ out, int d, int vocab) {
+  const int row = blockIdx.x;
+  const int id = ids[row];
+  float* o = out + (size_t)row * d;
+  if (id < 0 || id >= vocab) {
+    for (int i = threadIdx.x; i < d; i += 256) o[i] = __builtin_nanf("");
+    return;
+  }
+  const TT* src = table + (size_t)id * d;
+  for (int i = threadIdx.x; i < d; i += 256) o[i] = to_f32(src[i]);
+}
+
+MF_API int mf_embed(const void* table, int table_is_bf16, const int* ids, float* out, int rows,
+                    int d, int vocab, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (table_is_bf16)
+    embed_kernel<bf16><<<rows, 256, 0, stream>>>((const bf16*)table, ids, out, d, vocab);
+  else
+    embed_kernel<float><<<rows, 256, 0, stream>>>((const float*)table, ids, out, d, vocab);
+  return mf_launch_status();
+}
+
+// ---------------------------------------------------------------- RMSNorm
+// y = x * (1/sqrt(mean(x^2) + eps)) * w  (src/vec_ops.rs:500-522; eps inside the root).
+// Row r of the output reads row row_idx[r] of x when row_idx is given.
+template <typename OT>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x,
+                                                      const int* __restrict__ row_idx,
+                                                      const float* __restrict__ w,
+                                                      OT* __restrict__ out, int d, float eps) {
+  __shared__ float scratch[4];
+  const int row = blockIdx.x;
+  const float* xr = x + (size_t)(row_idx ? row_idx[row] : row) * d;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    const float v = xr[i];
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum<256>(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+  OT* o = out + (size_t)row * d;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    const float g = w ? w[i] : 1.0f;
+    o[i] = from_f32<OT>(xr[i] * scale * g);
+  }
+}
+
+MF_API int mf_rmsnorm(const float* x, const int* row_idx, const float* w, void* out,
+                      int out_is_bf16, int rows, int d, float eps, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (out_is_bf16)
+    rmsnorm_kernel<bf16><<<rows, 256, 0, stream>>>(x, row_idx, w, (bf16*)out, d, eps);
+  else
+    rmsnorm_kernel<float><<<rows, 256, 0, stream>>>(x, row_idx, w, (float*)out, d, eps);
+  return mf_launch_status();
+}
+
+// out[r][:] = x[idx[r]][:]  (generic row selection, src/graph/cpu_backend.rs:255-268)
+__global__ __launch_bounds__(256) void gather_rows_kernel(const float* __restrict__ x,
+                                                          const int* __restrict__ idx,
+                                                          float* __restrict__ out, int d) {
+  const float* src = x + (size_t)idx[blockIdx.x] * d;
+  float* o = out + (size_t)blockIdx.x * d;
+  for (int i = threadIdx.x; i < d; i += 256) o[i] = src[i];
+}
+
+MF_API int mf_gather_rows(const float* x, const int* idx, float* out, int rows, int d,
+                          hipStream_t stream) {
+  if (rows <= 0) return 0;
+  gather_rows_kernel<<<rows, 256, 0, stream>>>(x, idx, out, d);
+  return mf_launch_status();
+}
+
+// ---------------------------------------------------------------- SwiGLU
+// y[r][i] = silu(g[r][i]) * u[r][i], silu(z) = z / (1 + exp(-z))
+// (src/vec_ops.rs:131-146, src/graph/cpu_backend.rs:323-329).  g and u are the two halves
+// of one [rows][2*nf] buffer.
+template <typename IT, typename OT>
+__global__ __launch_bounds__(256) void swiglu_kernel(const IT* __restrict__ gu, OT* __restrict__ out,
+                                                     int nf) {
+  const IT* g = gu + (size_t)blockIdx.y * 2 * nf;
+  const IT* u = g + nf;
+  OT* o = out + (size_t)blockIdx.y * nf;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < nf) {
+    const float z = to_f32(g[i]);
+    o[i] = from_f32<OT>(z / (1.0f + expf(-z)) * to_f32(u[i]));
+  }
+}
+
+MF_API int mf_swiglu(const void* gu, int in_is_bf16, void* out, int out_is_bf16, int rows, int nf,
+                     hipStream_t stream) {
+  if (rows <= 0) return 0;
+  dim3 grid((nf + 255) / 256, rows);
+  if (in_is_bf16 && out_is_bf16)
+    swiglu_kernel<bf16, bf16><<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, nf);
+  else if (!in_is_bf16 && out_is_bf16)
+    swiglu_kernel<float, bf16><<<grid, 256, 0, stream>>>((const float*)gu, (bf16*)out, nf);
+  else if (!in_is_bf16 && !out_is_bf16)
+    swiglu_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)gu, (float*)out, nf);
+  else
+    return (int)hipErrorInvalidValue;
+  return mf_launch_status();
+}
+
+// ---------------------------------------------------------------- type conversion
+template <typename IT, typename OT>
+__global__ __launch_bounds__(256) void convert_kernel(const IT* __restrict__ in, OT* __restrict__ out,
+                                                      size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+    out[i] = from_f32<OT>(to_f32(in[i]));
+}
+
+MF_API int mf_convert(const void* in, int in_is_bf16, void* out, int out_is_bf16, size_t n,
+                      hipStream_t stream) {
+  if (n == 0) return 0;
+  const int blocks = (int)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  if (in_is_bf16 && !out_is_bf16)
+    convert_kernel<bf16, float><<<blocks, 256, 0, stream>>>((const bf16*)in, (float*)out, n);
+  else if (!in_is_bf16 && out_is_bf16)
+    convert_kernel<float, bf16><<<blocks, 256, 0, stream>>>((const float*)in, (bf16*)out, n);
+  else
+    return (int)hipErrorInvalidValue;
+  return mf_launch_status();
+}
+
+// ---------------------------------------------------------------- rotation
+// cos/sin[pos][i] of angle = pos * scale / theta^(2i/hd), computed in double and rounded
+// once (the reference forms the same angle in f32 per element and call,
+// src/graph/cpu_backend.rs:403-420).
+__global__ __launch_bounds__(256) void rope_table_kernel(float* __restrict__ cs, float* __restrict__ sn,
+                                                         int n_pos, int half, double theta,
+                                                         double freq_scale) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n_pos * half) return;
+  const int pos = idx / half, i = idx % half;
+  const double freq = freq_scale / pow(theta, (2.0 * i) / (2.0 * half));
+  const double ang = (double)pos * freq;
+  cs[idx] = (float)cos(ang);
+  sn[idx] = (float)sin(ang);
+}
+
+MF_API int mf_rope_table(float* cs, float* sn, int n_pos, int half, double theta,
+                         double freq_scale, hipStream_t stream) {
+  const int n = n_pos * half;
+  if (n <= 0) return 0;
+  rope_table_kernel<<<(n + 255) / 256, 256, 0, stream>>>(cs, sn, n_pos, half, theta, freq_scale);
+  return mf_launch_status();
+}
+
+// Half-split rotation of q and k (pair i with i + hd/2; x0' = x0 c - x1 s, x1' = x0 s + x1 c;
+// src/graph/cpu_backend.rs:421-431), v copied, k and v stored into the paged cache at the
+// token's position before attention reads it (src/graph/cpu_backend.rs:118-149).
+// qkv is [T][(nh + 2 nk) hd] in 32-bit with biases already added.  One block per
+// (token, head of q|k|v).
+template <typename OT>
+__global__ __launch_bounds__(64) void rope_kvwrite_kernel(
+    const float* __restrict__ qkv, const float* __restrict__ cs, const float* __restrict__ sn,
+    const int* __restrict__ positions, const int* __restrict__ seq_of_tok,
+    const int* __restrict__ page_table, int pt_stride, OT* __restrict__ q_out,
+    OT* __restrict__ kcache, OT* __restrict__ vcache, int nh, int nk, int hd, int write_kv) {
+  const int t = blockIdx.x, head = blockIdx.y;
+  const int half = hd >> 1;
+  const int pos = positions[t];
+  const float* src = qkv + ((size_t)t * (nh + 2 * nk) + head) * hd;
+  if (head < nh) {
+    OT* dst = q_out + ((size_t)t * nh + head) * hd;
+    for (int i = threadIdx.x; i < half; i += 64) {
+      const float c = cs[(size_t)pos * half + i], s = sn[(size_t)pos * half + i];
+      const float x0 = src[i], x1 = src[i + half];
+      dst[i] = from_f32<OT>(x0 * c - x1 * s);
+      dst[i + half] = from_f32<OT>(x0 * s + x1 * c);
+    }
+    return;
+  }
+  if (!write_kv) return;
+  const int page = page_table[(size_t)seq_of_tok[t] * pt_stride + pos / MF_PAGE];
+  if (page < 0) return;
+  const bool is_k = head < nh + nk;
+  const int hk = is_k ? head - nh : head - nh - nk;
+  OT* dst = (is_k ? kcache : vcache) + (((size_t)page * nk + hk) * MF_PAGE + pos % MF_PAGE) * hd;
+  if (is_k) {
+    for (int i = threadIdx.x; i < half; i += 64) {
+      const float c = cs[(size_t)pos * half + i], s = sn[(size_t)pos * half + i];
+      const float x0 = src[i], x1 = src[i + half];
+      dst[i] = from_f32<OT>(x0 * c - x1 * s);
+      dst[i + half] = from_f32<OT>(x0 * s + x1 * c);
+    }
+  } else {
+    for (int i = threadIdx.x; i < hd; i += 64) dst[i] = from_f32<OT>(src[i]);
+  }
+}
+
+MF_API int mf_rope_kvwrite(const float* qkv, const float* cs, const float* sn, const int* positions,
+                           const int* seq_of_tok, const int* page_table, int pt_stride, void* q_out,
+                           void* kcache, void* vcache, int is_bf16, int n_tok, int nh, int nk, int hd,
+                           int write_kv, hipStream_t stream) {
+  if (n_tok <= 0) return 0;
+  dim3 grid(n_tok, write_kv ? nh + 2 * nk : nh);
+  if (is_bf16)
+    rope_kvwrite_kernel<bf16><<<grid, 64, 0, stream>>>(qkv, cs, sn, positions, seq_of_tok, page_table,
+                                                       pt_stride, (bf16*)q_out, (bf16*)kcache,
+                                                       (bf16*)vcache, nh, nk, hd, write_kv);
+  else
+    rope_kvwrite_kernel<float><<<grid, 64, 0, stream>>>(qkv, cs, sn, positions, seq_of_tok, page_table,
+                                                        pt_stride, (float*)q_out, (float*)kcache,
+                                                        (float*)vcache, nh, nk, hd, write_kv);
+  return mf_launch_status();
+}
+
+// ---------------------------------------------------------------- seeded normal fill
+// value(i) depends only on (seed, i): two hashed uniforms through Box-Muller.
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+template <typename OT>
+__global__ __launch_bounds__(256) void fill_normal_kernel(OT* __restrict__ out, size_t n, uint64_t seed,
+                                                          float std) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    const uint64_t h = mix64(seed ^ mix64(i));
+    const float u1 = ((float)(uint32_t)(h >> 40) + 1.0f) * (1.0f / 16777216.0f);   // (0,1]
+    const float u2 = (float)(uint32_t)((h >> 8) & 0xFFFFFF) * (1.0f / 16777216.0f);  // [0,1)
+    const float r = sqrtf(-2.0f * logf(u1));
+    out[i] = from_f32<OT>(r * cosf(6.28318530717958647692f * u2) * std);
+  }
+}
+
+MF_API int mf_fill_normal(void* out, int is_bf16, size_t n, uint64_t seed, float std,
+                          hipStream_t stream) {
+  if (n == 0) return 0;
+  const int blocks = (int)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  if (is_bf16)
+    fill_normal_kernel<bf16><<<blocks, 256, 0, stream>>>((bf16*)out, n, seed, std);
+  else
+    fill_normal_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, n, seed, std);
+  return mf_launch_status();
+}

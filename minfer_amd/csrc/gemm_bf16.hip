@@ -1,0 +1,309 @@
+// bfloat16 matrix products on the gfx950 matrix cores, 32-bit accumulation:
+//   C[M][N] (+)= A[M][K] * W[N][K]^T (+ bias[N])
+// (out[t][o] = dot(W[o][:], x[t][:]) + b[o], src/graph/cpu_backend.rs:214-248 of
+// yusiwen/minfer; the reference's own matrix kernels are quantised and are not followed.)
+//
+// Two kernels:
+//  * `tile_kernel`: many rows (prompts).  A BM x BN block tile per 256 threads, K walked
+//    in steps of 64 through double-buffered LDS, 32x32x16 MFMA, each wave a WM x WN tile.
+//  * `skinny_kernel`: at most 64 rows (decode).  The time is the weight stream: each wave
+//    owns 16 weight rows and reads them from HBM straight into MFMA operands (16x16x32),
+//    the few activation rows are staged in LDS and shared by the block, K may be split
+//    over blocks with a fixed-order reduction afterwards.
+// Both operands have K contiguous, which is exactly the MFMA operand layout (8 consecutive
+// k per lane), so nothing is transposed.
+//
+// Epilogues: 0 store fp32, 1 add into fp32 (residual stream), 2 store bf16.
+#include "common.h"
+
+namespace {
+
+enum { EPI_F32 = 0, EPI_ACC_F32 = 1, EPI_BF16 = 2 };
+
+__device__ __forceinline__ void store_out(void* C, int ldc, int m, int n, float v, int epi) {
+  if (epi == EPI_BF16) {
+    ((bf16*)C)[(size_t)m * ldc + n] = (bf16)v;
+  } else {
+    float* c = (float*)C + (size_t)m * ldc + n;
+    *c = (epi == EPI_ACC_F32) ? *c + v : v;
+  }
+}
+
+// 8 consecutive k of one row, zero outside the matrix; vector load when aligned.
+__device__ __forceinline__ bf16x8 load8(const bf16* __restrict__ base, int ld, int row, int rows, int k,
+                                        int K, bool vec_ok) {
+  bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (row < rows && k < K) {
+    const bf16* p = base + (size_t)row * ld + k;
+    if (vec_ok && k + 8 <= K) {
+      v = *reinterpret_cast<const bf16x8*>(p);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (k + e < K) v[e] = p[e];
+    }
+  }
+  return v;
+}
+
+// ------------------------------------------------------------------ tiled kernel
+constexpr int BK = 64;
+constexpr int LDS_LD = BK + 8;   // row stride in elements: 144 bytes, conflict-free b128 reads
+
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(256) void tile_kernel(const bf16* __restrict__ A, int lda,
+                                                   const bf16* __restrict__ W, int ldw,
+                                                   const float* __restrict__ bias, void* __restrict__ C,
+                                                   int ldc, int M, int N, int K, int epi, int vec_ok,
+                                                   int tiles_m) {
+  static_assert((BM / WM) * (BN / WN) == 4, "four waves per block");
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int PA = BM / 32, PW = BN / 32;   // load passes: 32 rows x 64 k per pass
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  bf16* As = reinterpret_cast<bf16*>(smem);               // [2][BM][LDS_LD]
+  bf16* Ws = As + 2 * BM * LDS_LD;                        // [2][BN][LDS_LD]
+
+  // Consecutive blocks walk down M first, so blocks that run together share W tiles.
+  const int bm = blockIdx.x % tiles_m, bn = blockIdx.x / tiles_m;
+  const int m0 = bm * BM, n0 = bn * BN;
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  const int wm = (wid % (BM / WM)) * WM, wn = (wid / (BM / WM)) * WN;
+  const int lrow = tid >> 3, lk = (tid & 7) * 8;
+  const int fr = lane & 31, fk = (lane >> 5) * 8;
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  bf16x8 ra[PA], rw[PW];
+  const int nkt = (K + BK - 1) / BK;
+#pragma unroll
+  for (int p = 0; p < PA; ++p) ra[p] = load8(A, lda, m0 + p * 32 + lrow, M, lk, K, vec_ok);
+#pragma unroll
+  for (int p = 0; p < PW; ++p) rw[p] = load8(W, ldw, n0 + p * 32 + lrow, N, lk, K, vec_ok);
+#pragma unroll
+  for (int p = 0; p < PA; ++p)
+    *reinterpret_cast<bf16x8*>(&As[(p * 32 + lrow) * LDS_LD + lk]) = ra[p];
+#pragma unroll
+  for (int p = 0; p < PW; ++p)
+    *reinterpret_cast<bf16x8*>(&Ws[(p * 32 + lrow) * LDS_LD + lk]) = rw[p];
+  __syncthreads();
+
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int cur = kt & 1;
+    const bool more = kt + 1 < nkt;
+    if (more) {
+      const int k = (kt + 1) * BK + lk;
+#pragma unroll
+      for (int p = 0; p < PA; ++p) ra[p] = load8(A, lda, m0 + p * 32 + lrow, M, k, K, vec_ok);
+#pragma unroll
+      for (int p = 0; p < PW; ++p) rw[p] = load8(W, ldw, n0 + p * 32 + lrow, N, k, K, vec_ok);
+    }
+    const bf16* as = As + cur * BM * LDS_LD;
+    const bf16* ws = Ws + cur * BN * LDS_LD;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      bf16x8 fa[TM], fw[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        fa[i] = *reinterpret_cast<const bf16x8*>(&as[(wm + i * 32 + fr) * LDS_LD + ks * 16 + fk]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        fw[j] = *reinterpret_cast<const bf16x8*>(&ws[(wn + j * 32 + fr) * LDS_LD + ks * 16 + fk]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      bf16* an = As + (cur ^ 1) * BM * LDS_LD;
+      bf16* wn_ = Ws + (cur ^ 1) * BN * LDS_LD;
+#pragma unroll
+      for (int p = 0; p < PA; ++p)
+        *reinterpret_cast<bf16x8*>(&an[(p * 32 + lrow) * LDS_LD + lk]) = ra[p];
+#pragma unroll
+      for (int p = 0; p < PW; ++p)
+        *reinterpret_cast<bf16x8*>(&wn_[(p * 32 + lrow) * LDS_LD + lk]) = rw[p];
+    }
+    __syncthreads();
+  }
+
+  // D[m][n]: lane holds n = lane % 32, m = 8 (r / 4) + 4 (lane / 32) + r % 4
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn + j * 32 + fr;
+      if (n >= N) continue;
+      const float b = bias ? bias[n] : 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        if (m < M) store_out(C, ldc, m, n, acc[i][j][r] + b, epi);
+      }
+    }
+}
+
+template <int BM, int BN, int WM, int WN>
+int launch_tile(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
+                int M, int N, int K, int epi, int vec_ok, hipStream_t stream) {
+  constexpr int smem = 2 * (BM + BN) * LDS_LD * (int)sizeof(bf16);
+  static bool configured = false;
+  auto kern = tile_kernel<BM, BN, WM, WN>;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    configured = true;
+  }
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  kern<<<tiles_m * tiles_n, 256, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, vec_ok,
+                                                 tiles_m);
+  return mf_launch_status();
+}
+
+// ------------------------------------------------------------------ skinny kernel
+constexpr int KC = 256;          // k per staging step
+constexpr int SK_LD = KC + 8;    // LDS row stride in elements
+
+// Partial sums go to part[split][M][N]; with one split the epilogue runs in place.
+template <int MT>
+__global__ __launch_bounds__(256) void skinny_kernel(const bf16* __restrict__ A, int lda,
+                                                     const bf16* __restrict__ W, int ldw,
+                                                     const float* __restrict__ bias, void* __restrict__ C,
+                                                     int ldc, float* __restrict__ part, int M, int N,
+                                                     int K, int k_per_split, int epi, int vec_ok) {
+  __shared__ __attribute__((aligned(16))) bf16 As[MT * 16 * SK_LD];
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  const int n_row = blockIdx.x * 64 + wid * 16 + (lane & 15);   // weight row of this lane
+  const int kq = (lane >> 4) * 8;                               // k offset inside a 32-step
+  const int k_begin = blockIdx.y * k_per_split;
+  const int k_end = min(K, k_begin + k_per_split);
+
+  floatx4 acc[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  bf16x8 wcur[KC / 32], wnext[KC / 32];
+#pragma unroll
+  for (int s = 0; s < KC / 32; ++s)
+    wcur[s] = load8(W, ldw, n_row, N, k_begin + s * 32 + kq, k_end, vec_ok);
+
+  for (int k0 = k_begin; k0 < k_end; k0 += KC) {
+    __syncthreads();
+    // stage A[0..16 MT)[k0..k0+KC): 32 chunks of 8 per row
+    for (int c = tid; c < MT * 16 * (KC / 8); c += 256) {
+      const int r = c / (KC / 8), kk = (c % (KC / 8)) * 8;
+      *reinterpret_cast<bf16x8*>(&As[r * SK_LD + kk]) = load8(A, lda, r, M, k0 + kk, k_end, vec_ok);
+    }
+    __syncthreads();
+    if (k0 + KC < k_end) {
+#pragma unroll
+      for (int s = 0; s < KC / 32; ++s)
+        wnext[s] = load8(W, ldw, n_row, N, k0 + KC + s * 32 + kq, k_end, vec_ok);
+    }
+#pragma unroll
+    for (int s = 0; s < KC / 32; ++s) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const bf16x8 a =
+            *reinterpret_cast<const bf16x8*>(&As[(i * 16 + (lane & 15)) * SK_LD + s * 32 + kq]);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, wcur[s], acc[i], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < KC / 32; ++s) wcur[s] = wnext[s];
+  }
+
+  // D[m][n]: lane holds n = lane % 16, m = 4 (lane / 16) + r
+  if (n_row >= N) return;
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = i * 16 + (lane >> 4) * 4 + r;
+      if (m >= M) continue;
+      if (part) {
+        part[((size_t)blockIdx.y * M + m) * N + n_row] = acc[i][r];
+      } else {
+        store_out(C, ldc, m, n_row, acc[i][r] + (bias ? bias[n_row] : 0.f), epi);
+      }
+    }
+}
+
+__global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restrict__ part,
+                                                            const float* __restrict__ bias,
+                                                            void* __restrict__ C, int ldc, int M, int N,
+                                                            int splits, int epi) {
+  const int n = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
+  if (n >= N) return;
+  float v = 0.f;
+  for (int s = 0; s < splits; ++s) v += part[((size_t)s * M + m) * N + n];
+  store_out(C, ldc, m, n, v + (bias ? bias[n] : 0.f), epi);
+}
+
+template <int MT>
+int launch_skinny(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
+                  float* part, int M, int N, int K, int splits, int k_per_split, int epi, int vec_ok,
+                  hipStream_t stream) {
+  dim3 grid((N + 63) / 64, splits);
+  skinny_kernel<MT><<<grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, splits > 1 ? part : nullptr,
+                                              M, N, K, k_per_split, epi, vec_ok);
+  int rc = mf_launch_status();
+  if (rc == 0 && splits > 1) {
+    dim3 g2((N + 255) / 256, M);
+    skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, splits, epi);
+    rc = mf_launch_status();
+  }
+  return rc;
+}
+
+}  // namespace
+
+// `variant`: 0 picks by shape; 1: 256x256 tile, 2: 128x128, 3: 64x64 (tests name them).
+MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
+                        int ldc, int M, int N, int K, int epi, int variant, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || ldw < K || ldc < N || epi < 0 || epi > 2) return (int)hipErrorInvalidValue;
+  const int vec_ok = (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) &&
+                     ((uintptr_t)W % 16 == 0);
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  if (variant == 0) {
+    const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+    const long t128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    variant = (t256 >= 512) ? 1 : (t128 >= 64 || M > 64) ? 2 : 3;
+  }
+  switch (variant) {
+    case 1: return launch_tile<256, 256, 128, 128>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case 2: return launch_tile<128, 128, 64, 64>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case 3: return launch_tile<64, 64, 32, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+// M <= 64.  `part` holds splits*M*N floats when splits > 1; k_per_split is a multiple of 256.
+MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, const float* bias,
+                               void* C, int ldc, float* part, int M, int N, int K, int splits,
+                               int k_per_split, int epi, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || lda < K || ldw < K || ldc < N || epi < 0 || epi > 2 || splits < 1 ||
+      k_per_split % KC != 0 || (long)splits * k_per_split < K || (splits > 1 && !part))
+    return (int)hipErrorInvalidValue;
+  const int vec_ok = (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) &&
+                     ((uintptr_t)W % 16 == 0);
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  switch ((M + 15) / 16) {
+    case 1: return launch_skinny<1>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
+    case 2: return launch_skinny<2>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
+    case 3: return launch_skinny<3>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
+    case 4: return launch_skinny<4>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
+  }
+  return (int)hipErrorInvalidValue;
+}

@@ -1,0 +1,40 @@
+"""The ragged batch of one step as the parts see it.
+
+All sequences' new tokens are concatenated: token t belongs to sequence `seq_of_tok[t]`
+(an index into the step's batch, not a slot) and sits at absolute position `positions[t]`;
+it attends to its own sequence's cache rows up to that position and to nothing else.
+Positions are data, never structure (src/graph/ops.rs:3-6 of yusiwen/minfer), and a step's
+keys are stored before its attention reads them (src/graph/scheduler.rs:12-15).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+
+import torch
+
+
+@dataclass
+class StepContext:
+    cache: object                        # minfer_amd.cache.Cache
+    n_tokens: int
+    n_seqs: int
+    token_ids: torch.Tensor              # int32 [n_tokens]
+    positions: torch.Tensor              # int32 [n_tokens]
+    seq_of_tok: torch.Tensor             # int32 [n_tokens]
+    cu_seqlens: torch.Tensor             # int32 [n_seqs + 1], offsets of each sequence's tokens
+    start_pos: torch.Tensor              # int32 [n_seqs], tokens each sequence held before the step
+    slot_ids: torch.Tensor               # int32 [n_seqs], cache slot of each sequence
+    logit_rows: Optional[torch.Tensor]   # int32 [n_wanted] rows of the step whose logits are wanted
+    page_tables: Dict[int, torch.Tensor]  # id(group) -> int32 [n_seqs][n_cols]
+    max_len: int                         # bound on position + 1 over the step's tokens
+    max_new: int                         # longest run of new tokens of one sequence
+    all_decode: bool                     # every sequence brings exactly one token
+    # host copies, for parts that plan on the host (and for toy parts in tests)
+    host_slots: List[int] = field(default_factory=list)
+    host_new: List[int] = field(default_factory=list)
+    host_start: List[int] = field(default_factory=list)
+    new_lengths: Dict[int, int] = field(default_factory=dict)   # slot -> tokens held after the step
+
+    def page_table(self, group) -> torch.Tensor:
+        return self.page_tables[id(group)]

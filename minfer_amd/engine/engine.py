@@ -1,0 +1,133 @@
+"""The step function: a batch of sequences with unequal numbers of new tokens, run as one
+ragged batch from the cache, logits returned at the wanted places.
+
+The reference's step is `forward(tokens, positions, n_out) -> n_out x vocab logits` for one
+sequence per call, with a prompt as one call and then one token per call
+(src/models/mod.rs:21-22, src/models/qwen2/graph.rs:276-408, src/main.rs:497-502,595 of
+yusiwen/minfer); a batch there is one call per cache (src/server/chat.rs:218-249).  Here the
+whole batch is one call: tokens of all sequences concatenated, per-token position and
+sequence index as data.  There is no padding: only the tokens given are run.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Union
+
+import numpy as np
+import torch
+
+from ..cache.paged import PAGE, Cache, CacheError
+from .batch import StepContext
+from .model import DecoderModel
+
+Want = Union[str, Sequence[Sequence[int]]]
+
+
+class StepError(ValueError):
+    """A step that cannot run: the message says which sequence and why.  Nothing changed."""
+
+
+class Engine:
+    def __init__(self, model: DecoderModel, max_tokens: int, max_seqs: Optional[int] = None):
+        if not model.loaded:
+            raise RuntimeError("Engine needs a model with weights")
+        self.model = model
+        self.device = model.rt.device
+        n_pages = (max_tokens + PAGE - 1) // PAGE
+        self.max_seqs = int(max_seqs) if max_seqs else max(1, min(n_pages, 1024))
+        self.cache = Cache(model.cache_requests(), max_tokens, self.max_seqs, model.rt.dtype, self.device)
+        self.vocab_size = model.spec.vocab_size
+        self.max_positions = model.spec.max_positions
+
+    # ------------------------------------------------------------ sequences
+    def new_sequence(self) -> int:
+        """Takes a cache slot for a sequence that starts at position 0."""
+        return self.cache.alloc_slot()
+
+    def end_sequence(self, slot: int) -> None:
+        """Gives the slot and everything it holds back."""
+        self.cache.free_slot(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    # ------------------------------------------------------------ one step
+    def build_context(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], want: Want) -> StepContext:
+        """Checks the step, reserves its cache pages and uploads its metadata in one copy."""
+        if len(slots) != len(tokens) or not slots:
+            raise StepError("a step needs at least one sequence and as many token lists as slots")
+        if len(set(slots)) != len(slots):
+            raise StepError(f"a slot appears twice in one step: {list(slots)}")
+        n_new = [len(t) for t in tokens]
+        start, new_len = [], {}
+        for b, (s, n) in enumerate(zip(slots, n_new)):
+            if n < 1:
+                raise StepError(f"sequence {b} (slot {s}) brings no tokens")
+            try:
+                cur = self.cache.length(s)
+            except CacheError as e:
+                raise StepError(str(e)) from None
+            if cur + n > self.max_positions:
+                raise StepError(f"sequence {b} (slot {s}): position {cur + n - 1} exceeds the model's "
+                                f"{self.max_positions} positions")
+            start.append(cur)
+            new_len[s] = cur + n
+        flat = np.fromiter((t for seq in tokens for t in seq), dtype=np.int64, count=sum(n_new))
+        if flat.min() < 0 or flat.max() >= self.vocab_size:
+            bad = int(flat[(flat < 0) | (flat >= self.vocab_size)][0])
+            raise StepError(f"embedding id {bad} >= vocab {self.vocab_size}" if bad >= 0
+                            else f"embedding id {bad} is negative")
+        n_tok, n_seq = int(flat.size), len(slots)
+        cu = np.zeros(n_seq + 1, dtype=np.int64)
+        cu[1:] = np.cumsum(n_new)
+        if isinstance(want, str):
+            if want == "last":
+                rows: Optional[np.ndarray] = cu[1:] - 1
+            elif want == "all":
+                rows = None
+            else:
+                raise StepError(f"want must be 'last', 'all' or per-sequence offsets, got {want!r}")
+        else:
+            if len(want) != n_seq:
+                raise StepError("want needs one list of offsets per sequence")
+            picked = []
+            for b, offs in enumerate(want):
+                for o in offs:
+                    if not 0 <= int(o) < n_new[b]:
+                        raise StepError(f"sequence {b}: wanted offset {o} outside its {n_new[b]} new tokens")
+                    picked.append(cu[b] + int(o))
+            rows = np.asarray(picked, dtype=np.int64)
+
+        self.cache.reserve(new_len)          # CacheFull leaves everything as it was
+        max_len = max(new_len.values())
+        self.model.prepare(max_len)
+        n_cols = (max_len + PAGE - 1) // PAGE
+        seq_of_tok = np.repeat(np.arange(n_seq), n_new)
+        positions = np.concatenate([np.arange(s, s + n) for s, n in zip(start, n_new)])
+        pieces = [flat, positions, seq_of_tok, cu, np.asarray(start), np.asarray(slots),
+                  rows if rows is not None else np.zeros(0, dtype=np.int64)]
+        for g in self.cache.groups:
+            pieces.append(np.asarray(self.cache.page_rows(g, slots, n_cols), dtype=np.int64).reshape(-1))
+        packed = np.concatenate(pieces).astype(np.int32)
+        dev = torch.from_numpy(packed).to(self.device)
+        views, off = [], 0
+        for p in pieces:
+            views.append(dev[off:off + p.size])
+            off += p.size
+        tables = {id(g): views[7 + i].view(n_seq, n_cols) for i, g in enumerate(self.cache.groups)}
+        ctx = StepContext(
+            cache=self.cache, n_tokens=n_tok, n_seqs=n_seq, token_ids=views[0], positions=views[1],
+            seq_of_tok=views[2], cu_seqlens=views[3], start_pos=views[4], slot_ids=views[5],
+            logit_rows=None if rows is None else views[6], page_tables=tables, max_len=max_len,
+            max_new=max(n_new), all_decode=all(n == 1 for n in n_new),
+            host_slots=list(slots), host_new=n_new, host_start=start)
+        ctx.new_lengths = new_len
+        return ctx
+
+    def step(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], want: Want = "last") -> torch.Tensor:
+        """Runs the given new tokens of each sequence (after what its slot already holds) and
+        returns float32 logits `[wanted][vocab]`, ordered by sequence and then by offset.
+        `want`: 'last' (each sequence's last new token), 'all', or offsets per sequence."""
+        ctx = self.build_context(slots, tokens, want)
+        logits = self.model.forward(ctx)
+        self.cache.commit(ctx.new_lengths)
+        return logits

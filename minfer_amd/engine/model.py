@@ -1,0 +1,106 @@
+"""A decoder model put together from a `ModelSpec`: embedding, blocks in their run order,
+final norm, head.  Which parts, with which constants, comes from the spec alone.
+
+One step (src/models/qwen2/graph.rs:36-185 of yusiwen/minfer): rows of the embedding table
+-> every entry of the run order -> only the wanted rows go through the last block's
+feed-forward, the final norm and the head (the reference's tail-row reduction,
+graph.rs:126-138) -> float32 logits.
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, List, Optional
+
+import torch
+
+from ..kernels import ops
+from ..parts.base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Runtime, make_part)
+from ..parts.linear import Linear
+from ..parts.spec import BlockSpec, ModelSpec
+from ..weights.loader import TensorSpec
+
+
+def _build_block(bs: BlockSpec, rt: Runtime):
+    if bs.kind not in BLOCKS:
+        raise KeyError(f"unknown block arrangement {bs.kind!r}; registered: {', '.join(sorted(BLOCKS))}")
+    return BLOCKS[bs.kind](
+        make_part(MIXERS, bs.mixer, rt, "mixer"),
+        make_part(FEED_FORWARDS, bs.feed_forward, rt, "feed-forward"),
+        make_part(NORMS, bs.mixer_norm, rt, "norm"),
+        make_part(NORMS, bs.feed_forward_norm, rt, "norm"), rt)
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"run type must be float32 or bfloat16, got {dtype}")
+        self.spec = spec
+        self.rt = Runtime(dtype=dtype, device=torch.device(device))
+        self.blocks = [_build_block(bs, self.rt) for bs in spec.blocks]
+        self.final_norm = make_part(NORMS, spec.final_norm, self.rt, "norm")
+        self.embedding: Optional[torch.Tensor] = None
+        self.head: Optional[Linear] = None
+        self.loaded = False
+
+    # ------------------------------------------------------------ tensors
+    def expected_tensors(self) -> Dict[str, TensorSpec]:
+        s = self.spec
+        out = {s.embedding_name: TensorSpec((s.vocab_size, s.hidden_size))}
+        if s.head_name is not None:
+            out[s.head_name] = TensorSpec((s.vocab_size, s.hidden_size))
+        out.update(self.final_norm.tensor_specs())
+        for bs, block in zip(s.blocks, self.blocks):
+            for part in block.parts():
+                for name, ts in part.tensor_specs().items():
+                    full = bs.prefix + name
+                    if full in out:
+                        raise ValueError(f"tensor {full!r} is claimed by two parts")
+                    out[full] = ts
+        return out
+
+    def load(self, get: Callable[[str], torch.Tensor]) -> None:
+        """`get(full name)` returns a device tensor in its storage type."""
+        s = self.spec
+        self.embedding = get(s.embedding_name).contiguous()
+        # tied head: the same storage, no second copy (src/models/qwen2/loader.rs:260)
+        self.head = Linear(self.embedding if s.head_name is None else get(s.head_name))
+        self.final_norm.load(get)
+        for bs, block in zip(s.blocks, self.blocks):
+            for part in block.parts():
+                part.load(lambda name, p=bs.prefix: get(p + name))
+        self.loaded = True
+
+    # ------------------------------------------------------------ cache needs
+    def cache_requests(self) -> Dict[int, object]:
+        """cache entry -> what the mixer that writes it asks for."""
+        return {e.cache: self.blocks[e.block].mixer.cache_request()
+                for e in self.spec.schedule if e.writes_cache}
+
+    def prepare(self, max_len: int) -> None:
+        for block in self.blocks:
+            for part in block.parts():
+                part.prepare(max_len)
+
+    # ------------------------------------------------------------ the step
+    def forward(self, ctx) -> torch.Tensor:
+        """float32 logits [n_wanted][vocab] for ctx.logit_rows (all rows when None)."""
+        if not self.loaded:
+            raise RuntimeError("model has no weights yet")
+        s = self.spec
+        h = torch.empty((ctx.n_tokens, s.hidden_size), dtype=torch.float32, device=self.rt.device)
+        ops.embed(self.embedding, ctx.token_ids, h)
+        rows = ctx.logit_rows
+        last = len(s.schedule) - 1
+        for n, e in enumerate(s.schedule):
+            keep = rows if (n == last and rows is not None) else None
+            h = self.blocks[e.block].forward(h, ctx, e.cache, e.writes_cache, keep_rows=keep)
+        if not s.schedule and rows is not None:
+            kept = torch.empty((rows.numel(), s.hidden_size), dtype=torch.float32, device=h.device)
+            ops.gather_rows(h, rows, kept)
+            h = kept
+        x = self.final_norm.forward(h)
+        return self.head(x, out_dtype=torch.float32)
+
+
+def expected_tensors(spec: ModelSpec) -> Dict[str, TensorSpec]:
+    """Names, shapes and fill rules of a spec's tensors, without touching a device."""
+    return DecoderModel(spec, torch.float32, "cpu").expected_tensors()

@@ -1,0 +1,310 @@
+"""Python faces of the HIP kernels: each function checks its operands on the host (device,
+type, shape, contiguity), then launches on torch's current stream.  Outputs are written
+into tensors the caller allocated, so a captured step allocates nothing here except the
+cached workspaces below.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_double, c_float, c_int, c_size_t, c_uint64, c_void_p
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import build
+
+PAGE = 64          # tokens per cache page (MF_PAGE in csrc/common.h)
+HAVE_PREFILL_ATTENTION = False
+EPI_F32, EPI_ACC_F32, EPI_BF16 = 0, 1, 2
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_P = c_void_p
+_PROTOTYPES = {
+    "elementwise": {
+        "mf_embed": [_P, c_int, _P, _P, c_int, c_int, c_int, _P],
+        "mf_rmsnorm": [_P, _P, _P, _P, c_int, c_int, c_int, c_float, _P],
+        "mf_gather_rows": [_P, _P, _P, c_int, c_int, _P],
+        "mf_swiglu": [_P, c_int, _P, c_int, c_int, c_int, _P],
+        "mf_convert": [_P, c_int, _P, c_int, c_size_t, _P],
+        "mf_rope_table": [_P, _P, c_int, c_int, c_double, c_double, _P],
+        "mf_rope_kvwrite": [_P, _P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int,
+                            c_int, c_int, _P],
+        "mf_fill_normal": [_P, c_int, c_size_t, c_uint64, c_float, _P],
+    },
+    "gemm_f32": {
+        "mf_gemm_f32": [_P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+    },
+    "gemm_bf16": {
+        "mf_gemm_bf16": [_P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_gemm_bf16_skinny": [_P, c_int, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int,
+                                c_int, c_int, _P],
+    },
+    "attn_tokens_f32": {
+        "mf_attn_tokens_f32": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
+                               c_float, c_int, c_int, c_int, _P],
+    },
+    "attn_tokens_bf16": {
+        "mf_attn_tokens_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
+                                c_float, c_int, c_int, c_int, _P],
+    },
+    "attn_prefill_bf16": {
+        "mf_attn_prefill_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int,
+                                 c_int, c_float, c_int, _P],
+    },
+    "sampling": {
+        "mf_argmax": [_P, c_int, c_int, c_int, _P, _P],
+        "mf_sample": [_P, c_int, c_int, c_int, c_float, c_uint64, _P, _P, _P, _P, _P],
+        "mf_penalties": [_P, c_int, c_int, c_int, _P, c_int, _P, c_float, c_float, c_float, _P],
+        "mf_top_k": [_P, c_int, c_int, c_int, c_int, _P],
+        "mf_top_p": [_P, c_int, c_int, c_int, c_float, _P, _P],
+        "mf_advance": [_P, _P, _P, _P, c_int, _P],
+    },
+}
+_functions: Dict[str, object] = {}
+
+
+def _fn(lib: str, name: str):
+    f = _functions.get(name)
+    if f is None:
+        f = getattr(build.load(lib), name)
+        f.argtypes = _PROTOTYPES[lib][name]
+        f.restype = c_int
+        _functions[name] = f
+    return f
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise KernelError(f"{what}: HIP error {rc}"
+                          + (" (invalid argument: a size the kernel does not take)" if rc == 1 else ""))
+
+
+def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name}: must be a tensor on the GPU (there is no CPU path)")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: must be contiguous, got strides {t.stride()} for shape {tuple(t.shape)}")
+    if dtype is not None:
+        ok = t.dtype in dtype if isinstance(dtype, (tuple, list)) else t.dtype == dtype
+        if not ok:
+            raise KernelError(f"{name}: dtype {t.dtype}, expected {dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+
+
+def _is_bf16(t: torch.Tensor) -> int:
+    return 1 if t.dtype == torch.bfloat16 else 0
+
+
+_FLOATS = (torch.float32, torch.bfloat16)
+
+# ------------------------------------------------------------------ workspaces
+_workspaces: Dict[Tuple[str, int], torch.Tensor] = {}
+
+
+def workspace(tag: str, n_floats: int, device) -> torch.Tensor:
+    """A float32 scratch tensor of at least n_floats, kept per (tag, device) and grown when
+    needed.  Kernels that use one run in stream order, so sharing it is safe."""
+    key = (tag, torch.device(device).index or 0)
+    w = _workspaces.get(key)
+    if w is None or w.numel() < n_floats:
+        w = torch.empty(max(n_floats, 1 << 16), dtype=torch.float32, device=device)
+        _workspaces[key] = w
+    return w
+
+
+# ------------------------------------------------------------------ element-wise
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+    _need(table, "embed.table", _FLOATS)
+    _need(ids, "embed.ids", torch.int32)
+    n, d = ids.numel(), table.shape[1]
+    _need(out, "embed.out", torch.float32, (n, d))
+    _check(_fn("elementwise", "mf_embed")(_ptr(table), _is_bf16(table), _ptr(ids), _ptr(out), n, d,
+                                           table.shape[0], _stream()), "embed")
+
+
+def rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out: torch.Tensor,
+            row_idx: Optional[torch.Tensor] = None) -> None:
+    _need(x, "rmsnorm.x", torch.float32)
+    d = x.shape[-1]
+    rows = out.shape[0]
+    _need(out, "rmsnorm.out", _FLOATS, (rows, d))
+    if weight is not None:
+        _need(weight, "rmsnorm.weight", torch.float32, (d,))
+    if row_idx is not None:
+        _need(row_idx, "rmsnorm.row_idx", torch.int32, (rows,))
+    elif x.shape[0] != rows:
+        raise KernelError(f"rmsnorm: x has {x.shape[0]} rows, out has {rows}")
+    _check(_fn("elementwise", "mf_rmsnorm")(_ptr(x), _ptr(row_idx), _ptr(weight), _ptr(out),
+                                             _is_bf16(out), rows, d, float(eps), _stream()), "rmsnorm")
+
+
+def gather_rows(x: torch.Tensor, idx: torch.Tensor, out: torch.Tensor) -> None:
+    _need(x, "gather_rows.x", torch.float32)
+    _need(idx, "gather_rows.idx", torch.int32)
+    _need(out, "gather_rows.out", torch.float32, (idx.numel(), x.shape[1]))
+    _check(_fn("elementwise", "mf_gather_rows")(_ptr(x), _ptr(idx), _ptr(out), idx.numel(),
+                                                 x.shape[1], _stream()), "gather_rows")
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    _need(gate_up, "swiglu.gate_up", _FLOATS)
+    rows, two_nf = gate_up.shape
+    if two_nf % 2:
+        raise KernelError(f"swiglu: gate_up has an odd width {two_nf}")
+    _need(out, "swiglu.out", _FLOATS, (rows, two_nf // 2))
+    if _is_bf16(gate_up) and not _is_bf16(out):
+        raise KernelError("swiglu: bfloat16 input with float32 output is not provided")
+    _check(_fn("elementwise", "mf_swiglu")(_ptr(gate_up), _is_bf16(gate_up), _ptr(out), _is_bf16(out),
+                                            rows, two_nf // 2, _stream()), "swiglu")
+
+
+def convert(src: torch.Tensor, dst: torch.Tensor) -> None:
+    _need(src, "convert.src", _FLOATS)
+    _need(dst, "convert.dst", _FLOATS)
+    if src.numel() != dst.numel() or src.dtype == dst.dtype:
+        raise KernelError("convert: needs equal sizes and different types")
+    _check(_fn("elementwise", "mf_convert")(_ptr(src), _is_bf16(src), _ptr(dst), _is_bf16(dst),
+                                             src.numel(), _stream()), "convert")
+
+
+def fill_normal(out: torch.Tensor, seed: int, std: float) -> None:
+    _need(out, "fill_normal.out", _FLOATS)
+    _check(_fn("elementwise", "mf_fill_normal")(_ptr(out), _is_bf16(out), out.numel(),
+                                                 seed & 0xFFFFFFFFFFFFFFFF, float(std), _stream()),
+           "fill_normal")
+
+
+def rope_table(n_pos: int, half: int, theta: float, freq_scale: float, device):
+    cs = torch.empty((n_pos, half), dtype=torch.float32, device=device)
+    sn = torch.empty((n_pos, half), dtype=torch.float32, device=device)
+    _need(cs, "rope_table.out")
+    _check(_fn("elementwise", "mf_rope_table")(_ptr(cs), _ptr(sn), n_pos, half, float(theta),
+                                                float(freq_scale), _stream()), "rope_table")
+    return cs, sn
+
+
+def rope_kvwrite(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
+                 seq_of_tok: torch.Tensor, page_table: torch.Tensor, q_out: torch.Tensor,
+                 kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor], n_heads: int,
+                 n_kv_heads: int, head_dim: int, write_kv: bool = True) -> None:
+    n_tok = positions.numel()
+    _need(qkv, "rope.qkv", torch.float32, (n_tok, (n_heads + 2 * n_kv_heads) * head_dim))
+    _need(cos, "rope.cos", torch.float32)
+    _need(sin, "rope.sin", torch.float32, tuple(cos.shape))
+    if cos.shape[1] != head_dim // 2:
+        raise KernelError(f"rope: table has {cos.shape[1]} frequencies, head_dim {head_dim} needs {head_dim // 2}")
+    _need(positions, "rope.positions", torch.int32, (n_tok,))
+    _need(seq_of_tok, "rope.seq_of_tok", torch.int32, (n_tok,))
+    _need(page_table, "rope.page_table", torch.int32)
+    _need(q_out, "rope.q_out", _FLOATS, (n_tok, n_heads * head_dim))
+    if write_kv:
+        for name, c in (("rope.kcache", kcache), ("rope.vcache", vcache)):
+            _need(c, name, q_out.dtype)
+            if tuple(c.shape[1:]) != (n_kv_heads, PAGE, head_dim):
+                raise KernelError(f"{name}: shape {tuple(c.shape)}, expected [pages, {n_kv_heads}, {PAGE}, {head_dim}]")
+    _check(_fn("elementwise", "mf_rope_kvwrite")(
+        _ptr(qkv), _ptr(cos), _ptr(sin), _ptr(positions), _ptr(seq_of_tok), _ptr(page_table),
+        page_table.shape[1], _ptr(q_out), _ptr(kcache if write_kv else None),
+        _ptr(vcache if write_kv else None), _is_bf16(q_out), n_tok, n_heads, n_kv_heads, head_dim,
+        1 if write_kv else 0, _stream()), "rope_kvwrite")
+
+
+# ------------------------------------------------------------------ matrix products
+def skinny_plan(m: int, n: int, k: int, target_blocks: int = 1024) -> Tuple[int, int]:
+    """(splits, k_per_split) of the decode product: enough blocks to fill the chip."""
+    n_blocks = (n + 63) // 64
+    chunks = (k + 255) // 256
+    splits = max(1, min(chunks, target_blocks // max(1, n_blocks)))
+    per = (chunks + splits - 1) // splits
+    return (chunks + per - 1) // per, per * 256
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+           accumulate: bool = False, variant: int = 0) -> None:
+    """out (+)= x @ weight^T (+ bias).  weight is [out][in].  float32 weights take the true
+    32-bit kernel; bfloat16 weights take the matrix-core kernels (a few rows: the streaming
+    kernel).  `out` is float32, or bfloat16 for a bfloat16 product that is stored."""
+    _need(x, "linear.x", _FLOATS)
+    _need(weight, "linear.weight", x.dtype)
+    m, k = x.shape
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"linear: x is [{m},{k}], weight is {tuple(weight.shape)}")
+    _need(out, "linear.out", _FLOATS, (m, n))
+    if bias is not None:
+        _need(bias, "linear.bias", torch.float32, (n,))
+    if m == 0:
+        return
+    if x.dtype == torch.float32:
+        _need(out, "linear.out", torch.float32)
+        _check(_fn("gemm_f32", "mf_gemm_f32")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n, m,
+                                               n, k, 1 if accumulate else 0, _stream()), "gemm_f32")
+        return
+    if accumulate and out.dtype != torch.float32:
+        raise KernelError("linear: accumulation needs a float32 output")
+    epi = EPI_BF16 if out.dtype == torch.bfloat16 else (EPI_ACC_F32 if accumulate else EPI_F32)
+    if m <= 64 and variant == 0:
+        splits, per = skinny_plan(m, n, k)
+        part = workspace("skinny", splits * m * n, x.device) if splits > 1 else None
+        _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(bias),
+                                                        _ptr(out), n, _ptr(part), m, n, k, splits, per,
+                                                        epi, _stream()), "gemm_bf16_skinny")
+        return
+    _check(_fn("gemm_bf16", "mf_gemm_bf16")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n, m,
+                                             n, k, epi, variant, _stream()), "gemm_bf16")
+
+
+# ------------------------------------------------------------------ attention
+def split_plan(n_tok: int, n_kv_heads: int, group: int, head_dim: int, max_len: int,
+               target_blocks: int = 768) -> Tuple[int, int]:
+    """(n_splits, split_len) for the per-token attention: split the keys when tokens x kv
+    heads alone do not fill the chip.  Depends on the capacity, not on current lengths."""
+    gc = 8 if head_dim <= 128 else 4
+    blocks = n_tok * n_kv_heads * ((group + gc - 1) // gc)
+    n_splits = max(1, min(target_blocks // max(1, blocks), (max_len + 255) // 256))
+    split_len = ((max_len + n_splits - 1) // n_splits + 15) // 16 * 16
+    split_len = max(split_len, 16)
+    return (max_len + split_len - 1) // split_len, split_len
+
+
+def attn_tokens(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
+                positions: torch.Tensor, seq_of_tok: torch.Tensor, out: torch.Tensor, n_heads: int,
+                n_kv_heads: int, head_dim: int, scale: float, window: int, max_len: int) -> None:
+    """Each query token attends to its sequence's cache rows lo..position.  `max_len` bounds
+    position + 1 for every token (it only shapes the launch)."""
+    n_tok = positions.numel()
+    _need(q, "attn.q", _FLOATS, (n_tok, n_heads * head_dim))
+    _need(out, "attn.out", q.dtype, (n_tok, n_heads * head_dim))
+    for name, c in (("attn.kcache", kcache), ("attn.vcache", vcache)):
+        _need(c, name, q.dtype)
+        if tuple(c.shape[1:]) != (n_kv_heads, PAGE, head_dim):
+            raise KernelError(f"{name}: shape {tuple(c.shape)}, expected [pages, {n_kv_heads}, {PAGE}, {head_dim}]")
+    _need(page_table, "attn.page_table", torch.int32)
+    _need(positions, "attn.positions", torch.int32, (n_tok,))
+    _need(seq_of_tok, "attn.seq_of_tok", torch.int32, (n_tok,))
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise KernelError(f"attention: head_dim {head_dim} is not a multiple of 16 in [16, 256]")
+    if n_heads % n_kv_heads:
+        raise KernelError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
+    if max_len > page_table.shape[1] * PAGE:
+        raise KernelError(f"attention: max_len {max_len} exceeds the page table ({page_table.shape[1]} pages)")
+    n_splits, split_len = split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, head_dim, max_len)
+    part = workspace("attn", n_tok * n_heads * n_splits * (head_dim + 2), q.device) if n_splits > 1 else None
+    name = "attn_tokens_bf16" if q.dtype == torch.bfloat16 else "attn_tokens_f32"
+    _check(_fn(name, "mf_" + name)(
+        _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions),
+        _ptr(seq_of_tok), _ptr(out), _ptr(part), n_tok, n_heads, n_kv_heads, head_dim, float(scale),
+        int(window or 0), n_splits, split_len, _stream()), name)

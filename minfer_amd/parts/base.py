@@ -1,0 +1,128 @@
+"""Interfaces of the parts a block is put together from, and the registries that map a
+`PartSpec.kind` to a class.
+
+A part is built from its constants alone (`PartSpec.params`), says which tensors it wants
+(`tensor_specs`, names relative to the block's prefix), receives them (`load`), and runs.
+It never sees the configuration, the model, or which layer it is.  The step's ragged batch
+arrives as a `StepContext` (see `minfer_amd.engine.batch`).
+
+Numeric contract between parts: the residual stream `h` is float32 `[tokens][hidden]`;
+norms read it and write the run type (bfloat16 or float32); mixers and feed-forwards read
+the run type and *add* their result into `h` in 32-bit.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable, Dict, Optional
+
+import torch
+
+from ..weights.loader import TensorSpec
+from .spec import PartSpec
+
+
+@dataclass
+class Runtime:
+    """Where and in which precision a model runs."""
+    dtype: torch.dtype          # run type of activations, matrices and cache
+    device: torch.device
+
+    @property
+    def is_bf16(self) -> bool:
+        return self.dtype == torch.bfloat16
+
+
+class Part:
+    """Base of every part."""
+
+    def __init__(self, spec: PartSpec, rt: Runtime):
+        self.spec, self.rt = spec, rt
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {}
+
+    def load(self, get: Callable[[str], torch.Tensor]) -> None:
+        """`get(name)` returns the tensor on the device in its storage type."""
+
+    def prepare(self, max_len: int) -> None:
+        """Called before steps that may reach `max_len` positions (tables, workspaces), so
+        that a captured step allocates nothing of its own."""
+
+
+class Norm(Part):
+    def forward(self, h: torch.Tensor, out: Optional[torch.Tensor] = None,
+                row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """float32 rows in, run-type rows out; row r reads h[row_idx[r]] when given."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotate_and_store(self, qkv: torch.Tensor, ctx, q_out: torch.Tensor, kcache, vcache,
+                         page_table, n_heads: int, n_kv_heads: int, write_kv: bool) -> None:
+        """Encodes positions into q (written to q_out) and k, and stores k and v of the
+        step's tokens into the cache pages."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_request(self):
+        """A `KVRequest`, a `StateRequest` or None."""
+        return None
+
+    def forward(self, x: torch.Tensor, h: torch.Tensor, ctx, entry: int, writes_cache: bool) -> None:
+        """Adds the mixer's output for the step's tokens into h.  `entry` is the cache entry
+        (`ctx.cache.kv(entry)` / `ctx.cache.state(entry)`)."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, h: torch.Tensor, ctx) -> None:
+        """Adds the feed-forward's output into h (h may hold fewer rows than the step)."""
+        raise NotImplementedError
+
+
+class Block:
+    """An arrangement of parts.  `forward` returns the residual stream, reduced to the rows
+    `keep_rows` (int32 indices on the device) when given."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
+                 feed_forward_norm: Norm, rt: Runtime):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+        self.rt = rt
+
+    def parts(self):
+        return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
+
+    def forward(self, h, ctx, entry: int, writes_cache: bool, keep_rows=None):
+        raise NotImplementedError
+
+
+MIXERS: Dict[str, type] = {}
+FEED_FORWARDS: Dict[str, type] = {}
+NORMS: Dict[str, type] = {}
+POSITIONS: Dict[str, type] = {}
+BLOCKS: Dict[str, type] = {}
+
+
+def _registrar(table: Dict[str, type], what: str):
+    def register(kind: str):
+        def deco(cls):
+            table[kind] = cls
+            return cls
+        return deco
+    register.__doc__ = f"Class decorator: registers a {what} under a PartSpec.kind."
+    return register
+
+
+register_mixer = _registrar(MIXERS, "mixer")
+register_feed_forward = _registrar(FEED_FORWARDS, "feed-forward")
+register_norm = _registrar(NORMS, "norm")
+register_position = _registrar(POSITIONS, "position encoding")
+register_block = _registrar(BLOCKS, "block arrangement")
+
+
+def make_part(table: Dict[str, type], spec: PartSpec, rt: Runtime, what: str):
+    if spec.kind not in table:
+        raise KeyError(f"unknown {what} {spec.kind!r}; registered: {', '.join(sorted(table)) or '(none)'}")
+    return table[spec.kind](spec, rt)

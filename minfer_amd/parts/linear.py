@@ -1,0 +1,57 @@
+"""A weight matrix `[out][in]` with an optional bias, applied through the HIP products.
+
+out[t][o] = dot(W[o][:], x[t][:]) + b[o] (src/graph/cpu_backend.rs:214-248 of
+yusiwen/minfer).  A matrix stored in 32 bits stays in 32 bits and takes the 32-bit kernel
+even when activations are bfloat16 (they are widened, which is exact).  Biases are kept in
+float32 and added in the product's epilogue.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from ..kernels import ops
+
+
+def common_matrix_dtype(tensors: List[torch.Tensor]) -> torch.dtype:
+    return torch.bfloat16 if all(t.dtype == torch.bfloat16 for t in tensors) else torch.float32
+
+
+class Linear:
+    def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor] = None):
+        if weight.dim() != 2:
+            raise ValueError(f"Linear: weight must be a matrix, got {tuple(weight.shape)}")
+        self.weight = weight.contiguous()
+        self.bias = None if bias is None else bias.to(torch.float32).contiguous()
+        self.out_features, self.in_features = weight.shape
+
+    @classmethod
+    def stacked(cls, weights: List[torch.Tensor], biases: Optional[List[Optional[torch.Tensor]]] = None):
+        """Rows of several matrices over the same input in one matrix, so a step reads one
+        (the reference concatenates q|k|v and gate|up the same way for its GPU path,
+        src/models/qwen2/loader.rs:290-331)."""
+        dt = common_matrix_dtype(weights)
+        w = torch.cat([t.to(dt) for t in weights], dim=0)
+        b = None
+        if biases is not None and any(x is not None for x in biases):
+            b = torch.cat([torch.zeros(t.shape[0], dtype=torch.float32, device=t.device) if x is None
+                           else x.to(torch.float32) for t, x in zip(weights, biases)])
+        return cls(w, b)
+
+    def __call__(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
+                 out_dtype: torch.dtype = torch.float32, accumulate: bool = False) -> torch.Tensor:
+        rows = x.shape[0]
+        if out is None:
+            out = torch.empty((rows, self.out_features), dtype=out_dtype, device=x.device)
+        if self.weight.dtype == torch.float32 and x.dtype != torch.float32:
+            wide = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+            ops.convert(x, wide)
+            x = wide
+        if x.dtype == torch.float32 and out.dtype != torch.float32:
+            tmp = torch.empty(out.shape, dtype=torch.float32, device=x.device)
+            ops.linear(x, self.weight, self.bias, tmp)
+            ops.convert(tmp, out)
+            return out
+        ops.linear(x, self.weight, self.bias, out, accumulate=accumulate)
+        return out

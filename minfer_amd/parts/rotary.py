@@ -1,0 +1,42 @@
+"""Half-split ("NeoX") rotary position encoding over the whole head: element i pairs with
+i + head_dim/2, angle = position * freq_scale / theta^(2i/head_dim)
+(src/graph/cpu_backend.rs:403-434 of yusiwen/minfer; q and k are rotated after their bias
+and before the cache write, v is not, src/models/qwen2/graph.rs:100-113).  cos and sin come
+from a table built once on the device in double precision; the kernel that rotates also
+stores k and v into the cache pages."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import PositionEncoding, register_position
+
+
+@register_position("rope_neox")
+class RotaryNeoX(PositionEncoding):
+    """params: head_dim, theta, max_positions, freq_scale (default 1)."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        p = spec.params
+        self.head_dim, self.theta = int(p["head_dim"]), float(p["theta"])
+        self.freq_scale = float(p.get("freq_scale", 1.0))
+        self.max_positions = int(p["max_positions"])
+        if self.head_dim % 2:
+            raise ValueError(f"rope_neox: head_dim {self.head_dim} is odd")
+        self.cos = self.sin = None
+
+    def prepare(self, max_len: int) -> None:
+        if max_len > self.max_positions:
+            raise ValueError(f"position {max_len - 1} is beyond the model's {self.max_positions} positions")
+        have = 0 if self.cos is None else self.cos.shape[0]
+        if max_len > have:
+            n = min(self.max_positions, max(256, 1 << (max_len - 1).bit_length()))
+            self.cos, self.sin = ops.rope_table(n, self.head_dim // 2, self.theta, self.freq_scale,
+                                                self.rt.device)
+
+    def rotate_and_store(self, qkv, ctx, q_out, kcache, vcache, page_table, n_heads, n_kv_heads,
+                         write_kv: bool) -> None:
+        self.prepare(ctx.max_len)
+        ops.rope_kvwrite(qkv, self.cos, self.sin, ctx.positions, ctx.seq_of_tok, page_table, q_out,
+                         kcache, vcache, n_heads, n_kv_heads, self.head_dim, write_kv)

@@ -1,0 +1,83 @@
+"""Descriptions of a model as data: which parts make up each block, with which constants,
+and in which order blocks run.
+
+A configuration class turns its config.json keys into a `ModelSpec`; the builder in
+`minfer_amd.engine.model` turns a `ModelSpec` into parts by looking each `PartSpec.kind`
+up in the part registries.  No part ever sees the configuration or the model it is in.
+
+The reference builds its per-step graph from part constructors that take their constants
+as parameters (`rms_norm(x,w,eps)`, `rope(x,pos,style,meta)`, `attn(q,kv,pos,mode,meta)`,
+src/graph/builder.rs:79-286 of yusiwen/minfer) inside one loop over layers
+(src/models/qwen2/graph.rs:59-177).  Here that loop is the `schedule` list.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional, Tuple
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """One part: its registry name and its constants (sizes, eps, theta, tensor names...)."""
+    kind: str
+    params: Dict[str, Any] = field(default_factory=dict)
+
+    def get(self, key: str, default: Any = None) -> Any:
+        return self.params.get(key, default)
+
+
+@dataclass(frozen=True)
+class BlockSpec:
+    """One block: the arrangement (`kind`, e.g. pre-norm residual) and its four parts.
+    `prefix` is put before every tensor name of the block's parts."""
+    kind: str
+    prefix: str
+    mixer: PartSpec
+    feed_forward: PartSpec
+    mixer_norm: PartSpec
+    feed_forward_norm: PartSpec
+
+
+@dataclass(frozen=True)
+class RunEntry:
+    """One position of the run order.  `block` indexes `ModelSpec.blocks` and may appear
+    in several entries.  `cache` is the cache entry the mixer uses; entries that name the
+    same `cache` share keys and values, and only the entry with `writes_cache` stores
+    into it (the other reads what the first one wrote in the same step)."""
+    block: int
+    cache: int
+    writes_cache: bool = True
+
+
+@dataclass(frozen=True)
+class ModelSpec:
+    hidden_size: int
+    vocab_size: int
+    embedding_name: str
+    head_name: Optional[str]          # None: the head is the embedding table (tied)
+    final_norm: PartSpec
+    blocks: Tuple[BlockSpec, ...]
+    schedule: Tuple[RunEntry, ...]
+    max_positions: int
+    stop_tokens: Tuple[int, ...] = ()
+
+    def __post_init__(self):
+        for e in self.schedule:
+            if not 0 <= e.block < len(self.blocks):
+                raise ValueError(f"schedule names block {e.block}, model has {len(self.blocks)}")
+        writers = {}
+        for n, e in enumerate(self.schedule):
+            if e.writes_cache:
+                if e.cache in writers:
+                    raise ValueError(f"cache entry {e.cache} is written by schedule positions "
+                                     f"{writers[e.cache]} and {n}")
+                writers[e.cache] = n
+        for n, e in enumerate(self.schedule):
+            if not e.writes_cache and (e.cache not in writers or writers[e.cache] > n):
+                raise ValueError(f"schedule position {n} reads cache entry {e.cache} "
+                                 "before any position writes it")
+
+
+def straight_schedule(n_blocks: int) -> Tuple[RunEntry, ...]:
+    """Block i runs i-th and owns cache entry i."""
+    return tuple(RunEntry(block=i, cache=i) for i in range(n_blocks))

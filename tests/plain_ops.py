@@ -1,0 +1,136 @@
+"""Plain torch versions of every HIP kernel, with the kernels' own signatures.
+
+Two uses, both in tests only: (1) the reference each kernel is compared with on the GPU;
+(2) patched over `minfer_amd.kernels.ops` (`install`), they let the CPU-only tests drive
+the real engine, cache and generation loop where no GPU exists.  The product never imports
+this file.  Arithmetic is float64 inside, rounded once to the output type.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+PAGE = 64
+
+
+def embed(table, ids, out):
+    out.copy_(table[ids.long()].to(torch.float32))
+
+
+def rmsnorm(x, weight, eps, out, row_idx=None):
+    src = x if row_idx is None else x[row_idx.long()]
+    s = src.double()
+    y = s * (1.0 / torch.sqrt((s * s).mean(dim=-1, keepdim=True) + eps))
+    if weight is not None:
+        y = y * weight.double()
+    out.copy_(y.to(out.dtype))
+
+
+def gather_rows(x, idx, out):
+    out.copy_(x[idx.long()])
+
+
+def swiglu(gate_up, out):
+    nf = gate_up.shape[1] // 2
+    g, u = gate_up[:, :nf].double(), gate_up[:, nf:].double()
+    out.copy_((g / (1.0 + torch.exp(-g)) * u).to(out.dtype))
+
+
+def convert(src, dst):
+    dst.copy_(src.to(dst.dtype))
+
+
+def fill_normal(out, seed, std):
+    g = torch.Generator(device="cpu").manual_seed(seed & 0x7FFFFFFFFFFFFFFF)
+    out.copy_((torch.randn(out.shape, generator=g, dtype=torch.float32) * std).to(out.dtype))
+
+
+def rope_table(n_pos, half, theta, freq_scale, device):
+    i = torch.arange(half, dtype=torch.float64)
+    freq = freq_scale / torch.pow(torch.tensor(float(theta), dtype=torch.float64), 2.0 * i / (2 * half))
+    ang = torch.arange(n_pos, dtype=torch.float64)[:, None] * freq[None, :]
+    return torch.cos(ang).float().to(device), torch.sin(ang).float().to(device)
+
+
+def rope_kvwrite(qkv, cos, sin, positions, seq_of_tok, page_table, q_out, kcache, vcache,
+                 n_heads, n_kv_heads, head_dim, write_kv=True):
+    t = positions.numel()
+    half = head_dim // 2
+    x = qkv.double().view(t, n_heads + 2 * n_kv_heads, head_dim)
+    c = cos[positions.long()].double()[:, None, :]
+    s = sin[positions.long()].double()[:, None, :]
+
+    def rot(v):
+        v0, v1 = v[..., :half], v[..., half:]
+        return torch.cat([v0 * c - v1 * s, v0 * s + v1 * c], dim=-1)
+    q_out.copy_(rot(x[:, :n_heads]).reshape(t, n_heads * head_dim).to(q_out.dtype))
+    if not write_kv:
+        return
+    k = rot(x[:, n_heads:n_heads + n_kv_heads]).to(kcache.dtype)
+    v = x[:, n_heads + n_kv_heads:].to(vcache.dtype)
+    pos = positions.long()
+    page = page_table.long()[seq_of_tok.long(), pos // PAGE]
+    assert (page >= 0).all(), "token written to a page that was not reserved"
+    kcache[page, :, pos % PAGE, :] = k
+    vcache[page, :, pos % PAGE, :] = v
+
+
+def linear(x, weight, bias, out, accumulate=False, variant=0):
+    y = x.double() @ weight.double().t()
+    if bias is not None:
+        y = y + bias.double()
+    if accumulate:
+        y = y + out.double()
+    out.copy_(y.to(out.dtype))
+
+
+def gather_cache_rows(cache, page_table_row, length):
+    """[length][kv_heads][head_dim] rows 0..length-1 of one sequence."""
+    pos = torch.arange(length)
+    page = page_table_row.long()[pos // PAGE]
+    return cache[page, :, pos % PAGE, :]
+
+
+def attn_tokens(q, kcache, vcache, page_table, positions, seq_of_tok, out, n_heads, n_kv_heads,
+                head_dim, scale, window, max_len):
+    t = positions.numel()
+    g = n_heads // n_kv_heads
+    qh = q.double().view(t, n_heads, head_dim)
+    res = torch.zeros(t, n_heads, head_dim, dtype=torch.float64)
+    for i in range(t):
+        p = int(positions[i])
+        lo = max(0, p - window + 1) if window else 0
+        row = page_table[int(seq_of_tok[i])]
+        pos = torch.arange(lo, p + 1)
+        page = row.long()[pos // PAGE]
+        assert (page >= 0).all(), "attention reads a page that was given back"
+        k = kcache[page, :, pos % PAGE, :].double()      # [n][nk][hd]
+        v = vcache[page, :, pos % PAGE, :].double()
+        for h in range(n_heads):
+            s = (k[:, h // g, :] @ qh[i, h]) * scale
+            res[i, h] = torch.softmax(s, dim=0) @ v[:, h // g, :]
+    out.copy_(res.view(t, n_heads * head_dim).to(out.dtype))
+
+
+def attn_prefill(q, kcache, vcache, page_table, ctx, out, n_heads, n_kv_heads, head_dim, scale, window):
+    attn_tokens(q, kcache, vcache, page_table, ctx.positions, ctx.seq_of_tok, out, n_heads, n_kv_heads,
+                head_dim, scale, window, ctx.max_len)
+
+
+# ------------------------------------------------------------------ sampling
+def argmax(logits, out):
+    out.copy_(torch.argmax(logits, dim=-1).to(out.dtype))   # first maximum
+
+
+NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", "rope_table",
+         "rope_kvwrite", "linear", "attn_tokens", "attn_prefill"]
+
+
+def install(monkeypatch):
+    """Replaces the HIP launchers by the plain versions and lets models live on the CPU."""
+    from minfer_amd.engine import loading
+    from minfer_amd.kernels import ops
+    for name in NAMES:
+        monkeypatch.setattr(ops, name, globals()[name])
+    monkeypatch.setattr(loading, "require_gpu", lambda device: torch.device("cpu"))
