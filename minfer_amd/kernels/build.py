@@ -27,7 +27,6 @@ LIBRARIES: Dict[str, str] = {
     "gemm_bf16": "gemm_bf16.hip",
     "attn_tokens_f32": "attn_tokens_f32.hip",
     "attn_tokens_bf16": "attn_tokens_bf16.hip",
-    "attn_prefill_bf16": "attn_prefill_bf16.hip",
     "sampling": "sampling.hip",
 }
 HEADERS = ["common.h", "attn_tokens_impl.h"]

@@ -60,7 +60,7 @@ _PROTOTYPES = {
         "mf_sample": [_P, c_int, c_int, c_int, c_float, c_uint64, _P, _P, _P, _P, _P],
         "mf_penalties": [_P, c_int, c_int, c_int, _P, c_int, _P, c_float, c_float, c_float, _P],
         "mf_top_k": [_P, c_int, c_int, c_int, c_int, _P],
-        "mf_top_p": [_P, c_int, c_int, c_int, c_float, _P, _P],
+        "mf_top_p": [_P, c_int, c_int, c_int, c_float, _P],
         "mf_advance": [_P, _P, _P, _P, c_int, _P],
     },
 }
@@ -308,3 +308,64 @@ def attn_tokens(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions),
         _ptr(seq_of_tok), _ptr(out), _ptr(part), n_tok, n_heads, n_kv_heads, head_dim, float(scale),
         int(window or 0), n_splits, split_len, _stream()), name)
+
+
+# ------------------------------------------------------------------ sampling
+def _logit_rows(logits: torch.Tensor, name: str):
+    _need(logits, name, torch.float32)
+    if logits.dim() != 2:
+        raise KernelError(f"{name}: expected [rows][vocab], got {tuple(logits.shape)}")
+    return logits.shape
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    rows, vocab = _logit_rows(logits, "argmax.logits")
+    _need(out, "argmax.out", torch.int32, (rows,))
+    _check(_fn("sampling", "mf_argmax")(_ptr(logits), vocab, rows, vocab, _ptr(out), _ptr(None), _stream()),
+           "argmax")
+
+
+def sample(logits: torch.Tensor, temp: float, seed: int, keys: torch.Tensor, steps: torch.Tensor,
+           out: torch.Tensor, forced_r: Optional[torch.Tensor] = None) -> None:
+    """Temperature draw per row (greedy when temp < 1e-6).  The uniform of row i is
+    `rng.uniform(seed, keys[i], steps[i])`, or forced_r[i] when given (tests)."""
+    rows, vocab = _logit_rows(logits, "sample.logits")
+    _need(keys, "sample.keys", torch.int64, (rows,))
+    _need(steps, "sample.steps", torch.int32, (rows,))
+    _need(out, "sample.out", torch.int32, (rows,))
+    if forced_r is not None:
+        _need(forced_r, "sample.forced_r", torch.float32, (rows,))
+    _check(_fn("sampling", "mf_sample")(_ptr(logits), vocab, rows, vocab, float(temp),
+                                         seed & 0xFFFFFFFFFFFFFFFF, _ptr(keys), _ptr(steps),
+                                         _ptr(forced_r), _ptr(out), _stream()), "sample")
+
+
+def penalties(logits: torch.Tensor, prev: torch.Tensor, n_prev: torch.Tensor, repeat: float,
+              frequency: float, presence: float) -> None:
+    rows, vocab = _logit_rows(logits, "penalties.logits")
+    _need(prev, "penalties.prev", torch.int32)
+    if prev.dim() != 2 or prev.shape[0] != rows:
+        raise KernelError(f"penalties.prev: expected [{rows}][window], got {tuple(prev.shape)}")
+    _need(n_prev, "penalties.n_prev", torch.int32, (rows,))
+    _check(_fn("sampling", "mf_penalties")(_ptr(logits), vocab, rows, vocab, _ptr(prev), prev.shape[1],
+                                            _ptr(n_prev), float(repeat), float(frequency),
+                                            float(presence), _stream()), "penalties")
+
+
+def top_k(logits: torch.Tensor, k: int) -> None:
+    rows, vocab = _logit_rows(logits, "top_k.logits")
+    _check(_fn("sampling", "mf_top_k")(_ptr(logits), vocab, rows, vocab, int(k), _stream()), "top_k")
+
+
+def top_p(logits: torch.Tensor, p: float) -> None:
+    rows, vocab = _logit_rows(logits, "top_p.logits")
+    _check(_fn("sampling", "mf_top_p")(_ptr(logits), vocab, rows, vocab, float(p), _stream()), "top_p")
+
+
+def advance(next_ids: torch.Tensor, sampled: torch.Tensor, positions: torch.Tensor,
+            steps: torch.Tensor) -> None:
+    n = next_ids.numel()
+    for name, t in (("next_ids", next_ids), ("sampled", sampled), ("positions", positions), ("steps", steps)):
+        _need(t, "advance." + name, torch.int32, (n,))
+    _check(_fn("sampling", "mf_advance")(_ptr(next_ids), _ptr(sampled), _ptr(positions), _ptr(steps), n,
+                                          _stream()), "advance")

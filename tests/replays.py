@@ -1,0 +1,107 @@
+"""Shared helpers of the replay tests: requests, the three ways of cutting them into
+steps, and the comparison with the plain implementation."""
+from __future__ import annotations
+
+import numpy as np
+
+from tiny import random_tokens
+
+# tolerance of bfloat16 logits, as a fraction of the logits' standard deviation: bfloat16
+# keeps 8 bits, the run rounds activations a few times per layer
+BF16_REL = 0.04
+F32_ABS = 1e-4
+
+
+def requests_for(vocab: int, lengths, seed: int = 0):
+    return {f"r{i}": random_tokens(vocab, n, seed * 100 + i) for i, n in enumerate(lengths)}
+
+
+def plain_logits(plain, requests):
+    return {rid: plain.forward(toks) for rid, toks in requests.items()}
+
+
+def whole_steps(requests):
+    """Each request alone and whole: one step with all its tokens, all logits wanted."""
+    steps = []
+    for rid, toks in requests.items():
+        steps.append(dict(step=len(steps), entries=[dict(id=rid, tokens=toks, want=list(range(len(toks))))],
+                          end=[rid]))
+    return steps
+
+
+def tail_steps(requests, tail: int = 32):
+    """First len - tail tokens in one step, then the last `tail` one by one."""
+    steps = []
+    for rid, toks in requests.items():
+        head = max(0, len(toks) - tail)
+        if head:
+            steps.append(dict(step=len(steps), entries=[dict(id=rid, tokens=toks[:head], want=list(range(head)))],
+                              end=[]))
+        for i in range(head, len(toks)):
+            steps.append(dict(step=len(steps), entries=[dict(id=rid, tokens=[toks[i]], want=[0])],
+                              end=[rid] if i == len(toks) - 1 else []))
+    return steps
+
+
+def batch_steps(requests, batches, prompt_frac: float = 0.6):
+    """Batches of unequal lengths that start together: prompts (a fraction of each
+    request) in one step, then one token each per step; a request whose tokens run out ends
+    while the others go on; the next batch starts afterwards, so slots are used again."""
+    steps = []
+    for batch in batches:
+        plen = {rid: max(1, int(len(requests[rid]) * prompt_frac)) for rid in batch}
+        done = {rid: plen[rid] for rid in batch}
+        ends = [rid for rid in batch if done[rid] == len(requests[rid])]
+        steps.append(dict(step=len(steps),
+                          entries=[dict(id=rid, tokens=requests[rid][:plen[rid]], want=list(range(plen[rid])))
+                                   for rid in batch], end=ends))
+        live = [rid for rid in batch if rid not in ends]
+        while live:
+            entries, ends = [], []
+            for rid in live:
+                entries.append(dict(id=rid, tokens=[requests[rid][done[rid]]], want=[0]))
+                done[rid] += 1
+                if done[rid] == len(requests[rid]):
+                    ends.append(rid)
+            steps.append(dict(step=len(steps), entries=entries, end=ends))
+            live = [rid for rid in live if rid not in ends]
+    return steps
+
+
+def run_steps(engine, steps):
+    """Drives Engine.step with trace steps; returns {(request, position): logits row}."""
+    slots, pos, rows = {}, {}, {}
+    for st in steps:
+        ents = st["entries"]
+        for e in ents:
+            if e["id"] not in slots:
+                slots[e["id"]] = engine.new_sequence()
+                pos[e["id"]] = 0
+        logits = engine.step([slots[e["id"]] for e in ents], [e["tokens"] for e in ents],
+                             [e["want"] for e in ents]).cpu().numpy()
+        r = 0
+        for e in ents:
+            for w in e["want"]:
+                rows[(e["id"], pos[e["id"]] + w)] = logits[r]
+                r += 1
+            pos[e["id"]] += len(e["tokens"])
+        assert r == logits.shape[0]
+        for rid in st["end"]:
+            engine.end_sequence(slots.pop(rid))
+        engine.cache.check_invariants()
+    return rows
+
+
+def compare(rows, ref, dtype: str, what: str):
+    """Every produced row against the plain implementation's; names the first bad place."""
+    assert rows, "nothing was produced"
+    worst = 0.0
+    for (rid, p), got in sorted(rows.items()):
+        want = ref[rid][p]
+        err = float(np.abs(got.astype(np.float64) - want).max())
+        tol = F32_ABS if dtype == "float32" else BF16_REL * float(want.std())
+        assert np.isfinite(got).all(), f"{what}: non-finite logits at request {rid} position {p}"
+        assert err <= tol, (f"{what} [{dtype}]: request {rid} position {p} (of {len(ref[rid])}): "
+                            f"max abs err {err:.3e} > {tol:.3e}")
+        worst = max(worst, err)
+    return worst

@@ -1,0 +1,304 @@
+"""Each HIP kernel alone against its plain torch version (tests/plain_ops.py), at sizes
+other than the engine's: widths and vocabularies that are no power of two, partial tiles,
+head sizes in steps of 16, several group sizes."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from minfer_amd.kernels import ops as o
+    return o
+
+
+def rnd(shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def close(a, b, atol, rtol=0.0):
+    a, b = a.detach().cpu().double(), b.detach().cpu().double()
+    err = (a - b).abs()
+    lim = atol + rtol * b.abs()
+    assert bool((err <= lim).all()), f"max err {err.max().item():.3e} (limit {atol}+{rtol}*|ref|)"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,d,vocab", [(1, 64, 50), (7, 200, 777), (33, 3584, 1000)])
+def test_embed(ops, dtype, rows, d, vocab):
+    table = rnd((vocab, d), dtype, 1)
+    ids = torch.randint(0, vocab, (rows,), dtype=torch.int32)
+    out = torch.empty(rows, d, dtype=torch.float32, device=DEV)
+    ops.embed(table.to(DEV), ids.to(DEV), out)
+    ref = torch.empty(rows, d)
+    plain_ops.embed(table, ids, ref)
+    assert torch.equal(out.cpu(), ref)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,d,eps", [(1, 64, 1e-6), (5, 200, 1e-5), (130, 3584, 1e-6), (3, 1000, 0.1)])
+def test_rmsnorm(ops, out_dtype, rows, d, eps):
+    x = rnd((rows, d), seed=2, scale=3.0)
+    w = rnd((d,), seed=3) + 1.0
+    out = torch.empty(rows, d, dtype=out_dtype, device=DEV)
+    ops.rmsnorm(x.to(DEV), w.to(DEV), eps, out)
+    ref = torch.empty(rows, d, dtype=torch.float64)
+    plain_ops.rmsnorm(x, w, eps, ref)
+    tol = 2e-6 if out_dtype == torch.float32 else 1e-2
+    close(out, ref, tol * 3, tol)
+    # with a row gather
+    idx = torch.tensor([rows - 1, 0, rows // 2], dtype=torch.int32)
+    out2 = torch.empty(3, d, dtype=out_dtype, device=DEV)
+    ops.rmsnorm(x.to(DEV), w.to(DEV), eps, out2, idx.to(DEV))
+    close(out2, ref[idx.long()], tol * 3, tol)
+
+
+def test_gather_rows(ops):
+    x = torch.tensor([[1., 2, 3, 4], [10, 20, 30, 40], [100, 200, 300, 400]])
+    idx = torch.tensor([2, 0], dtype=torch.int32)
+    out = torch.empty(2, 4, device=DEV)
+    ops.gather_rows(x.to(DEV), idx.to(DEV), out)
+    assert out.cpu().tolist() == [[100, 200, 300, 400], [1, 2, 3, 4]]
+
+
+@pytest.mark.parametrize("in_dtype,out_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
+                                                (torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("rows,nf", [(1, 176), (9, 344), (64, 18944)])
+def test_swiglu(ops, in_dtype, out_dtype, rows, nf):
+    gu = rnd((rows, 2 * nf), in_dtype, 4, 3.0)
+    gu[0, :4] = torch.tensor([0.0, 88.0, -88.0, 30.0]).to(in_dtype)
+    out = torch.empty(rows, nf, dtype=out_dtype, device=DEV)
+    ops.swiglu(gu.to(DEV), out)
+    ref = torch.empty(rows, nf, dtype=torch.float64)
+    plain_ops.swiglu(gu, ref)
+    assert torch.isfinite(out).all()
+    tol = 1e-6 if out_dtype == torch.float32 else 8e-3
+    close(out, ref, tol, tol)
+
+
+def test_convert(ops):
+    x = rnd((1000, 37), seed=5)
+    b = torch.empty(1000, 37, dtype=torch.bfloat16, device=DEV)
+    ops.convert(x.to(DEV), b)
+    assert torch.equal(b.cpu(), x.to(torch.bfloat16))
+    f = torch.empty(1000, 37, dtype=torch.float32, device=DEV)
+    ops.convert(b, f)
+    assert torch.equal(f.cpu(), x.to(torch.bfloat16).float())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fill_normal(ops, dtype):
+    a = torch.empty(1 << 20, dtype=dtype, device=DEV)
+    b = torch.empty(1 << 20, dtype=dtype, device=DEV)
+    ops.fill_normal(a, 1234, 0.02)
+    ops.fill_normal(b, 1234, 0.02)
+    assert torch.equal(a, b)
+    ops.fill_normal(b, 1235, 0.02)
+    assert not torch.equal(a, b)
+    a = a.float().cpu()
+    assert abs(a.mean().item()) < 2e-4 and abs(a.std().item() - 0.02) < 2e-4
+    assert a.abs().max().item() < 0.02 * 7
+
+
+@pytest.mark.parametrize("theta,half", [(10000.0, 8), (1e6, 64), (50000.0, 24)])
+def test_rope_table(ops, theta, half):
+    cs, sn = ops.rope_table(300, half, theta, 1.0, DEV)
+    rc, rs = plain_ops.rope_table(300, half, theta, 1.0, "cpu")
+    close(cs, rc, 2e-7)
+    close(sn, rs, 2e-7)
+
+
+def make_cache(n_pages, nk, hd, dtype, seed=0):
+    k = rnd((n_pages, nk, 64, hd), dtype, seed)
+    v = rnd((n_pages, nk, 64, hd), dtype, seed + 1)
+    return k, v
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nk,hd", [(4, 2, 16), (9, 3, 48), (28, 4, 128), (2, 2, 256)])
+def test_rope_kvwrite(ops, dtype, nh, nk, hd):
+    # three sequences with scattered pages; tokens at positions straddling a page edge
+    pos = torch.tensor([0, 1, 62, 63, 64, 65, 5, 130], dtype=torch.int32)
+    seq = torch.tensor([0, 0, 1, 1, 1, 1, 2, 2], dtype=torch.int32)
+    table = torch.tensor([[5, -1, -1], [7, 2, -1], [0, 3, 9]], dtype=torch.int32)
+    t = pos.numel()
+    qkv = rnd((t, (nh + 2 * nk) * hd), seed=6)
+    cs, sn = plain_ops.rope_table(256, hd // 2, 1e4, 1.0, "cpu")
+    kc, vc = make_cache(10, nk, hd, dtype, 7)
+    q_ref = torch.empty(t, nh * hd, dtype=dtype)
+    kr, vr = kc.clone(), vc.clone()
+    plain_ops.rope_kvwrite(qkv, cs, sn, pos, seq, table, q_ref, kr, vr, nh, nk, hd)
+    q = torch.empty(t, nh * hd, dtype=dtype, device=DEV)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    ops.rope_kvwrite(qkv.to(DEV), cs.to(DEV), sn.to(DEV), pos.to(DEV), seq.to(DEV), table.to(DEV), q,
+                     kd, vd, nh, nk, hd)
+    tol = 2e-6 if dtype == torch.float32 else 2e-2
+    close(q, q_ref, tol, tol)
+    close(kd, kr, tol, tol)
+    close(vd, vr, tol, tol)
+    # untouched rows stay untouched
+    assert torch.equal(kd.cpu()[1], kc[1]) and torch.equal(vd.cpu()[4], vc[4])
+
+
+def test_rope_position_zero_is_identity_and_pairs_are_half_split(ops):
+    nh, nk, hd = 2, 1, 32
+    qkv = torch.zeros(2, (nh + 2 * nk) * hd)
+    qkv[:, 3] = 1.0                      # element 3 of head 0
+    cs, sn = ops.rope_table(64, hd // 2, 100.0, 1.0, DEV)
+    pos = torch.tensor([0, 9], dtype=torch.int32, device=DEV)
+    seq = torch.zeros(2, dtype=torch.int32, device=DEV)
+    table = torch.zeros(1, 1, dtype=torch.int32, device=DEV)
+    kc = torch.zeros(1, nk, 64, hd, device=DEV)
+    vc = torch.zeros(1, nk, 64, hd, device=DEV)
+    q = torch.empty(2, nh * hd, device=DEV)
+    ops.rope_kvwrite(qkv.to(DEV), cs, sn, pos, seq, table, q, kc, vc, nh, nk, hd)
+    q = q.cpu()
+    assert torch.equal(q[0], qkv[0, :nh * hd])
+    nz = torch.nonzero(q[1]).flatten().tolist()
+    assert nz == [3, 3 + hd // 2]        # energy moves to i + hd/2, not to i + 1
+    ang = 9.0 / 100.0 ** (2 * 3 / hd)
+    assert abs(q[1, 3].item() - math.cos(ang)) < 1e-6 and abs(q[1, 3 + hd // 2].item() - math.sin(ang)) < 1e-6
+
+
+GEMM_SHAPES = [(1, 64, 64), (3, 176, 64), (17, 1000, 344), (64, 512, 128), (65, 200, 232), (130, 777, 200),
+               (300, 4608, 3584), (33, 96, 18944)]
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+def test_gemm_f32(ops, m, n, k):
+    x, w, b = rnd((m, k), seed=8), rnd((n, k), seed=9, scale=0.05), rnd((n,), seed=10)
+    ref = x.double() @ w.double().t() + b.double()
+    out = torch.empty(m, n, device=DEV)
+    ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), out)
+    close(out, ref, 1e-5 * math.sqrt(k) / 8, 1e-5)
+    base = rnd((m, n), seed=11)
+    acc = base.to(DEV).clone()
+    ops.linear(x.to(DEV), w.to(DEV), None, acc, accumulate=True)
+    close(acc, ref - b.double() + base.double(), 1e-5 * math.sqrt(k) / 8, 1e-5)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(2048, 512, 256), (1, 152064, 64), (64, 3584, 3584)])
+def test_gemm_bf16(ops, variant, m, n, k):
+    if variant and (m * n * k > 3e9):
+        pytest.skip("large shape is covered by the default variant")
+    x, w, b = rnd((m, k), torch.bfloat16, 8), rnd((n, k), torch.bfloat16, 9, 0.05), rnd((n,), seed=10)
+    ref = x.double() @ w.double().t() + b.double()
+    xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+    tol = 2e-5 * math.sqrt(k)
+    out = torch.empty(m, n, device=DEV)
+    ops.linear(xd, wd, bd, out, variant=variant)
+    close(out, ref, tol, 1e-5)
+    out2 = torch.empty(m, n, device=DEV)
+    ops.linear(xd, wd, bd, out2, variant=variant)
+    assert torch.equal(out, out2), "two runs differ"
+    base = rnd((m, n), seed=11)
+    acc = base.to(DEV).clone()
+    ops.linear(xd, wd, None, acc, accumulate=True, variant=variant)
+    close(acc, ref - b.double() + base.double(), tol, 1e-5)
+    ob = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    ops.linear(xd, wd, bd, ob, variant=variant)
+    close(ob, ref, tol, 8e-3)
+
+
+def test_gemm_reference_vector(ops):
+    # src/graph/cpu_backend.rs:540-566: W diag-like, b, x -> then silu and *2
+    w = torch.tensor([[1., 0, 0, 0], [0, 2, 0, 0], [0, 0, 3, 0]])
+    b = torch.tensor([0.5, -1.0, 0.25])
+    x = torch.tensor([[1., 2, 3, 4]])
+    out = torch.empty(1, 3, device=DEV)
+    ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), out)
+    assert out.cpu().tolist() == [[1.5, 3.0, 9.25]]
+    ob = torch.empty(1, 3, device=DEV)
+    ops.linear(x.to(DEV).bfloat16(), w.to(DEV).bfloat16(), b.to(DEV), ob)
+    assert ob.cpu().tolist() == [[1.5, 3.0, 9.25]]
+
+
+def build_attention_case(nh, nk, hd, lengths, dtype, seed, n_pages_extra=3):
+    """Sequences of the given lengths in shuffled pages; one query token per sequence at its
+    last position, plus a few mid-sequence queries."""
+    rng = np.random.default_rng(seed)
+    n_cols = max((l + 63) // 64 for l in lengths)
+    n_pages = sum((l + 63) // 64 for l in lengths) + n_pages_extra
+    perm = rng.permutation(n_pages)
+    table = -np.ones((len(lengths), n_cols), dtype=np.int32)
+    nxt = 0
+    for b, l in enumerate(lengths):
+        for c in range((l + 63) // 64):
+            table[b, c] = perm[nxt]
+            nxt += 1
+    kc, vc = make_cache(n_pages, nk, hd, dtype, seed)
+    pos, seq = [], []
+    for b, l in enumerate(lengths):
+        for p in sorted({l - 1, l // 2, 0}):
+            pos.append(p)
+            seq.append(b)
+    pos = torch.tensor(pos, dtype=torch.int32)
+    seq = torch.tensor(seq, dtype=torch.int32)
+    q = rnd((pos.numel(), nh * hd), dtype, seed + 5)
+    return q, kc, vc, torch.from_numpy(table), pos, seq
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nk,hd,window", [(4, 2, 16, 0), (4, 1, 32, 0), (9, 3, 48, 0), (28, 4, 128, 0),
+                                             (8, 8, 64, 0), (20, 2, 80, 0), (4, 2, 256, 0), (4, 2, 64, 40),
+                                             (12, 1, 128, 100)])
+def test_attn_tokens(ops, dtype, nh, nk, hd, window):
+    lengths = [1, 5, 30, 33, 64, 65, 100, 240, 1000]
+    q, kc, vc, table, pos, seq = build_attention_case(nh, nk, hd, lengths, dtype, 12)
+    scale = 1.0 / math.sqrt(hd)
+    ref = torch.empty(q.shape, dtype=torch.float64)
+    plain_ops.attn_tokens(q, kc, vc, table, pos, seq, ref, nh, nk, hd, scale, window, max(lengths))
+    dq, dk, dv, dt, dp, ds = (t.to(DEV) for t in (q, kc, vc, table, pos, seq))
+    tol = 3e-6 if dtype == torch.float32 else 1.5e-2
+    outs = []
+    for max_len in (max(lengths), 4096):          # different key splits, same result
+        out = torch.empty(q.shape, dtype=dtype, device=DEV)
+        ops.attn_tokens(dq, dk, dv, dt if max_len <= table.shape[1] * 64 else
+                        torch.nn.functional.pad(dt, (0, 64 - table.shape[1]), value=-1).contiguous(),
+                        dp, ds, out, nh, nk, hd, scale, window, max_len)
+        close(out, ref, tol, tol)
+        outs.append(out)
+    again = torch.empty(q.shape, dtype=dtype, device=DEV)
+    ops.attn_tokens(dq, dk, dv, dt, dp, ds, again, nh, nk, hd, scale, window, max(lengths))
+    assert torch.equal(again, outs[0]), "two runs differ"
+
+
+def test_attention_one_key_gives_v_and_far_key_is_found(ops):
+    # one key -> output = V exactly (src/graph/cpu_backend.rs:640-682), broadcast over the group
+    nh, nk, hd = 4, 2, 16
+    kc = torch.zeros(20, nk, 64, hd)
+    vc = rnd((20, nk, 64, hd), seed=13)
+    q = rnd((1, nh * hd), seed=14)
+    table = torch.arange(20, dtype=torch.int32).view(1, 20)
+    pos0 = torch.zeros(1, dtype=torch.int32)
+    seq0 = torch.zeros(1, dtype=torch.int32)
+    out = torch.empty(1, nh * hd, device=DEV)
+    ops.attn_tokens(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), pos0.to(DEV), seq0.to(DEV), out,
+                    nh, nk, hd, 0.25, 0, 1)
+    got = out.cpu().view(nh, hd)
+    for h in range(nh):
+        assert torch.allclose(got[h], vc[0, h // 2, 0], atol=1e-6)
+    # a far key among many: scale one key so its score stands out; output ~= its V row
+    far = 777
+    kc = rnd((20, nk, 64, hd), seed=15, scale=0.1)
+    qv = q.view(nh, hd)
+    kc[far // 64, 0, far % 64] = qv[0] * 50.0
+    pos = torch.tensor([1200], dtype=torch.int32)
+    ops.attn_tokens(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), pos.to(DEV), seq0.to(DEV), out,
+                    nh, nk, hd, 1.0, 0, 1280)
+    assert torch.allclose(out.cpu().view(nh, hd)[0], vc[far // 64, 0, far % 64], atol=1e-4)
+    # the same key just outside a window is not seen, just inside it is
+    for window, seen in ((1200 - far, False), (1200 - far + 1, True)):
+        ops.attn_tokens(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), pos.to(DEV), seq0.to(DEV), out,
+                        nh, nk, hd, 1.0, window, 1280)
+        hit = torch.allclose(out.cpu().view(nh, hd)[0], vc[far // 64, 0, far % 64], atol=1e-4)
+        assert hit == seen
