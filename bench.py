@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the Qwen2.5-7B-shaped model with random weights on one
+MI355X: `python bench.py [--gpus 1] [--steps K] [--warmup W]` prints one JSON line.
+
+A step is one decode step of the whole batch (model, sampling, feeding the token back),
+replayed from the captured HIP graph; `value` is decoded tokens per second at batch 8 with
+unequal prompt lengths up to 2048 in a context of 4096.  The line also carries the prefill
+of 2,048 tokens, the decode step's share of the HBM roofline, and decode at batch 1 and 64.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import statistics
+import sys
+import time
+
+HBM_GBS = 8000.0          # MI355X HBM3E, GB/s
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+QWEN25_7B = dict(
+    architectures=["Qwen2ForCausalLM"], model_type="qwen2", hidden_act="silu",
+    num_hidden_layers=28, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+    intermediate_size=18944, vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-6,
+    max_position_embeddings=32768, tie_word_embeddings=False, use_sliding_window=False,
+    initializer_range=0.02)
+FULL_LAYERS = QWEN25_7B["num_hidden_layers"]
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--prompt-max", type=int, default=2048)
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-graph", action="store_true")
+    return ap.parse_args()
+
+
+def matrix_params(cfg):
+    """(elements of the matrices one decode step reads per layer, of the head)."""
+    h, nh, nk = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    hd = cfg.get("head_dim") or h // nh
+    per_layer = (nh + 2 * nk) * hd * h + h * nh * hd + 3 * cfg["intermediate_size"] * h
+    small = (nh + 2 * nk) * hd + 2 * h
+    return per_layer, small, cfg["vocab_size"] * h
+
+
+def decode_bytes(cfg, elem, total_context):
+    per_layer, small, head = matrix_params(cfg)
+    nk, hd = cfg["num_key_value_heads"], cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_attention_heads"]
+    L = cfg["num_hidden_layers"]
+    weights = (L * per_layer + head) * elem + (L * small + cfg["hidden_size"]) * 4
+    kv = total_context * 2 * L * nk * hd * elem
+    return weights + kv
+
+
+def prefill_flops(cfg, t):
+    per_layer, _, head = matrix_params(cfg)
+    nh, hd = cfg["num_attention_heads"], cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_attention_heads"]
+    L = cfg["num_hidden_layers"]
+    gemm = 2.0 * t * L * per_layer + 2.0 * head          # the head runs on the one wanted row
+    attn = L * 2.0 * nh * hd * t * (t + 1)               # causal: QK^T and PV over t(t+1)/2 pairs
+    return gemm + attn
+
+
+def prompt_lengths(batch, prompt_max, seed=0):
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    lens = [int(x) for x in rng.integers(1, prompt_max + 1, size=batch)]
+    lens[0] = prompt_max
+    return lens
+
+
+def run_decode(llm, cfg, batch, prompt_max, steps, warmup, use_graph, elem):
+    """Prefills `batch` unequal prompts (untimed), then times `steps` decode steps."""
+    import numpy as np
+    import torch
+    from minfer_amd.sampling import Sampler, SamplingParams
+    eng = llm.engine
+    rng = np.random.default_rng(1)
+    lens = prompt_lengths(batch, prompt_max)
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], size=n)] for n in lens]
+    slots = [eng.new_sequence() for _ in prompts]
+    first, group, toks = [], [], 0
+    for i, p in enumerate(prompts):            # prompts in steps of at most 8192 tokens
+        group.append(i)
+        toks += len(p)
+        if toks >= 8192 or i == len(prompts) - 1:
+            lg = eng.step([slots[j] for j in group], [prompts[j] for j in group], "last")
+            first += torch.argmax(lg, dim=-1).cpu().tolist()
+            group, toks = [], 0
+    sampler = Sampler(SamplingParams.greedy())
+    sess = eng.decode_session(batch, prompt_max + warmup + steps + 8, sampler, use_graph=use_graph)
+    sess.bind(slots, first, list(range(batch)), [1] * batch)
+    for _ in range(warmup):
+        sess.step()
+    ctx_start = sum(eng.length(s) for s in slots)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        sess.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ctx_end = sum(eng.length(s) for s in slots)
+    for s in slots:
+        eng.end_sequence(s)
+    nbytes = decode_bytes(cfg, elem, (ctx_start + ctx_end) / 2.0)
+    return dict(tok_s=batch * steps / dt, ms=dt / steps * 1e3, gbs=nbytes / (dt / steps) / 1e9, bytes=nbytes)
+
+
+def run_prefill(llm, cfg, n_tokens, repeats=5):
+    import numpy as np
+    import torch
+    eng = llm.engine
+    rng = np.random.default_rng(2)
+    prompt = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=n_tokens)]
+    times = []
+    for i in range(repeats + 2):
+        s = eng.new_sequence()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.step([s], [prompt], "last")
+        torch.cuda.synchronize()
+        if i >= 2:
+            times.append(time.perf_counter() - t0)
+        eng.end_sequence(s)
+    return statistics.median(times)
+
+
+def main() -> int:
+    a = parse()
+    if a.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {a.gpus} is not supported (this engine runs on a single MI355X)")
+        return 2
+    import torch
+    from minfer_amd import LLM
+    cfg = dict(QWEN25_7B, num_hidden_layers=a.layers)
+    dtype = {"bf16": "bfloat16", "fp32": "float32"}[a.dtype]
+    elem = 2 if a.dtype == "bf16" else 4
+    batches = [a.batch] + ([] if a.no_points else [1, 64])
+    max_tokens = max(batches) * a.context
+    llm = LLM(config=cfg, random_weights=True, weight_seed=0, dtype=dtype, n_ctx=a.context,
+              n_slots=max(batches), max_tokens=max_tokens)
+    main_run = run_decode(llm, cfg, a.batch, a.prompt_max, a.steps, a.warmup, not a.no_graph, elem)
+    pre_s = run_prefill(llm, cfg, a.prefill_tokens)
+    points = {}
+    for b in batches[1:]:
+        r = run_decode(llm, cfg, b, a.prompt_max, max(16, a.steps // 2), max(4, a.warmup // 2),
+                       not a.no_graph, elem)
+        points[f"decode_b{b}"] = round(r["tok_s"], 1)
+    flops = prefill_flops(cfg, a.prefill_tokens)
+    out = {
+        "metric": "decode tok/s, Qwen2.5-7B shape, batch 8", "value": round(main_run["tok_s"], 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(main_run["ms"], 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": a.dtype, "data": "synthetic",
+        "config": {"model": "Qwen2.5-7B shape, random weights", "layers": a.layers, "layers_full": FULL_LAYERS,
+                   "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+                   "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["hidden_size"] // cfg["num_attention_heads"],
+                   "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
+                   "global_batch": a.batch, "seq_len": a.context, "prompt_max": a.prompt_max,
+                   "prefill_tokens": a.prefill_tokens, "parallelism": "single GPU",
+                   "decode_graph": not a.no_graph},
+        "prefill": {"value": round(a.prefill_tokens / pre_s, 1), "tokens": a.prefill_tokens,
+                    "ms": round(pre_s * 1e3, 3), "frac": round(flops / pre_s / PEAK_FLOPS[a.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(main_run["gbs"], 1), "peak": HBM_GBS, "unit": "GB/s",
+                     "frac": round(main_run["gbs"] / HBM_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

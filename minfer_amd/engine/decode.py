@@ -1,0 +1,119 @@
+"""Decode steps with everything that changes per step kept on the device, so that one step
+(model, sampling, moving every sequence on by one) can be captured once as a HIP graph and
+replayed.
+
+The reference reuses its built graph across decode steps because positions are data, not
+structure (src/graph/params.rs:39-52, src/graph/cache.rs:37-54 of yusiwen/minfer), and its
+CUDA path captures the step as a CUDA graph (src/cuda.rs:480-527).  Here token ids,
+positions, page tables, sampler counters and the recent-token windows live in buffers of a
+fixed size per batch size; the host only reserves pages ahead and reads the sampled tokens.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from ..cache.paged import PAGE
+from ..kernels import ops
+from ..sampling.params import REPEAT_LAST_N
+from .batch import StepContext
+
+
+class DecodeSession:
+    """Buffers (and, once captured, the graph) for `n_seqs` sequences decoding up to
+    `max_len` positions.  `bind` points it at a set of live sequences."""
+
+    def __init__(self, engine, n_seqs: int, max_len: int, sampler, use_graph: bool = True):
+        self.engine, self.n, self.sampler = engine, n_seqs, sampler
+        self.max_len = max_len
+        self.n_cols = (max_len + PAGE - 1) // PAGE
+        self.use_graph = use_graph and engine.device.type == "cuda"
+        dev = engine.device
+        i32 = dict(dtype=torch.int32, device=dev)
+        self.token_ids = torch.zeros(n_seqs, **i32)
+        self.positions = torch.zeros(n_seqs, **i32)
+        self.seq_of_tok = torch.arange(n_seqs, **i32)
+        self.cu_seqlens = torch.arange(n_seqs + 1, **i32)
+        self.slot_ids = torch.zeros(n_seqs, **i32)
+        self.tables: Dict[int, torch.Tensor] = {
+            id(g): torch.full((n_seqs, self.n_cols), -1, **i32) for g in engine.cache.groups}
+        self.keys = torch.zeros(n_seqs, dtype=torch.int64, device=dev)
+        self.steps = torch.zeros(n_seqs, **i32)
+        self.sampled = torch.zeros(n_seqs, **i32)
+        self.prev = torch.zeros((n_seqs, REPEAT_LAST_N), **i32)
+        self.n_prev = torch.zeros(n_seqs, **i32)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.warm = False
+        self.slots: List[int] = []
+        self._host_tables: Dict[int, List[List[int]]] = {}
+        engine.model.prepare(max_len)
+
+    # ------------------------------------------------------------ binding
+    def bind(self, slots: Sequence[int], next_tokens: Sequence[int], keys: Sequence[int],
+             steps: Sequence[int]) -> None:
+        """The sequences in `slots` will each be fed `next_tokens[i]` at their current length."""
+        if len(slots) != self.n:
+            raise ValueError(f"session is for {self.n} sequences, got {len(slots)}")
+        cache, dev = self.engine.cache, self.engine.device
+        self.slots = list(slots)
+        lengths = [cache.length(s) for s in slots]
+        self.token_ids.copy_(torch.tensor(list(next_tokens), dtype=torch.int32))
+        self.positions.copy_(torch.tensor(lengths, dtype=torch.int32))
+        self.slot_ids.copy_(torch.tensor(self.slots, dtype=torch.int32))
+        self.keys.copy_(torch.tensor(list(keys), dtype=torch.int64))
+        self.steps.copy_(torch.tensor(list(steps), dtype=torch.int32))
+        self._host_tables = {}
+
+    def set_windows(self, windows: Sequence[Sequence[int]]) -> None:
+        """Recent tokens of each sequence for the penalties (at most the last 64)."""
+        rows = [list(w)[-REPEAT_LAST_N:] for w in windows]
+        flat = torch.zeros((self.n, REPEAT_LAST_N), dtype=torch.int32)
+        for i, r in enumerate(rows):
+            if r:
+                flat[i, :len(r)] = torch.tensor(r, dtype=torch.int32)
+        self.prev.copy_(flat)
+        self.n_prev.copy_(torch.tensor([len(r) for r in rows], dtype=torch.int32))
+
+    # ------------------------------------------------------------ one step
+    def _context(self) -> StepContext:
+        return StepContext(
+            cache=self.engine.cache, n_tokens=self.n, n_seqs=self.n, token_ids=self.token_ids,
+            positions=self.positions, seq_of_tok=self.seq_of_tok, cu_seqlens=self.cu_seqlens,
+            start_pos=self.positions, slot_ids=self.slot_ids, logit_rows=None, page_tables=self.tables,
+            max_len=self.max_len, max_new=1, all_decode=True, host_slots=list(self.slots),
+            host_new=[1] * self.n, host_start=None)
+
+    def _run(self) -> None:
+        logits = self.engine.model.forward(self._context())
+        self.sampler(logits, self.keys, self.steps, self.sampled, self.prev, self.n_prev)
+        ops.advance(self.token_ids, self.sampled, self.positions, self.steps)
+
+    def step(self) -> List[int]:
+        """Runs one token of every bound sequence and returns the next sampled tokens."""
+        cache = self.engine.cache
+        new_len = {s: cache.length(s) + 1 for s in self.slots}
+        if max(new_len.values()) > self.max_len:
+            raise ValueError(f"decode session was sized for {self.max_len} positions")
+        cache.reserve(new_len)
+        for g in cache.groups:
+            rows = cache.page_rows(g, self.slots, self.n_cols)
+            if self._host_tables.get(id(g)) != rows:
+                self.tables[id(g)].copy_(torch.tensor(rows, dtype=torch.int32))
+                self._host_tables[id(g)] = rows
+        if not self.use_graph:
+            self._run()
+        elif self.graph is not None:
+            self.graph.replay()
+        elif not self.warm:
+            self._run()                      # first step runs eagerly: loads and sizes everything
+            self.warm = True
+        else:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self._run()
+            self.graph = graph
+            graph.replay()
+        tokens = self.sampled.cpu().tolist()
+        cache.commit(new_len)
+        return tokens

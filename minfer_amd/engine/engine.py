@@ -37,6 +37,7 @@ class Engine:
         self.cache = Cache(model.cache_requests(), max_tokens, self.max_seqs, model.rt.dtype, self.device)
         self.vocab_size = model.spec.vocab_size
         self.max_positions = model.spec.max_positions
+        self._sessions = {}
 
     # ------------------------------------------------------------ sequences
     def new_sequence(self) -> int:
@@ -49,6 +50,25 @@ class Engine:
 
     def length(self, slot: int) -> int:
         return self.cache.length(slot)
+
+    def capacity_tokens(self) -> int:
+        """Tokens the cache can hold when nothing is live (whole pages)."""
+        return self.cache.n_pages * PAGE
+
+    def stop_tokens(self):
+        """The model's own stop tokens (config.json eos_token_id; the reference stops on
+        eos or <|im_end|>, src/main.rs:626-628 of yusiwen/minfer)."""
+        return tuple(self.model.spec.stop_tokens)
+
+    def decode_session(self, n_seqs: int, max_len: int, sampler, use_graph: bool = True):
+        """A `DecodeSession` for this batch size, reused (with its captured graph) while the
+        size, the reach and the sampling options stay the same."""
+        from .decode import DecodeSession
+        max_len = min(self.max_positions, (max_len + 255) // 256 * 256)
+        key = (n_seqs, max_len, sampler.params, use_graph)
+        if key not in self._sessions:
+            self._sessions[key] = DecodeSession(self, n_seqs, max_len, sampler, use_graph)
+        return self._sessions[key]
 
     # ------------------------------------------------------------ one step
     def build_context(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], want: Want) -> StepContext:

@@ -1,0 +1,168 @@
+"""The generation loop: batches of unequal prompts, stop tokens, sequences that end
+earlier, and as many batches one after another as there are requests.
+
+Shape of the reference's loop (src/main.rs:495-598 of yusiwen/minfer): the prompt in one
+call, then `sample -> stop? -> append -> forward(one token)`.  A stop token ends the
+sequence before it is appended and is not fed back (src/main.rs:568); the bound is the
+number of new tokens (src/main.rs:559); a full context ends the sequence with reason
+'length' (src/server/chat.rs:117-121).  Prefill and decode are timed apart and the decode
+rate excludes the prefill (src/main.rs:505-508,615-623).  Unlike the reference, no forward
+is run for a token that will not be followed by another.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Optional, Sequence
+
+import torch
+
+from ..cache.paged import PAGE
+from ..sampling.params import REPEAT_LAST_N, SamplingParams
+from ..sampling.sampler import Sampler
+
+
+@dataclass
+class GenerationResult:
+    tokens: List[List[int]]                 # generated ids per request, stop token not included
+    finish_reasons: List[str]               # 'stop' | 'length'
+    prefill_tokens: int = 0
+    prefill_seconds: float = 0.0
+    decode_tokens: int = 0                  # tokens produced by decode steps
+    decode_seconds: float = 0.0
+    batches: List[List[int]] = field(default_factory=list)   # request indices of each batch
+
+    @property
+    def prefill_rate(self) -> float:
+        return self.prefill_tokens / self.prefill_seconds if self.prefill_seconds > 0 else 0.0
+
+    @property
+    def decode_rate(self) -> float:
+        return self.decode_tokens / self.decode_seconds if self.decode_seconds > 0 else 0.0
+
+
+def _sync(engine) -> None:
+    if getattr(engine, "device", None) is not None and engine.device.type == "cuda":
+        torch.cuda.synchronize(engine.device)
+
+
+def plan_batches(prompt_lengths: Sequence[int], max_new: int, capacity_tokens: int, max_batch: int,
+                 max_positions: int) -> List[List[int]]:
+    """Requests in order, as many per batch as the cache can hold to their last token (each
+    rounded up to whole pages) and as there are slots."""
+    batches, cur, used = [], [], 0
+    for i, n in enumerate(prompt_lengths):
+        if n < 1:
+            raise ValueError(f"request {i}: empty prompt")
+        if n > max_positions:
+            raise ValueError(f"request {i}: prompt of {n} tokens exceeds the model's {max_positions} positions")
+        need = (min(n + max_new, max_positions) + PAGE - 1) // PAGE * PAGE
+        if need > capacity_tokens:
+            raise ValueError(f"request {i}: needs {need} cache tokens, the cache holds {capacity_tokens}")
+        if cur and (used + need > capacity_tokens or len(cur) >= max_batch):
+            batches.append(cur)
+            cur, used = [], 0
+        cur.append(i)
+        used += need
+    if cur:
+        batches.append(cur)
+    return batches
+
+
+def generate(engine, prompts: Sequence[Sequence[int]], params: Optional[SamplingParams] = None,
+             max_new: int = 512, stop_tokens: Optional[Sequence[int]] = None, max_batch: Optional[int] = None,
+             use_graph: bool = True, on_token: Optional[Callable[[int, int], None]] = None,
+             n_ctx: Optional[int] = None) -> GenerationResult:
+    """Generates up to `max_new` tokens for every prompt (lists of token ids).  `stop_tokens`
+    defaults to the model's own; `on_token(request, token)` is called for each emitted token;
+    `n_ctx` bounds the positions of one sequence (default: the model's own bound)."""
+    params = params or SamplingParams()
+    sampler = Sampler(params)
+    if stop_tokens is None:
+        stop_tokens = engine.stop_tokens()
+    stops = set(int(t) for t in stop_tokens)
+    n_req = len(prompts)
+    result = GenerationResult(tokens=[[] for _ in range(n_req)], finish_reasons=["length"] * n_req)
+    if n_req == 0 or max_new <= 0:
+        return result
+    capacity = engine.capacity_tokens()
+    max_batch = min(max_batch or engine.max_seqs, engine.max_seqs)
+    limit = min(engine.max_positions, n_ctx) if n_ctx else engine.max_positions
+    result.batches = plan_batches([len(p) for p in prompts], max_new, capacity, max_batch, limit)
+    dev = engine.device
+
+    def decide(req: int, tok: int, slot: int, live: Dict[int, int]) -> None:
+        """After sampling `tok` for request `req`: stop, emit, or emit and end."""
+        if tok in stops:
+            result.finish_reasons[req] = "stop"
+        else:
+            result.tokens[req].append(tok)
+            if on_token:
+                on_token(req, tok)
+            if len(result.tokens[req]) < max_new and engine.length(slot) + 1 <= limit:
+                live[req] = slot
+                return
+            result.finish_reasons[req] = "length"
+        engine.end_sequence(slot)
+
+    for batch in result.batches:
+        slots = {r: engine.new_sequence() for r in batch}
+        windows = {r: list(prompts[r])[-REPEAT_LAST_N:] for r in batch}
+        _sync(engine)
+        t0 = time.perf_counter()
+        logits = engine.step([slots[r] for r in batch], [list(prompts[r]) for r in batch], "last")
+        first = _sample(sampler, logits, batch, [0] * len(batch), [windows[r] for r in batch], dev)
+        _sync(engine)
+        result.prefill_seconds += time.perf_counter() - t0
+        result.prefill_tokens += sum(len(prompts[r]) for r in batch)
+        live: Dict[int, int] = {}
+        for r, tok in zip(batch, first):
+            windows[r] = (windows[r] + [tok])[-REPEAT_LAST_N:]
+            decide(r, tok, slots[r], live)
+        next_tok = {r: result.tokens[r][-1] for r in live}
+
+        t0 = time.perf_counter()
+        session, bound = None, None
+        while live:
+            order = sorted(live)
+            if use_graph and hasattr(engine, "decode_session"):
+                if bound != order:
+                    cap = max(min(len(prompts[r]) + max_new, limit) for r in order)
+                    session = engine.decode_session(len(order), cap, sampler)
+                    session.bind([live[r] for r in order], [next_tok[r] for r in order], order,
+                                 [len(result.tokens[r]) for r in order])
+                    bound = order
+                if params.has_penalties:
+                    session.set_windows([windows[r] for r in order])
+                toks = session.step()
+            else:
+                logits = engine.step([live[r] for r in order], [[next_tok[r]] for r in order], "last")
+                toks = _sample(sampler, logits, order, [len(result.tokens[r]) for r in order],
+                               [windows[r] for r in order], dev)
+            result.decode_tokens += len(order)
+            was, live = live, {}
+            for r, tok in zip(order, toks):
+                windows[r] = (windows[r] + [tok])[-REPEAT_LAST_N:]
+                decide(r, tok, was[r], live)
+            next_tok = {r: result.tokens[r][-1] for r in live}
+        _sync(engine)
+        result.decode_seconds += time.perf_counter() - t0
+    return result
+
+
+def _sample(sampler: Sampler, logits: torch.Tensor, keys: Sequence[int], steps: Sequence[int],
+            windows: Sequence[Sequence[int]], device) -> List[int]:
+    n = logits.shape[0]
+    out = torch.empty(n, dtype=torch.int32, device=device)
+    prev = n_prev = None
+    if sampler.params.has_penalties:
+        flat = torch.zeros((n, REPEAT_LAST_N), dtype=torch.int32)
+        for i, w in enumerate(windows):
+            w = list(w)[-REPEAT_LAST_N:]
+            if w:
+                flat[i, :len(w)] = torch.tensor(w, dtype=torch.int32)
+        prev = flat.to(device)
+        n_prev = torch.tensor([min(len(w), REPEAT_LAST_N) for w in windows], dtype=torch.int32, device=device)
+    sampler(logits, torch.tensor(list(keys), dtype=torch.int64, device=device),
+            torch.tensor(list(steps), dtype=torch.int32, device=device), out, prev, n_prev)
+    return out.cpu().tolist()

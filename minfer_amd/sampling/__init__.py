@@ -1,0 +1,5 @@
+from .params import REPEAT_LAST_N, SamplingParams
+from .rng import mix64, uniform
+from .sampler import Sampler
+
+__all__ = ["REPEAT_LAST_N", "SamplingParams", "Sampler", "mix64", "uniform"]

@@ -120,11 +120,50 @@ def attn_prefill(q, kcache, vcache, page_table, ctx, out, n_heads, n_kv_heads, h
 
 # ------------------------------------------------------------------ sampling
 def argmax(logits, out):
-    out.copy_(torch.argmax(logits, dim=-1).to(out.dtype))   # first maximum
+    import plain_qwen2 as pq
+    for i in range(logits.shape[0]):
+        out[i] = pq.greedy(logits[i].numpy())
+
+
+def sample(logits, temp, seed, keys, steps, out, forced_r=None):
+    import plain_qwen2 as pq
+    from minfer_amd.sampling.rng import uniform
+    for i in range(logits.shape[0]):
+        if temp < 1e-6:
+            out[i] = pq.greedy(logits[i].numpy())
+            continue
+        r = float(forced_r[i]) if forced_r is not None else uniform(seed, int(keys[i]), int(steps[i]))
+        out[i] = pq.sample_from_probs(pq.temperature_probs(logits[i].numpy(), temp), r)
+
+
+def penalties(logits, prev, n_prev, repeat, frequency, presence):
+    import plain_qwen2 as pq
+    for i in range(logits.shape[0]):
+        window = prev[i, :int(n_prev[i])].tolist()
+        logits[i] = torch.from_numpy(pq.apply_penalties(logits[i].numpy(), window, repeat, frequency, presence))
+
+
+def top_k(logits, k):
+    import plain_qwen2 as pq
+    for i in range(logits.shape[0]):
+        logits[i] = torch.from_numpy(pq.apply_top_k(logits[i].numpy(), k))
+
+
+def top_p(logits, p):
+    import plain_qwen2 as pq
+    for i in range(logits.shape[0]):
+        logits[i] = torch.from_numpy(pq.apply_top_p(logits[i].numpy(), p))
+
+
+def advance(next_ids, sampled, positions, steps):
+    next_ids.copy_(sampled)
+    positions += 1
+    steps += 1
 
 
 NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", "rope_table",
-         "rope_kvwrite", "linear", "attn_tokens", "attn_prefill"]
+         "rope_kvwrite", "linear", "attn_tokens", "attn_prefill", "argmax", "sample", "penalties",
+         "top_k", "top_p", "advance"]
 
 
 def install(monkeypatch):
