@@ -260,14 +260,16 @@ def temperature_probs(logits: np.ndarray, temp: float) -> np.ndarray:
     return e * inv
 
 
-def sample_from_probs(probs: np.ndarray, r: float) -> int:
+def sample_from_probs(probs: np.ndarray, r: float, acc=np.float32) -> int:
     """Walk indices upward, skipping p <= 0, return the first whose running sum reaches r;
-    the last index if none does.  src/sampler.rs:253-266."""
-    cum = np.float32(0.0)
+    the last index if none does.  src/sampler.rs:253-266.  The reference keeps the running
+    sum in f32 (`acc`); over a vocabulary of 10^5 entries that sum drifts by about 1e-4, so
+    tests of large vocabularies pass acc=np.float64, the same walk without the drift."""
+    cum = acc(0.0)
     for i, v in enumerate(probs):
         if v <= 0.0:
             continue
-        cum = np.float32(cum + v)
+        cum = acc(cum + acc(v))
         if r <= cum:
             return i
     return len(probs) - 1

@@ -1,0 +1,188 @@
+"""Generation on the GPU through the entry points: greedy and sampled tokens against the
+plain implementation, the captured decode step against the eager one, long decoding, the
+first tokens of a sequence, the command line, and trace replay as a program."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import plain_qwen2 as pq
+from minfer_amd.sampling import uniform
+from replays import (batch_steps, compare, plain_logits, requests_for, run_steps, tail_steps, whole_steps)
+from tiny import TINIES, random_tokens, write_tiny
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("gen")
+    return {n: write_tiny(tmp, n, seed=7) for n in TINIES}
+
+
+def plain_generate(plain, prompt, n, temp, seed, key, **opts):
+    seq, out = list(prompt), []
+    for s in range(n):
+        logits = plain.forward(seq)[-1].astype(np.float32)
+        t = pq.sample(logits, temp, uniform(seed, key, s), opts.get("top_k", 40), opts.get("top_p", 0.95),
+                      opts.get("repeat", 1.1), 0.0, 0.0, pq.recent_window(seq))
+        out.append(t)
+        seq.append(t)
+    return out
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_and_sampled_generation_match_plain(folders, name):
+    from minfer_amd import LLM
+    plain = pq.PlainQwen2.from_folder(folders[name])
+    vocab = TINIES[name]["vocab_size"]
+    lens = (5, 9, 13) if name == "A" else (1, 7, 31, 64)
+    steps = 8 if name == "A" else 16
+    prompts = [random_tokens(vocab, n, 10 + i) for i, n in enumerate(lens)]
+    llm = LLM(folders[name], dtype="float32", n_ctx=128, n_slots=4)
+    for temp in (0.0, 0.8):
+        eager = llm.generate(prompts, max_new=steps, temp=temp, seed=1, stop_tokens=[], use_graph=False)
+        graph = llm.generate(prompts, max_new=steps, temp=temp, seed=1, stop_tokens=[], use_graph=True)
+        assert eager.tokens == graph.tokens
+        for i, p in enumerate(prompts):
+            assert graph.tokens[i] == plain_generate(plain, p, steps, temp, 1, i), (name, temp, i)
+    # bfloat16: the same tokens from the captured and the eager step
+    lb = LLM(folders[name], dtype="bfloat16", n_ctx=128, n_slots=4)
+    a = lb.generate(prompts, max_new=steps, temp=0.0, repeat_penalty=1.0, stop_tokens=[], use_graph=False)
+    b = lb.generate(prompts, max_new=steps, temp=0.0, repeat_penalty=1.0, stop_tokens=[], use_graph=True)
+    assert a.tokens == b.tokens and all(len(t) == steps for t in b.tokens)
+    assert not lb.engine.cache.live_slots()
+
+
+def test_stop_tokens_end_sequences_early_and_batches_follow_each_other(folders):
+    from minfer_amd import LLM
+    plain = pq.PlainQwen2.from_folder(folders["A"])
+    prompts = [random_tokens(512, n, 30 + i) for i, n in enumerate((4, 11, 6, 20, 3))]
+    llm = LLM(folders["A"], dtype="float32", n_ctx=64, n_slots=2)
+    free = llm.generate(prompts, max_new=12, temp=0.8, seed=5, stop_tokens=[])
+    assert free.batches == [[0, 1], [2, 3], [4]]
+    # declare each request's 4th token (if new to it) a stop token for everyone
+    stops = {t[3] for t in free.tokens}
+    res = llm.generate(prompts, max_new=12, temp=0.8, seed=5, stop_tokens=sorted(stops))
+    for i, p in enumerate(prompts):
+        want = plain_generate(plain, p, 12, 0.8, 5, i)
+        cut = next((j for j, t in enumerate(want) if t in stops), 12)
+        assert res.tokens[i] == want[:cut]
+        assert res.finish_reasons[i] == ("stop" if cut < 12 else "length")
+    llm.engine.cache.check_invariants()
+
+
+def test_long_decoding_crosses_pages(folders):
+    """300 decode steps after a short prompt, through the captured step, teacher-forced
+    against the plain implementation at a few places."""
+    from minfer_amd import LLM
+    plain = pq.PlainQwen2.from_folder(folders["B"])
+    llm = LLM(folders["B"], dtype="float32", n_ctx=512, n_slots=2)
+    prompts = [random_tokens(1000, 3, 40), random_tokens(1000, 62, 41)]
+    res = llm.generate(prompts, max_new=300, temp=0.9, seed=2, stop_tokens=[])
+    assert [len(t) for t in res.tokens] == [300, 300]
+    for i, p in enumerate(prompts):
+        seq = list(p) + res.tokens[i]
+        full = plain.forward(seq[:-1]).astype(np.float32)
+        for s in (0, 1, 2, 61, 62, 63, 64, 65, 127, 128, 199, 256, 299):
+            window = pq.recent_window(seq[:len(p) + s])
+            t = pq.sample(full[len(p) + s - 1], 0.9, uniform(2, i, s), 40, 0.95, 1.1, 0, 0, window)
+            assert t == res.tokens[i][s], (i, s)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(folders, dtype):
+    """Prompts of one token, the first decoded token, a prompt that ends on a page edge."""
+    from minfer_amd import Engine, load_model
+    plain = pq.PlainQwen2.from_folder(folders["C"])
+    eng = Engine(load_model(folders["C"], dtype=dtype), max_tokens=64 * 6)
+    reqs = requests_for(777, (1, 2, 64, 65), seed=9)
+    ref = plain_logits(plain, reqs)
+    steps = []
+    ids = list(reqs)
+    steps.append(dict(step=0, entries=[dict(id=r, tokens=reqs[r][:1] if len(reqs[r]) < 3 else reqs[r][:-1],
+                                            want=[0] if len(reqs[r]) < 3 else [len(reqs[r]) - 2])
+                                       for r in ids], end=["r0"]))
+    steps.append(dict(step=1, entries=[dict(id=r, tokens=reqs[r][-1:], want=[0]) for r in ids[1:]], end=ids[1:]))
+    compare(run_steps(eng, steps), ref, dtype, "first tokens")
+
+
+def test_command_line(folders, tmp_path):
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    exe = [sys.executable, os.path.join(ROOT, "bin", "minfer")]
+    r = subprocess.run(exe + [folders["A"], "--prompt-tokens", "5,6,7;9,10", "--greedy", "--repeat-penalty", "1.0",
+                              "-n", "5", "--dtype", "float32", "--n-ctx", "64", "--stop-token", "100000"],
+                       capture_output=True, text=True, env=env, timeout=300)
+    assert r.returncode == 0, r.stderr
+    lines = [l for l in r.stdout.strip().splitlines() if l]
+    plain = pq.PlainQwen2.from_folder(folders["A"])
+    for line, prompt in zip(lines, ([5, 6, 7], [9, 10])):
+        seq = list(prompt)
+        for t in (int(x) for x in line.split(",")):
+            assert t == pq.greedy(plain.forward(seq)[-1])
+            seq.append(t)
+    assert "Prefill: 5 tokens" in r.stderr and "Generated:" in r.stderr and "Total:" in r.stderr
+    cfg = tmp_path / "c.json"
+    cfg.write_text(json.dumps(TINIES["B"]))
+    r = subprocess.run(exe + ["--config", str(cfg), "--random-weights", "--prompt-tokens", "1,2,3", "--max-new", "4",
+                              "--temp", "0.8", "--seed", "3"], capture_output=True, text=True, env=env, timeout=300)
+    assert r.returncode == 0 and len(r.stdout.strip().split(",")) <= 4, r.stderr
+    r = subprocess.run(exe + [folders["A"], "--bogus"], capture_output=True, text=True, env=env, timeout=60)
+    assert r.returncode == 1 and "unknown option --bogus" in r.stderr and "USAGE" in r.stderr
+    r = subprocess.run(exe + [folders["A"], "--prompt-tokens", "1", "--temp"], capture_output=True, text=True,
+                       env=env, timeout=60)
+    assert r.returncode == 1 and "requires a value" in r.stderr
+
+
+def replay_program(folder, dtype, steps, out_dir, max_tokens):
+    """Runs bin/trace_run as a program; sends each step only after the last `done`."""
+    exe = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+           "--out", out_dir, "--max-tokens", str(max_tokens)]
+    p = subprocess.Popen(exe, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, bufsize=1)
+    pos, rows = {}, {}
+    vocab = json.load(open(os.path.join(folder, "config.json")))["vocab_size"]
+    try:
+        for st in steps:
+            p.stdin.write(json.dumps(st) + "\n")
+            p.stdin.flush()
+            assert p.stdout.readline().strip() == f"done {st['step']}"
+            n_want = sum(len(e["want"]) for e in st["entries"])
+            path = os.path.join(out_dir, f"{st['step']}.f32")
+            if n_want:
+                arr = np.fromfile(path, dtype="<f4").reshape(n_want, vocab)
+                r = 0
+                for e in st["entries"]:
+                    for w in e["want"]:
+                        rows[(e["id"], pos.get(e["id"], 0) + w)] = arr[r]
+                        r += 1
+            else:
+                assert not os.path.exists(path)
+            for e in st["entries"]:
+                pos[e["id"]] = pos.get(e["id"], 0) + len(e["tokens"])
+        p.stdin.close()
+        assert p.wait(timeout=60) == 0
+    finally:
+        if p.poll() is None:
+            p.kill()
+    return rows
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(folders, tmp_path, dtype):
+    plain = pq.PlainQwen2.from_folder(folders["B"])
+    reqs = requests_for(1000, (1, 7, 31, 64, 90), seed=8)
+    ref = plain_logits(plain, reqs)
+    ids = list(reqs)
+    # peak: the batch of three at its end, each request rounded up to 64
+    peak = max(sum((len(reqs[r]) + 63) // 64 * 64 for r in b) for b in (ids[:3], ids[3:]))
+    plans = {"whole": whole_steps(reqs), "tail": tail_steps(reqs), "batches": batch_steps(reqs, [ids[:3], ids[3:]])}
+    # a step that wants nothing writes no file
+    plans["batches"][0]["entries"][0]["want"] = []
+    for what, steps in plans.items():
+        out = tmp_path / f"{dtype}_{what}"
+        rows = replay_program(folders["B"], dtype, steps, str(out), peak if what == "batches" else 128)
+        compare(rows, ref, dtype, f"trace_run {what}")

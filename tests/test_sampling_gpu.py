@@ -1,0 +1,150 @@
+"""The sampling kernels against the plain sampler (tests/plain_qwen2.py)."""
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen2 as pq
+from minfer_amd.sampling import Sampler, SamplingParams, uniform
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from minfer_amd.kernels import ops as o
+    return o
+
+
+def logits_rows(rows, vocab, seed, scale=3.0):
+    return (torch.randn(rows, vocab, generator=torch.Generator().manual_seed(seed)) * scale).float()
+
+
+@pytest.mark.parametrize("rows,vocab", [(1, 4), (5, 1000), (3, 152064), (64, 777)])
+def test_argmax_first_maximum(ops, rows, vocab):
+    l = logits_rows(rows, vocab, 1)
+    l[0, vocab // 2] = l[0, vocab - 1] = 50.0                 # a tie: the lower index wins
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    ops.argmax(l.to(DEV), out)
+    assert out.cpu().tolist() == [pq.greedy(r.numpy()) for r in l]
+    assert out[0].item() == vocab // 2
+
+
+def test_reference_vectors(ops):
+    def run(fn, vals, *a):
+        t = torch.tensor([vals], dtype=torch.float32, device=DEV)
+        fn(t, *a)
+        return t.cpu()[0].tolist()
+    out = torch.empty(1, dtype=torch.int32, device=DEV)
+    ops.argmax(torch.tensor([[1., 5, -2, 3]], device=DEV), out)
+    assert out.item() == 1                                                    # src/sampler.rs:313-317
+    k = run(ops.top_k, [1., 5, 2, 4], 2)
+    assert k[1] == 5 and k[3] == 4 and k[0] == k[2] == float("-inf")           # :344-351
+    p = run(ops.top_p, [1., 2, 3, 4], 0.5)
+    assert p[3] == 4.0 and all(v == float("-inf") for v in p[:3])              # :354-363
+    prev = torch.tensor([[3, 3, 0, 0]], dtype=torch.int32, device=DEV)
+    n1, n2 = (torch.tensor([n], dtype=torch.int32, device=DEV) for n in (1, 2))
+    assert run(ops.penalties, [1., 2, 3, 4], prev, n1, 2.0, 0.0, 0.0)[3] == 2.0      # :320-333
+    assert run(ops.penalties, [-4., -2, -1, -3], prev, n1, 2.0, 0.0, 0.0)[3] == -6.0
+    assert run(ops.penalties, [1., 2, 3, 4], prev, n2, 1.0, 0.5, 0.0) == [1, 2, 3, 3]  # :388-397
+    assert abs(run(ops.penalties, [1., 2, 3, 4], prev, n2, 1.0, 0.0, 0.8)[3] - 3.2) < 1e-6
+    prev0 = torch.tensor([[0, 99]], dtype=torch.int32, device=DEV)
+    assert run(ops.penalties, [4., -4, 0, 0], prev0, n2, 2.0, 1.0, 1.0) == [1, -4, 0, 0]  # :411-427, :448-452
+
+
+@pytest.mark.parametrize("vocab,k", [(1000, 40), (152064, 40), (777, 1), (50, 49), (3000, 700)])
+def test_top_k_matches_plain(ops, vocab, k):
+    l = logits_rows(4, vocab, 2)
+    l[1, :50] = 1.25                                           # many ties around the threshold
+    d = l.to(DEV).clone()
+    ops.top_k(d, k)
+    for i in range(4):
+        assert np.array_equal(d[i].cpu().numpy(), pq.apply_top_k(l[i].numpy(), k))
+
+
+@pytest.mark.parametrize("vocab,p,pre_k", [(1000, 0.95, 40), (152064, 0.95, 40), (500, 0.5, 0), (4000, 0.9, 0),
+                                           (64, 0.3, 0)])
+def test_top_p_matches_plain(ops, vocab, p, pre_k):
+    l = logits_rows(4, vocab, 3)
+    l[2, :10] = 2.0                                            # equal probabilities: index order decides
+    if pre_k:
+        l = torch.stack([torch.from_numpy(pq.apply_top_k(r.numpy(), pre_k)) for r in l])
+    d = l.to(DEV).clone()
+    ops.top_p(d, p)
+    for i in range(4):
+        want = pq.apply_top_p(l[i].numpy(), p)
+        got = d[i].cpu().numpy()
+        if not np.array_equal(got, want):
+            # the two may differ by one element only when the cumulative mass touches p within rounding
+            kept_w, kept_g = np.isfinite(want), np.isfinite(got)
+            assert abs(int(kept_w.sum()) - int(kept_g.sum())) <= 1
+            probs = torch.softmax(l[i].double(), 0).numpy()
+            assert abs(min(probs[kept_w].sum(), probs[kept_g].sum()) - p) < 1e-5
+
+
+@pytest.mark.parametrize("vocab,temp", [(100, 0.8), (152064, 0.8), (777, 1.3), (1000, 0.05)])
+def test_temperature_draw_matches_plain(ops, vocab, temp):
+    rows = 16
+    l = logits_rows(rows, vocab, 4)
+    if vocab == 100:
+        l = (torch.arange(100).float() * 0.1).repeat(rows, 1)              # src/sampler.rs:366-375
+    rs = np.random.default_rng(5).random(rows).astype(np.float32)
+    rs[0], rs[1] = 0.0, 0.99999994
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    keys = torch.zeros(rows, dtype=torch.int64, device=DEV)
+    steps = torch.zeros(rows, dtype=torch.int32, device=DEV)
+    ops.sample(l.to(DEV), temp, 0, keys, steps, out, torch.from_numpy(rs).to(DEV))
+    for i in range(rows):
+        probs = pq.temperature_probs(l[i].numpy(), temp)
+        # the kernel keeps the running sum in double; so does the oracle for a large vocabulary
+        # (the reference's f32 running sum drifts by ~1e-4 over 10^5 entries)
+        acc = np.float32 if vocab <= 1000 else np.float64
+        want, got = pq.sample_from_probs(probs, float(rs[i]), acc), int(out[i])
+        if want != got:          # only when the draw is within rounding of the running sum at both
+            cum = np.cumsum(probs.astype(np.float64))
+            assert abs(cum[got] - rs[i]) < 1e-6 and abs(cum[want] - rs[i]) < 1e-6, (i, want, got)
+    # masked entries are never drawn
+    m = torch.full((1, 50), float("-inf"))
+    m[0, 7] = m[0, 31] = 1.0
+    for r, want in ((0.0, 7), (0.49, 7), (0.51, 31), (0.999, 31)):
+        ops.sample(m.to(DEV), 1.0, 0, keys[:1], steps[:1], out[:1], torch.tensor([r], device=DEV))
+        assert out[0].item() == want
+
+
+def test_device_uniform_is_the_host_uniform_and_draws_follow_softmax(ops):
+    rows, vocab = 4000, 3
+    small = torch.tensor([0.0, 1.0, 2.0]).repeat(rows, 1).to(DEV)
+    keys = torch.arange(rows, dtype=torch.int64, device=DEV)
+    steps = (torch.arange(rows, dtype=torch.int32, device=DEV) % 7)
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    ops.sample(small, 1.0, 42, keys, steps, out)
+    probs = pq.temperature_probs(np.array([0, 1, 2], dtype=np.float32), 1.0)
+    want = [pq.sample_from_probs(probs, uniform(42, i, i % 7)) for i in range(rows)]
+    assert out.cpu().tolist() == want
+    counts = np.bincount(out.cpu().numpy(), minlength=3)
+    expect = probs * rows
+    assert (np.abs(counts - expect) < 4 * np.sqrt(expect)).all()
+
+
+def test_pipeline_order_and_greedy_with_penalty():
+    l = torch.tensor([[1., 2, 3, 4]], device=DEV)
+    out = torch.empty(1, dtype=torch.int32, device=DEV)
+    keys, steps = torch.zeros(1, dtype=torch.int64, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV)
+    prev, n = torch.tensor([[3]], dtype=torch.int32, device=DEV), torch.ones(1, dtype=torch.int32, device=DEV)
+    Sampler(SamplingParams(temp=0.0, repeat_penalty=2.0))(l, keys, steps, out, prev, n)
+    assert out.item() == 2                                                  # src/sampler.rs:378-383
+    rows, vocab = 8, 5000
+    base = logits_rows(rows, vocab, 6)
+    params = SamplingParams(temp=0.7, top_k=40, top_p=0.9, repeat_penalty=1.3, frequency_penalty=0.2,
+                            presence_penalty=0.1, seed=9)
+    windows = [[int(t) for t in np.random.default_rng(i).integers(0, vocab, size=20)] for i in range(rows)]
+    prev = torch.zeros(rows, 64, dtype=torch.int32)
+    for i, w in enumerate(windows):
+        w[0] = int(torch.argmax(base[i]))                  # penalise the favourite
+        prev[i, :20] = torch.tensor(w)
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    Sampler(params)(base.to(DEV).clone(), torch.arange(rows, dtype=torch.int64, device=DEV),
+                    torch.full((rows,), 3, dtype=torch.int32, device=DEV), out, prev.to(DEV),
+                    torch.full((rows,), 20, dtype=torch.int32, device=DEV))
+    want = [pq.sample(base[i].numpy(), 0.7, uniform(9, i, 3), 40, 0.9, 1.3, 0.2, 0.1, windows[i]) for i in range(rows)]
+    assert out.cpu().tolist() == want
