@@ -1,0 +1,253 @@
+"""Each part alone against the plain functions, and a model put together from other parts
+than the architecture's: a toy mixer with state of its own, defined here, is registered,
+built and stepped without a change to the framework's files; its model runs one block
+twice and lets a layer read another layer's cache."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen2 as pq
+from minfer_amd.cache import Cache, KVRequest, StateRequest
+from minfer_amd.engine.batch import StepContext
+from minfer_amd.parts import (BlockSpec, ModelSpec, PartSpec, RunEntry, Runtime, Mixer, make_part, register_mixer,
+                              FEED_FORWARDS, MIXERS, NORMS, POSITIONS)
+from minfer_amd.weights import TensorSpec
+from replays import batch_steps, compare, requests_for, run_steps, tail_steps, whole_steps
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def context(cache, slots, new, start):
+    """A StepContext built by hand for part-level tests."""
+    n_tok = sum(new)
+    seq = torch.repeat_interleave(torch.arange(len(slots)), torch.tensor(new)).int()
+    pos = torch.cat([torch.arange(s, s + n) for s, n in zip(start, new)]).int()
+    new_len = {s: st + n for s, st, n in zip(slots, start, new)}
+    cache.reserve(new_len)
+    max_len = max(new_len.values())
+    cols = (max_len + 63) // 64
+    tables = {id(g): torch.tensor(cache.page_rows(g, slots, cols), dtype=torch.int32, device=DEV) for g in cache.groups}
+    cu = torch.tensor([0] + list(np.cumsum(new)), dtype=torch.int32)
+    return StepContext(cache=cache, n_tokens=n_tok, n_seqs=len(slots), token_ids=torch.zeros(n_tok, dtype=torch.int32, device=DEV),
+                       positions=pos.to(DEV), seq_of_tok=seq.to(DEV), cu_seqlens=cu.to(DEV),
+                       start_pos=torch.tensor(start, dtype=torch.int32, device=DEV),
+                       slot_ids=torch.tensor(slots, dtype=torch.int32, device=DEV), logit_rows=None, page_tables=tables,
+                       max_len=max_len, max_new=max(new), all_decode=all(n == 1 for n in new), host_slots=list(slots),
+                       host_new=list(new), host_start=list(start), new_lengths=new_len)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_part(dtype):
+    rt = Runtime(dtype, DEV)
+    part = make_part(NORMS, PartSpec("rmsnorm", dict(size=200, eps=3e-6, weight="n.weight")), rt, "norm")
+    assert part.tensor_specs() == {"n.weight": TensorSpec((200,), init="ones")}
+    w, x = rnd(200, seed=1) + 1, rnd(9, 200, seed=2, scale=4.0)
+    part.load(lambda name: w.to(DEV).to(dtype))
+    ref = pq.rms_norm(x.double().numpy(), w.to(dtype).double().numpy(), 3e-6)
+    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    assert np.abs(part.forward(x.to(DEV)).float().cpu().numpy() - ref).max() < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_part_adds_into_the_residual(dtype):
+    rt = Runtime(dtype, DEV)
+    part = make_part(FEED_FORWARDS, PartSpec("swiglu", dict(hidden_size=72, intermediate_size=100, gate="g", up="u", down="d")), rt, "ffn")
+    assert sorted(part.tensor_specs()) == ["d.weight", "g.weight", "u.weight"]
+    w = {"g.weight": rnd(100, 72, seed=3, scale=0.2), "u.weight": rnd(100, 72, seed=4, scale=0.2),
+         "d.weight": rnd(72, 100, seed=5, scale=0.2)}
+    part.load(lambda name: w[name].to(DEV).to(dtype))
+    x, h = rnd(5, 72, seed=6), rnd(5, 72, seed=7)
+    hd = h.to(DEV).clone()
+    part.forward(x.to(DEV).to(dtype), hd, None)
+    wd = {k: v.to(dtype).double().numpy() for k, v in w.items()}
+    ref = h.double().numpy() + pq.swiglu_ffn(x.to(dtype).double().numpy(), wd["g.weight"], wd["u.weight"], wd["d.weight"])
+    assert np.abs(hd.cpu().numpy() - ref).max() < (1e-5 if dtype == torch.float32 else 3e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [None, 50])
+def test_attention_part_prompt_then_decode(dtype, window):
+    nh, nk, hd, hidden = 6, 2, 32, 80
+    rt = Runtime(dtype, DEV)
+    position = PartSpec("rope_neox", dict(head_dim=hd, theta=5000.0, max_positions=512))
+    spec = PartSpec("gqa_attention", dict(hidden_size=hidden, n_heads=nh, n_kv_heads=nk, head_dim=hd, scale=0.2,
+                                          window=window, qkv_bias=True, out_bias=False, position=position,
+                                          q="q", k="k", v="v", o="o"))
+    part = make_part(MIXERS, spec, rt, "mixer")
+    assert part.cache_request() == KVRequest(nk, hd, window)
+    specs = part.tensor_specs()
+    assert specs["k.weight"].shape == (nk * hd, hidden) and specs["o.weight"].shape == (hidden, nh * hd) and "o.bias" not in specs
+    w = {n: rnd(*s.shape, seed=10 + i, scale=0.15) for i, (n, s) in enumerate(sorted(specs.items()))}
+    part.load(lambda name: w[name].to(DEV).to(dtype))
+    cache = Cache({0: part.cache_request()}, 64 * 8, 4, dtype, DEV)
+    lens = [70, 130]
+    slots = [cache.alloc_slot() for _ in lens]
+    xs = [rnd(n, hidden, seed=20 + i) for i, n in enumerate(lens)]
+    wd = {k: v.to(dtype).double().numpy() for k, v in w.items()}
+
+    def plain(x, n):
+        x = x[:n].to(dtype).double().numpy()
+        pos = np.arange(n)
+        q = pq.rope_neox(pq.linear(x, wd["q.weight"], wd["q.bias"]), pos, nh, hd, 5000.0)
+        k = pq.rope_neox(pq.linear(x, wd["k.weight"], wd["k.bias"]), pos, nk, hd, 5000.0)
+        v = pq.linear(x, wd["v.weight"], wd["v.bias"])
+        return pq.linear(pq.gqa_attention(q, k, v, pos, pos, nh, nk, hd, 0.2, window), wd["o.weight"])
+    tol = 2e-5 if dtype == torch.float32 else 4e-2
+    # prompts (all but the last 3 tokens) in one step, then one token each
+    heads = [n - 3 for n in lens]
+    ctx = context(cache, slots, heads, [0, 0])
+    h = torch.zeros(sum(heads), hidden, device=DEV)
+    part.forward(torch.cat([x[:n] for x, n in zip(xs, heads)]).to(DEV).to(dtype), h, ctx, 0, True)
+    cache.commit(ctx.new_lengths)
+    ref = np.concatenate([plain(x, n) for x, n in zip(xs, heads)])
+    assert np.abs(h.cpu().numpy() - ref).max() < tol
+    for step in range(3):
+        at = [n + step for n in heads]
+        ctx = context(cache, slots, [1, 1], at)
+        h = torch.zeros(2, hidden, device=DEV)
+        part.forward(torch.stack([x[a] for x, a in zip(xs, at)]).to(DEV).to(dtype), h, ctx, 0, True)
+        cache.commit(ctx.new_lengths)
+        ref = np.stack([plain(x, a + 1)[a] for x, a in zip(xs, at)])
+        assert np.abs(h.cpu().numpy() - ref).max() < tol
+    cache.check_invariants()
+
+
+def test_unknown_part_and_unsupported_head_size():
+    rt = Runtime(torch.float32, DEV)
+    with pytest.raises(KeyError, match="unknown mixer 'nope'"):
+        make_part(MIXERS, PartSpec("nope", {}), rt, "mixer")
+    position = PartSpec("rope_neox", dict(head_dim=24, theta=1e4, max_positions=64))
+    with pytest.raises(ValueError, match="head_dim 24"):
+        make_part(MIXERS, PartSpec("gqa_attention", dict(hidden_size=48, n_heads=2, n_kv_heads=2, head_dim=24, scale=1.0,
+                                                         position=position, q="q", k="k", v="v", o="o")), rt, "mixer")
+
+
+# ------------------------------------------------------------------ a toy architecture
+DECAY = 0.75
+
+
+@register_mixer("toy_decay_state")
+class ToyDecayMixer(Mixer):
+    """state s (one vector per sequence): s <- DECAY * s + x_t; output W s.  Written with
+    torch operations on the device: a toy, not a kernel."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.hidden = int(spec.params["hidden_size"])
+        self.w = None
+
+    def tensor_specs(self):
+        return {"toy.weight": TensorSpec((self.hidden, self.hidden))}
+
+    def load(self, get):
+        self.w = get("toy.weight").float()
+
+    def cache_request(self):
+        return StateRequest((self.hidden,), torch.float32)
+
+    def forward(self, x, h, ctx, entry, writes_cache):
+        state = ctx.cache.state(entry)
+        off = 0
+        for slot, n in zip(ctx.host_slots, ctx.host_new):
+            s = state[slot]
+            for t in range(off, off + n):
+                s = DECAY * s + x[t].float()
+                h[t] += self.w @ s
+            state[slot] = s
+            off += n
+
+
+class ToyConfig:
+    """Layer 0: attention; layer 1: the toy mixer; run order 0, 1, 0 again (its own cache
+    entry), then a second attention-only block that reads entry 0 instead of writing."""
+
+    def __init__(self, raw):
+        self.raw = raw
+        self.hidden, self.vocab = raw["hidden_size"], raw["vocab_size"]
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(raw)
+
+    def to_dict(self):
+        return dict(self.raw)
+
+    def random_init_std(self, name):
+        return 0.08
+
+    def model_spec(self):
+        hid = self.hidden
+        norm = lambda n: PartSpec("rmsnorm", dict(size=hid, eps=1e-5, weight=n))
+        pos = PartSpec("rope_neox", dict(head_dim=16, theta=1e4, max_positions=256))
+        attn = PartSpec("gqa_attention", dict(hidden_size=hid, n_heads=3, n_kv_heads=1, head_dim=16, scale=0.25, window=None,
+                                              qkv_bias=False, out_bias=False, position=pos, q="a.q", k="a.k", v="a.v", o="a.o"))
+        ffn = PartSpec("swiglu", dict(hidden_size=hid, intermediate_size=40, gate="f.g", up="f.u", down="f.d"))
+        toy = PartSpec("toy_decay_state", dict(hidden_size=hid))
+        blocks = (BlockSpec("prenorm", "l0.", attn, ffn, norm("n1"), norm("n2")),
+                  BlockSpec("prenorm", "l1.", toy, ffn, norm("n1"), norm("n2")),
+                  BlockSpec("prenorm", "l2.", attn, ffn, norm("n1"), norm("n2")))
+        schedule = (RunEntry(0, 0), RunEntry(1, 1), RunEntry(0, 2), RunEntry(2, 0, writes_cache=False))
+        return ModelSpec(hidden_size=hid, vocab_size=self.vocab, embedding_name="emb", head_name=None,
+                         final_norm=norm("nf"), blocks=blocks, schedule=schedule, max_positions=256)
+
+
+class PlainToy:
+    """The toy model, whole sequences, numpy float64."""
+
+    def __init__(self, folder):
+        from safetensors.torch import load_file
+        self.w = {k: v.double().numpy() for k, v in load_file(folder + "/model.safetensors").items()}
+
+    def attn(self, p, x, pos, kv=None):
+        w = self.w
+        q = pq.rope_neox(pq.linear(x, w[p + "a.q.weight"]), pos, 3, 16, 1e4)
+        if kv is None:
+            kv = (pq.rope_neox(pq.linear(x, w[p + "a.k.weight"]), pos, 1, 16, 1e4), pq.linear(x, w[p + "a.v.weight"]))
+        return pq.linear(pq.gqa_attention(q, kv[0], kv[1], pos, pos, 3, 1, 16, 0.25), w[p + "a.o.weight"]), kv
+
+    def ffn(self, p, h):
+        w = self.w
+        return h + pq.swiglu_ffn(pq.rms_norm(h, w[p + "n2"], 1e-5), w[p + "f.g.weight"], w[p + "f.u.weight"], w[p + "f.d.weight"])
+
+    def forward(self, tokens):
+        w, pos = self.w, np.arange(len(tokens))
+        h = w["emb"][tokens]
+        a, kv0 = self.attn("l0.", pq.rms_norm(h, w["l0.n1"], 1e-5), pos)
+        h = self.ffn("l0.", h + a)
+        x, s, out = pq.rms_norm(h, w["l1.n1"], 1e-5), np.zeros(h.shape[1]), np.zeros_like(h)
+        for t in range(len(tokens)):
+            s = DECAY * s + x[t]
+            out[t] = w["l1.toy.weight"] @ s
+        h = self.ffn("l1.", h + out)
+        a, _ = self.attn("l0.", pq.rms_norm(h, w["l0.n1"], 1e-5), pos)
+        h = self.ffn("l0.", h + a)
+        a, _ = self.attn("l2.", pq.rms_norm(h, w["l2.n1"], 1e-5), pos, kv=kv0)     # reads layer 0's keys and values
+        h = self.ffn("l2.", h + a)
+        return pq.rms_norm(h, w["nf"], 1e-5) @ w["emb"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
+    from minfer_amd import Engine, load_model, register_architecture, write_random_model
+    register_architecture("ToyStateLM", ToyConfig)
+    cfg = ToyConfig(dict(architectures=["ToyStateLM"], hidden_size=48, vocab_size=300))
+    folder = write_random_model(str(tmp_path / "toy"), cfg, seed=3)
+    model = load_model(folder, dtype=dtype)
+    reqs = model.cache_requests()
+    assert isinstance(reqs[1], StateRequest) and reqs[0] == reqs[2] == KVRequest(1, 16, None)
+    assert "l2.a.k.weight" in model.expected_tensors()        # loaded though this entry only reads a cache
+    eng = Engine(model, max_tokens=64 * 6, max_seqs=3)
+    plain = PlainToy(folder)
+    requests = requests_for(300, (5, 70, 33, 9), seed=4)
+    ref = {r: plain.forward(t) for r, t in requests.items()}
+    ids = list(requests)
+    compare(run_steps(eng, whole_steps(requests)), ref, dtype, "toy whole")
+    compare(run_steps(eng, tail_steps(requests, tail=8)), ref, dtype, "toy one by one")
+    compare(run_steps(eng, batch_steps(requests, [ids[:3], ids[3:]])), ref, dtype, "toy batches")   # slots used again
