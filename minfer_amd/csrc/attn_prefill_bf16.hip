@@ -1,0 +1,228 @@
+// Causal grouped-query attention for many query tokens per sequence (prompts), bfloat16,
+// on the gfx950 matrix cores, reading keys and values from the paged cache.
+//
+// Semantics as the reference's attention (src/graph/cpu_backend.rs:437-494 of
+// yusiwen/minfer): a query at position p sees cache rows lo..p of its own sequence
+// (lo = 0, or p - window + 1), scores q.k * scale, softmax, weighted sum of v; query head h
+// reads kv head h / (nh / nk).  The softmax is the online form of the reference's CUDA
+// kernel (src/cuda_kernels.cu:673-790); scores, maxima, sums and the output accumulate in
+// 32-bit, probabilities are rounded to bfloat16 for the second product.
+//
+// A block (4 waves) owns 128 consecutive query tokens of one sequence and one query head;
+// each wave 32 of them.  Per cache page (64 keys): K goes to LDS as stored, V transposed.
+//   S^T[key][q] = K Q^T      32x32x16 MFMA, A = K rows from LDS, B = Q held in registers
+//   lane <-> query column, so the row statistics of the softmax are per-lane scalars
+//   O^T[d][q]  += V^T P^T    A = V^T from LDS, B = P^T, which is S^T's own register layout
+// The k index of the second product is permuted the same way on both operands (the sum
+// does not care), which is what lets P stay in registers.
+#include "common.h"
+
+namespace {
+
+constexpr int BQ = 128;             // query tokens per block
+constexpr int KT = MF_PAGE;         // keys per step: one page
+constexpr int VT_LD = KT + 4;       // LDS row stride of V^T in elements: 34 words, conflict-free 8-byte reads
+
+template <int NKS>                  // head_dim / 16
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const int* __restrict__ page_table, int pt_stride, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ start_pos, const int* __restrict__ tile_seq,
+    const int* __restrict__ tile_q0, bf16* __restrict__ out, int nh, int nk, float scale, int window) {
+  constexpr int HD = NKS * 16;
+  constexpr int NDT = (NKS + 1) / 2;          // 32-wide output tiles over head_dim
+  constexpr int HDP = NDT * 32;
+  constexpr int K_LD = HD + 8;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  bf16* Ks = reinterpret_cast<bf16*>(smem);              // [KT][K_LD]
+  bf16* Vt = Ks + KT * K_LD;                              // [HDP][VT_LD]
+  bf16* Os = reinterpret_cast<bf16*>(smem);              // [4][32][K_LD], after the last step
+
+  const int b = tile_seq[blockIdx.x], q0 = tile_q0[blockIdx.x];
+  const int h = blockIdx.y, hk = h / (nh / nk);
+  const int tok0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - tok0, start = start_pos[b];
+  const int* pt = page_table + (size_t)b * pt_stride;
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  const int ql = lane & 31, hf = lane >> 5;
+
+  // this lane's query
+  const int qi = q0 + wid * 32 + ql;                     // index among the sequence's new tokens
+  const bool q_ok = qi < n_new;
+  const int pq = start + qi;                             // its position
+  bf16x8 qf[NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    qf[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    if (q_ok)
+      qf[ks] = *reinterpret_cast<const bf16x8*>(q + ((size_t)(tok0 + qi) * nh + h) * HD + ks * 16 + hf * 8);
+  }
+  // positions this wave and this block need
+  const int wave_q_last = min(q0 + wid * 32 + 31, n_new - 1);
+  const int wave_p_hi = start + wave_q_last;
+  const int wave_p_lo = start + q0 + wid * 32;
+  const int blk_p_hi = start + min(q0 + BQ - 1, n_new - 1);
+  const int blk_p_lo = start + q0;
+  const int key_lo = window > 0 ? max(0, blk_p_lo - window + 1) : 0;
+
+  floatx16 oacc[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  if (HDP > HD) {   // rows of V^T beyond head_dim stay zero
+    for (int i = tid; i < (HDP - HD) * VT_LD; i += 256) Vt[HD * VT_LD + i] = (bf16)0.f;
+  }
+
+  for (int page_i = key_lo / KT; page_i <= blk_p_hi / KT; ++page_i) {
+    const int page = pt[page_i];
+    const bf16* kp = kc + ((size_t)page * nk + hk) * KT * HD;
+    const bf16* vp = vc + ((size_t)page * nk + hk) * KT * HD;
+    __syncthreads();                                     // the previous step's reads are done
+    // K as stored: thread -> (row, 8-element chunk), coalesced
+    for (int c = tid; c < KT * (HD / 8); c += 256) {
+      const int row = c / (HD / 8), ch = c % (HD / 8);
+      *reinterpret_cast<bf16x8*>(&Ks[row * K_LD + ch * 8]) =
+          *reinterpret_cast<const bf16x8*>(kp + (size_t)row * HD + ch * 8);
+    }
+    // V transposed: lane = key, so that the 2-byte LDS writes of a wave fall side by side.
+    // Rows after the block's last position were never written (a page is not cleared when
+    // it is taken): they are masked out of P, but 0 * garbage could still be NaN, so they
+    // enter as zeros.
+    const bool v_written = page_i * KT + lane <= blk_p_hi;
+    for (int c = wid; c < HD / 8; c += 4) {
+      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (v_written) v = *reinterpret_cast<const bf16x8*>(vp + (size_t)lane * HD + c * 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) Vt[(c * 8 + e) * VT_LD + lane] = v[e];
+    }
+    __syncthreads();
+    const int key0 = page_i * KT;
+    if (key0 > wave_p_hi) continue;                      // every key is later than every query here
+    if (window > 0 && key0 + KT - 1 <= wave_p_lo - window) continue;   // or left of every window
+
+    // S^T = K Q^T, two tiles of 32 keys
+    floatx16 s[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[kt][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&Ks[(kt * 32 + ql) * K_LD + ks * 16 + hf * 8]);
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s[kt], 0, 0, 0);
+      }
+    }
+    // mask, running maximum: reg r of tile kt is key key0 + 32 kt + 8 (r / 4) + 4 hf + r % 4
+    float m_new = m_run;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = key0 + kt * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
+        const bool vis = q_ok && key <= pq && (window <= 0 || key > pq - window);
+        s[kt][r] = vis ? s[kt][r] * scale : -INFINITY;
+        m_new = fmaxf(m_new, s[kt][r]);
+      }
+    m_new = fmaxf(m_new, __shfl_xor(m_new, 32, MF_WAVE));
+    const float corr = (m_new == -INFINITY) ? 1.f : __expf(m_run - m_new);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    float psum = 0.f;
+    bf16x8 pb[4];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float pe = __expf(s[kt][r] - m_use);       // exp(-inf) = 0 for masked keys
+        psum += pe;
+        pb[kt * 2 + (r >> 3)][r & 7] = (bf16)pe;
+      }
+    l_run = l_run * corr + psum;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[dt][r] *= corr;
+    // O^T += V^T P^T; operand element e of group kg is key 16 kg + 8 (e / 4) + 4 hf + e % 4
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int kg = 0; kg < 4; ++kg) {
+        const bf16* vrow = &Vt[(dt * 32 + ql) * VT_LD + kg * 16 + hf * 4];
+        const bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vrow);
+        const bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vrow + 8);
+        const bf16x8 a = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[kg], oacc[dt], 0, 0, 0);
+      }
+  }
+
+  // normalise; O^T regs: d = 32 dt + 8 (r / 4) + 4 hf + r % 4 for this lane's query
+  const float l_tot = l_run + __shfl_xor(l_run, 32, MF_WAVE);
+  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+  __syncthreads();                                       // all waves are done with Ks and Vt
+  bf16* ow = Os + (size_t)wid * 32 * K_LD;
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb) {
+      const int d = dt * 32 + rb * 8 + hf * 4;
+      if (d < HD) {
+        const bf16x4 v = {(bf16)(oacc[dt][rb * 4 + 0] * inv), (bf16)(oacc[dt][rb * 4 + 1] * inv),
+                          (bf16)(oacc[dt][rb * 4 + 2] * inv), (bf16)(oacc[dt][rb * 4 + 3] * inv)};
+        *reinterpret_cast<bf16x4*>(&ow[ql * K_LD + d]) = v;
+      }
+    }
+  __syncthreads();
+  // rows of this wave's 32 queries, 16 bytes per lane
+  for (int c = lane; c < 32 * (HD / 8); c += 64) {
+    const int row = c / (HD / 8), ch = c % (HD / 8);
+    const int qrow = q0 + wid * 32 + row;
+    if (qrow < n_new)
+      *reinterpret_cast<bf16x8*>(out + ((size_t)(tok0 + qrow) * nh + h) * HD + ch * 8) =
+          *reinterpret_cast<const bf16x8*>(&ow[row * K_LD + ch * 8]);
+  }
+}
+
+template <int NKS>
+int launch(const bf16* q, const bf16* kc, const bf16* vc, const int* page_table, int pt_stride,
+           const int* cu_seqlens, const int* start_pos, const int* tile_seq, const int* tile_q0, bf16* out,
+           int n_tiles, int nh, int nk, float scale, int window, hipStream_t stream) {
+  constexpr int HD = NKS * 16, HDP = ((NKS + 1) / 2) * 32, K_LD = HD + 8;
+  constexpr int kv_bytes = (KT * K_LD + HDP * VT_LD) * 2;
+  constexpr int o_bytes = 4 * 32 * K_LD * 2;
+  constexpr int smem = kv_bytes > o_bytes ? kv_bytes : o_bytes;
+  static bool configured = false;
+  auto kern = attn_prefill_kernel<NKS>;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    configured = true;
+  }
+  kern<<<dim3(n_tiles, nh), 256, smem, stream>>>(q, kc, vc, page_table, pt_stride, cu_seqlens, start_pos,
+                                                 tile_seq, tile_q0, out, nh, nk, scale, window);
+  return mf_launch_status();
+}
+
+}  // namespace
+
+// tile_seq[i], tile_q0[i]: sequence (index in the step's batch) and first new token of the
+// i-th block of 128 query tokens; the host lists them.
+MF_API int mf_attn_prefill_bf16(const void* q, const void* kc, const void* vc, const int* page_table,
+                                int pt_stride, const int* cu_seqlens, const int* start_pos,
+                                const int* tile_seq, const int* tile_q0, void* out, int n_tiles, int nh,
+                                int nk, int hd, float scale, int window, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (hd % 16 != 0 || hd < 16 || hd > 256 || nk <= 0 || nh % nk != 0) return (int)hipErrorInvalidValue;
+#define MF_CASE(E)                                                                                        \
+  case E:                                                                                                 \
+    return launch<E>((const bf16*)q, (const bf16*)kc, (const bf16*)vc, page_table, pt_stride, cu_seqlens, \
+                     start_pos, tile_seq, tile_q0, (bf16*)out, n_tiles, nh, nk, scale, window, stream);
+  switch (hd / 16) {
+    MF_CASE(1) MF_CASE(2) MF_CASE(3) MF_CASE(4) MF_CASE(5) MF_CASE(6) MF_CASE(7) MF_CASE(8)
+    MF_CASE(9) MF_CASE(10) MF_CASE(11) MF_CASE(12) MF_CASE(13) MF_CASE(14) MF_CASE(15) MF_CASE(16)
+  }
+#undef MF_CASE
+  return (int)hipErrorInvalidValue;
+}

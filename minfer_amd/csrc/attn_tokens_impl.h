@@ -9,10 +9,13 @@
 // all in 32-bit.
 //
 // Work split: a block owns (token, kv head, chunk of up to GC query heads, key split).
-// 16 lanes share one key row, each holding EPL = head_dim/16 consecutive elements; a block
-// of 4 waves walks 16 rows per step.  With several key splits each block writes an
-// unnormalised partial (acc, max, sum) and `attn_combine_kernel` merges them; the merge
-// order is fixed, so results are the same bits run to run.
+// 16 lanes share one key row, each holding EPL = head_dim/16 consecutive elements; each
+// group of 16 lanes takes R rows per step so that 2R independent loads are in flight and
+// the running maximum is updated once per R rows.  A block of 4 waves (16 groups) walks
+// 16 R rows per step, a divisor of the page size, so a step stays inside one page.  With
+// several key splits each block writes an unnormalised partial (acc, max, sum) and
+// `attn_combine_kernel` merges them; the merge order is fixed, so results are the same
+// bits run to run.
 //
 // Used for decode in both precisions and for whole prompts in the 32-bit path.
 #pragma once
@@ -21,6 +24,11 @@
 namespace attn_tokens {
 
 template <int EPL> struct Chunk { static constexpr int GC = (EPL <= 8) ? 8 : 4; };
+// rows per 16-lane group per step: 16 bytes of a row per lane -> 4 rows, more -> fewer
+template <typename T, int EPL> struct Rows {
+  static constexpr int BYTES = EPL * (int)sizeof(T);
+  static constexpr int R = BYTES <= 16 ? 4 : (BYTES <= 32 ? 2 : 1);
+};
 
 template <typename T> __device__ __forceinline__ float exp_for(float x);
 template <> __device__ __forceinline__ float exp_for<float>(float x) { return expf(x); }
@@ -35,6 +43,25 @@ __device__ __forceinline__ void load_elems(const T* __restrict__ p, float (&dst)
   for (int e = 0; e < EPL; ++e) dst[e] = to_f32(a[e]);
 }
 
+// the same elements kept in their storage type (for loads issued a step ahead)
+template <typename T, int EPL>
+__device__ __forceinline__ void load_raw(const T* __restrict__ p, T (&dst)[EPL]) {
+  constexpr int BYTES = EPL * (int)sizeof(T);
+  constexpr int ALIGN = (BYTES % 16 == 0) ? 16 : (BYTES % 8 == 0) ? 8 : (BYTES % 4 == 0) ? 4 : 2;
+  const T* a = (const T*)__builtin_assume_aligned(p, ALIGN);
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) dst[e] = a[e];
+}
+
+// sum over the 16 lanes of a row group, result in every lane (DPP, no LDS traffic)
+__device__ __forceinline__ float group16_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // lane ^ 1
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // lane ^ 2
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // mirror in 8
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // mirror in 16
+  return v;
+}
+
 template <typename T, int EPL>
 __global__ __launch_bounds__(256) void attn_tokens_kernel(
     const T* __restrict__ q, const T* __restrict__ kc, const T* __restrict__ vc,
@@ -42,6 +69,8 @@ __global__ __launch_bounds__(256) void attn_tokens_kernel(
     const int* __restrict__ seq_of_tok, T* __restrict__ out, float* __restrict__ part, int nh, int nk,
     float scale, int window, int n_splits, int split_len) {
   constexpr int GC = Chunk<EPL>::GC;
+  constexpr int R = Rows<T, EPL>::R;
+  constexpr int TILE = 16 * R;
   constexpr int HD = 16 * EPL;
   __shared__ float sm_acc[4][GC][HD];
   __shared__ float sm_ml[4][GC][2];
@@ -56,7 +85,7 @@ __global__ __launch_bounds__(256) void attn_tokens_kernel(
   const int split = blockIdx.z;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int sub = lane & 15, rg = lane >> 4;
-  const int R = w * 4 + rg;
+  const int gi = w * 4 + rg;
 
   const int p = positions[t];
   const int* pt = page_table + (size_t)seq_of_tok[t] * pt_stride;
@@ -74,32 +103,60 @@ __global__ __launch_bounds__(256) void attn_tokens_kernel(
     if (g < gcount) load_elems<T, EPL>(q + ((size_t)t * nh + h0 + g) * HD + sub * EPL, qr[g]);
   }
 
-  for (int tile = j_begin & ~15; tile < j_end; tile += 16) {
-    const int j = tile + R;
-    const bool valid = j >= j_begin && j < j_end;
-    const int jj = valid ? j : j_begin;
-    const int page = pt[jj / MF_PAGE];
-    const size_t row = (((size_t)page * nk + hk) * MF_PAGE + (jj % MF_PAGE)) * HD + sub * EPL;
-    float kr[EPL], vr[EPL];
-    load_elems<T, EPL>(kc + row, kr);
-    load_elems<T, EPL>(vc + row, vr);
+  // K and V of a step are loaded one step ahead, in their storage type
+  T kn[R][EPL], vn[R][EPL];
+  auto issue = [&](int tile) {
+    const int page = pt[tile / MF_PAGE];
+    const size_t base = (((size_t)page * nk + hk) * MF_PAGE + (tile % MF_PAGE)) * HD + sub * EPL;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int row = gi * R + r;                    // row inside the tile
+      const int j = tile + row;
+      const bool ok = j >= j_begin && j < j_end;
+      const int rr = ok ? row : (j_begin > tile ? j_begin - tile : 0);   // a row that exists
+      load_raw<T, EPL>(kc + base + (size_t)rr * HD, kn[r]);
+      load_raw<T, EPL>(vc + base + (size_t)rr * HD, vn[r]);
+    }
+  };
+  const int tile0 = j_begin & ~(TILE - 1);
+  if (tile0 < j_end) issue(tile0);
+  for (int tile = tile0; tile < j_end; tile += TILE) {
+    float kr[R][EPL], vr[R][EPL];
+    bool valid[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int j = tile + gi * R + r;
+      valid[r] = j >= j_begin && j < j_end;
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) { kr[r][e] = to_f32(kn[r][e]); vr[r][e] = to_f32(vn[r][e]); }
+    }
+    if (tile + TILE < j_end) issue(tile + TILE);
 #pragma unroll
     for (int g = 0; g < GC; ++g) {
       if (g < gcount) {
-        float s = 0.f;
+        float s[R];
+        float m_new = m[g];
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) s = fmaf(qr[g][e], kr[e], s);
-        s += __shfl_xor(s, 1, MF_WAVE);
-        s += __shfl_xor(s, 2, MF_WAVE);
-        s += __shfl_xor(s, 4, MF_WAVE);
-        s += __shfl_xor(s, 8, MF_WAVE);
-        s = valid ? s * scale : -INFINITY;
-        const float m_new = fmaxf(m[g], s);
+        for (int r = 0; r < R; ++r) {
+          float d = 0.f;
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) d = fmaf(qr[g][e], kr[r][e], d);
+          d = group16_sum(d);
+          s[r] = valid[r] ? d * scale : -INFINITY;
+          m_new = fmaxf(m_new, s[r]);
+        }
         const float corr = (m_new == -INFINITY) ? 1.f : exp_for<T>(m[g] - m_new);
-        const float pe = valid ? exp_for<T>(s - m_new) : 0.f;
-        l[g] = l[g] * corr + pe;
+        float lsum = l[g] * corr;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[g][e] = fmaf(pe, vr[e], acc[g][e] * corr);
+        for (int e = 0; e < EPL; ++e) acc[g][e] *= corr;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const float pe = valid[r] ? exp_for<T>(s[r] - m_new) : 0.f;
+          lsum += pe;
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) acc[g][e] = fmaf(pe, vr[r][e], acc[g][e]);
+        }
+        l[g] = lsum;
         m[g] = m_new;
       }
     }
@@ -171,26 +228,29 @@ __global__ __launch_bounds__(256) void attn_tokens_kernel(
   }
 }
 
-// out[t][h][:] = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M)
+// out[t][h][:] = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M); at most 64 splits.
+// One wave per (token, head): lane s weighs split s, then the lanes share the head's elements.
 template <typename T>
 __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restrict__ part,
                                                           T* __restrict__ out, int hd, int n_splits) {
+  __shared__ float wgt[64];
   const size_t th = blockIdx.x;   // t * nh + h
   const float* base = part + th * n_splits * (hd + 2);
-  float mm = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, base[(size_t)s * (hd + 2) + hd]);
+  const int lane = threadIdx.x;
+  const float ms = lane < n_splits ? base[(size_t)lane * (hd + 2) + hd] : -INFINITY;
+  const float ls = lane < n_splits ? base[(size_t)lane * (hd + 2) + hd + 1] : 0.f;
+  const float mm = wave_max(ms);
+  const float wv = (ms == -INFINITY) ? 0.f : exp_for<T>(ms - mm);
+  wgt[lane] = wv;
+  // fixed order: lane 0 adds the weighted sums one after another
+  __syncthreads();
   float L = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float ms = base[(size_t)s * (hd + 2) + hd];
-    L += base[(size_t)s * (hd + 2) + hd + 1] * (ms == -INFINITY ? 0.f : exp_for<T>(ms - mm));
-  }
+  for (int s = 0; s < n_splits; ++s) L += __shfl(ls, s, MF_WAVE) * wgt[s];
   const float inv = L > 0.f ? 1.0f / L : 0.f;
-  for (int d = threadIdx.x; d < hd; d += 64) {
+  for (int d = lane; d < hd; d += 64) {
     float a = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float ms = base[(size_t)s * (hd + 2) + hd];
-      a += base[(size_t)s * (hd + 2) + d] * (ms == -INFINITY ? 0.f : exp_for<T>(ms - mm));
-    }
+#pragma unroll 8
+    for (int s = 0; s < n_splits; ++s) a += base[(size_t)s * (hd + 2) + d] * wgt[s];
     out[th * hd + d] = from_f32<T>(a * inv);
   }
 }
@@ -218,8 +278,8 @@ int launch(const void* q, const void* kc, const void* vc, const int* page_table,
            const int* positions, const int* seq_of_tok, void* out, float* part, int n_tok, int nh,
            int nk, int hd, float scale, int window, int n_splits, int split_len, hipStream_t stream) {
   if (n_tok <= 0) return 0;
-  if (hd % 16 != 0 || hd < 16 || hd > 256 || nk <= 0 || nh % nk != 0 || n_splits < 1 ||
-      split_len < 16 || split_len % 16 != 0 || (n_splits > 1 && part == nullptr))
+  if (hd % 16 != 0 || hd < 16 || hd > 256 || nk <= 0 || nh % nk != 0 || n_splits < 1 || n_splits > 64 ||
+      split_len < MF_PAGE || split_len % MF_PAGE != 0 || (n_splits > 1 && part == nullptr))
     return (int)hipErrorInvalidValue;
 #define MF_CASE(E)                                                                                  \
   case E:                                                                                           \

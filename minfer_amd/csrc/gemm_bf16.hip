@@ -3,17 +3,21 @@
 // (out[t][o] = dot(W[o][:], x[t][:]) + b[o], src/graph/cpu_backend.rs:214-248 of
 // yusiwen/minfer; the reference's own matrix kernels are quantised and are not followed.)
 //
-// Two kernels:
+// Three kernels:
 //  * `tile_kernel`: many rows (prompts).  A BM x BN block tile per 256 threads, K walked
 //    in steps of 64 through double-buffered LDS, 32x32x16 MFMA, each wave a WM x WN tile.
-//  * `skinny_kernel`: at most 64 rows (decode).  The time is the weight stream: each wave
-//    owns 16 weight rows and reads them from HBM straight into MFMA operands (16x16x32),
-//    the few activation rows are staged in LDS and shared by the block, K may be split
-//    over blocks with a fixed-order reduction afterwards.
+//  * `skinny16_kernel`: at most 16 rows (decode).  The time is the weight stream: the waves
+//    of a block split K, each reads weights and activations straight into MFMA operands
+//    (16x16x32) and the partial sums meet in LDS.
+//  * `skinny_kernel`: 17 to 64 rows.  Each wave owns 16 weight rows and reads them from HBM
+//    straight into MFMA operands, the activation rows are staged in LDS and shared by the
+//    block, K may be split over blocks with a fixed-order reduction afterwards.
 // Both operands have K contiguous, which is exactly the MFMA operand layout (8 consecutive
 // k per lane), so nothing is transposed.
 //
 // Epilogues: 0 store fp32, 1 add into fp32 (residual stream), 2 store bf16.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace {
@@ -236,6 +240,94 @@ __global__ __launch_bounds__(256) void skinny_kernel(const bf16* __restrict__ A,
     }
 }
 
+// At most 16 rows: no LDS staging at all.  A block owns 16 NT weight rows; its NW waves split
+// K between them, each streaming its slice of the weights from HBM and the matching slice of
+// the few activation rows from L2 straight into MFMA operands, S steps (32 S k) of loads in
+// flight ahead of the matrix cores.  The waves' sums meet in LDS and wave 0 adds them in a
+// fixed order and runs the epilogue, so there is no second kernel and no atomics.
+template <int NW, int NT, int S>
+__global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restrict__ A, int lda,
+                                                           const bf16* __restrict__ W, int ldw,
+                                                           const float* __restrict__ bias,
+                                                           void* __restrict__ C, int ldc, int M, int N,
+                                                           int K, int k_per_wave, int epi, int vec_ok) {
+  __shared__ float red[NW][NT][64][4];
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int n_base = blockIdx.x * 16 * NT + (lane & 15);
+  const int m_row = lane & 15;
+  const int kq = (lane >> 4) * 8;
+  const int k_begin = wid * k_per_wave;
+  const int k_end = min(K, k_begin + k_per_wave);
+  floatx4 acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 wc[NT][S], ac[S], wn[NT][S], an[S];
+  if (k_begin < k_end) {
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        wc[j][s] = load8(W, ldw, n_base + 16 * j, N, k_begin + s * 32 + kq, k_end, vec_ok);
+      ac[s] = load8(A, lda, m_row, M, k_begin + s * 32 + kq, k_end, vec_ok);
+    }
+  }
+  for (int k0 = k_begin; k0 < k_end; k0 += S * 32) {
+    const bool more = k0 + S * 32 < k_end;
+    if (more) {
+#pragma unroll
+      for (int s = 0; s < S; ++s) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          wn[j][s] = load8(W, ldw, n_base + 16 * j, N, k0 + (S + s) * 32 + kq, k_end, vec_ok);
+        an[s] = load8(A, lda, m_row, M, k0 + (S + s) * 32 + kq, k_end, vec_ok);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ac[s], wc[j][s], acc[j], 0, 0, 0);
+    if (more) {
+#pragma unroll
+      for (int s = 0; s < S; ++s) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) wc[j][s] = wn[j][s];
+        ac[s] = an[s];
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wid][j][lane][r] = acc[j][r];
+  __syncthreads();
+  if (wid != 0) return;
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int n = n_base + 16 * j;
+    if (n >= N) continue;
+    const float b = bias ? bias[n] : 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = (lane >> 4) * 4 + r;      // D[m][n]: n = lane % 16, m = 4 (lane / 16) + r
+      if (m >= M) continue;
+      float v = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) v += red[w][j][lane][r];
+      store_out(C, ldc, m, n, v + b, epi);
+    }
+  }
+}
+
+template <int NW, int NT, int S>
+int launch_skinny16(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
+                    int M, int N, int K, int epi, int vec_ok, hipStream_t stream) {
+  const int k_per_wave = ((K + NW - 1) / NW + S * 32 - 1) / (S * 32) * (S * 32);
+  skinny16_kernel<NW, NT, S><<<(N + 16 * NT - 1) / (16 * NT), NW * 64, 0, stream>>>(
+      A, lda, W, ldw, bias, C, ldc, M, N, K, k_per_wave, epi, vec_ok);
+  return mf_launch_status();
+}
+
 __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restrict__ part,
                                                             const float* __restrict__ bias,
                                                             void* __restrict__ C, int ldc, int M, int N,
@@ -299,6 +391,20 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
                      ((uintptr_t)W % 16 == 0);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
+  static const int variant16 = getenv("MF_SKINNY16") ? atoi(getenv("MF_SKINNY16")) : 0;
+  if (M <= 16 && splits == 1) {
+    // few weight rows: more waves per block so that enough loads are in flight
+    // Measured at 3584..152064 weight rows: many rows -> 4 waves with two 16-row tiles each
+    // (less activation traffic per weight byte); a row count that would leave a short second
+    // round of 16-row blocks -> 8 waves with two tiles; otherwise 8 waves, one tile.
+    const int blocks16 = (N + 15) / 16;
+    int v = variant16;
+    if (v == 0) v = blocks16 >= 1024 ? 4 : (blocks16 > 256 && blocks16 <= 512 ? 3 : 1);
+    if (v == 1) return launch_skinny16<8, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    if (v == 2) return launch_skinny16<4, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    if (v == 3) return launch_skinny16<8, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    return launch_skinny16<4, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+  }
   switch ((M + 15) / 16) {
     case 1: return launch_skinny<1>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
     case 2: return launch_skinny<2>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);

@@ -35,6 +35,22 @@ class StepContext:
     host_new: List[int] = field(default_factory=list)
     host_start: List[int] = field(default_factory=list)
     new_lengths: Dict[int, int] = field(default_factory=dict)   # slot -> tokens held after the step
+    _memo: Dict = field(default_factory=dict, repr=False)
 
     def page_table(self, group) -> torch.Tensor:
         return self.page_tables[id(group)]
+
+    def query_tiles(self, block: int):
+        """(tile_seq, tile_q0) int32 on the device: the blocks of `block` consecutive new
+        tokens of each sequence, for kernels that give a workgroup to each.  Built from the
+        host's copy of the step once and kept."""
+        key = ("query_tiles", block)
+        if key not in self._memo:
+            seqs, starts = [], []
+            for b, n in enumerate(self.host_new):
+                for q0 in range(0, n, block):
+                    seqs.append(b)
+                    starts.append(q0)
+            both = torch.tensor([seqs, starts], dtype=torch.int32).to(self.token_ids.device)
+            self._memo[key] = (both[0], both[1])
+        return self._memo[key]

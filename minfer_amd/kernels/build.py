@@ -20,16 +20,18 @@ from typing import Dict, List
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 LIB_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "_lib")
 
-# library name -> source file; headers every library depends on
+# library name -> source file; HEADERS: what each includes (default: common.h)
 LIBRARIES: Dict[str, str] = {
     "elementwise": "elementwise.hip",
     "gemm_f32": "gemm_f32.hip",
     "gemm_bf16": "gemm_bf16.hip",
     "attn_tokens_f32": "attn_tokens_f32.hip",
     "attn_tokens_bf16": "attn_tokens_bf16.hip",
+    "attn_prefill_bf16": "attn_prefill_bf16.hip",
     "sampling": "sampling.hip",
 }
-HEADERS = ["common.h", "attn_tokens_impl.h"]
+HEADERS = {"attn_tokens_f32": ["common.h", "attn_tokens_impl.h"],
+           "attn_tokens_bf16": ["common.h", "attn_tokens_impl.h"]}
 
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-shared", "-std=c++17",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -51,7 +53,7 @@ def _hipcc() -> str:
 def source_hash(name: str) -> str:
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
-    for fname in [LIBRARIES[name]] + HEADERS:
+    for fname in [LIBRARIES[name]] + HEADERS.get(name, ["common.h"]):
         with open(os.path.join(CSRC, fname), "rb") as f:
             h.update(fname.encode())
             h.update(f.read())

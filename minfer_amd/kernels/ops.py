@@ -14,7 +14,8 @@ import torch
 from . import build
 
 PAGE = 64          # tokens per cache page (MF_PAGE in csrc/common.h)
-HAVE_PREFILL_ATTENTION = False
+HAVE_PREFILL_ATTENTION = True
+PREFILL_BLOCK = 128     # query tokens per workgroup of the prompt attention kernel
 EPI_F32, EPI_ACC_F32, EPI_BF16 = 0, 1, 2
 
 
@@ -225,6 +226,8 @@ def rope_kvwrite(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positi
 # ------------------------------------------------------------------ matrix products
 def skinny_plan(m: int, n: int, k: int, target_blocks: int = 1024) -> Tuple[int, int]:
     """(splits, k_per_split) of the decode product: enough blocks to fill the chip."""
+    if m <= 16:
+        return 1, (k + 255) // 256 * 256      # one kernel: K is split between the waves of a block
     n_blocks = (n + 63) // 64
     chunks = (k + 255) // 256
     splits = max(1, min(chunks, target_blocks // max(1, n_blocks)))
@@ -269,14 +272,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
 
 # ------------------------------------------------------------------ attention
 def split_plan(n_tok: int, n_kv_heads: int, group: int, head_dim: int, max_len: int,
-               target_blocks: int = 768) -> Tuple[int, int]:
+               target_blocks: int = 1024) -> Tuple[int, int]:
     """(n_splits, split_len) for the per-token attention: split the keys when tokens x kv
-    heads alone do not fill the chip.  Depends on the capacity, not on current lengths."""
+    heads alone do not fill the chip.  Depends on the capacity, not on current lengths;
+    split_len is a multiple of the page size and at least four pages; at most 64 splits."""
     gc = 8 if head_dim <= 128 else 4
     blocks = n_tok * n_kv_heads * ((group + gc - 1) // gc)
-    n_splits = max(1, min(target_blocks // max(1, blocks), (max_len + 255) // 256))
-    split_len = ((max_len + n_splits - 1) // n_splits + 15) // 16 * 16
-    split_len = max(split_len, 16)
+    n_splits = max(1, min(target_blocks // max(1, blocks), (max_len + 4 * PAGE - 1) // (4 * PAGE), 64))
+    split_len = ((max_len + n_splits - 1) // n_splits + PAGE - 1) // PAGE * PAGE
     return (max_len + split_len - 1) // split_len, split_len
 
 
@@ -308,6 +311,36 @@ def attn_tokens(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions),
         _ptr(seq_of_tok), _ptr(out), _ptr(part), n_tok, n_heads, n_kv_heads, head_dim, float(scale),
         int(window or 0), n_splits, split_len, _stream()), name)
+
+
+def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
+                 ctx, out: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
+                 window: int) -> None:
+    """bfloat16 attention of a step that brings several tokens per sequence: every new token
+    attends to its sequence's cache rows up to its own position (the step's keys are already
+    stored).  `ctx` gives the ragged layout (cu_seqlens, start_pos, the query blocks)."""
+    n_tok = ctx.n_tokens
+    _need(q, "attn_prefill.q", torch.bfloat16, (n_tok, n_heads * head_dim))
+    _need(out, "attn_prefill.out", torch.bfloat16, (n_tok, n_heads * head_dim))
+    for name, c in (("attn_prefill.kcache", kcache), ("attn_prefill.vcache", vcache)):
+        _need(c, name, torch.bfloat16)
+        if tuple(c.shape[1:]) != (n_kv_heads, PAGE, head_dim):
+            raise KernelError(f"{name}: shape {tuple(c.shape)}, expected [pages, {n_kv_heads}, {PAGE}, {head_dim}]")
+    _need(page_table, "attn_prefill.page_table", torch.int32)
+    _need(ctx.cu_seqlens, "attn_prefill.cu_seqlens", torch.int32, (ctx.n_seqs + 1,))
+    _need(ctx.start_pos, "attn_prefill.start_pos", torch.int32, (ctx.n_seqs,))
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise KernelError(f"attention: head_dim {head_dim} is not a multiple of 16 in [16, 256]")
+    if n_heads % n_kv_heads:
+        raise KernelError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
+    if ctx.max_len > page_table.shape[1] * PAGE or page_table.shape[0] != ctx.n_seqs:
+        raise KernelError(f"attention: page table {tuple(page_table.shape)} does not cover "
+                          f"{ctx.n_seqs} sequences of up to {ctx.max_len} positions")
+    tile_seq, tile_q0 = ctx.query_tiles(PREFILL_BLOCK)
+    _check(_fn("attn_prefill_bf16", "mf_attn_prefill_bf16")(
+        _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(ctx.cu_seqlens),
+        _ptr(ctx.start_pos), _ptr(tile_seq), _ptr(tile_q0), _ptr(out), tile_seq.numel(), n_heads,
+        n_kv_heads, head_dim, float(scale), int(window or 0), _stream()), "attn_prefill_bf16")
 
 
 # ------------------------------------------------------------------ sampling

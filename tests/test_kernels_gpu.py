@@ -222,6 +222,17 @@ def test_gemm_reference_vector(ops):
     assert ob.cpu().tolist() == [[1.5, 3.0, 9.25]]
 
 
+def poison_unwritten(kc, vc, table, lengths):
+    """Rows of a page after its sequence's last token were never written: a page is not
+    cleared when it is taken, so they may hold anything.  NaN makes a kernel that touches
+    them show."""
+    for b, l in enumerate(lengths):
+        if l % 64:
+            page = int(table[b, l // 64])
+            kc[page, :, l % 64:] = float("nan")
+            vc[page, :, l % 64:] = float("nan")
+
+
 def build_attention_case(nh, nk, hd, lengths, dtype, seed, n_pages_extra=3):
     """Sequences of the given lengths in shuffled pages; one query token per sequence at its
     last position, plus a few mid-sequence queries."""
@@ -236,6 +247,7 @@ def build_attention_case(nh, nk, hd, lengths, dtype, seed, n_pages_extra=3):
             table[b, c] = perm[nxt]
             nxt += 1
     kc, vc = make_cache(n_pages, nk, hd, dtype, seed)
+    poison_unwritten(kc, vc, table, lengths)
     pos, seq = [], []
     for b, l in enumerate(lengths):
         for p in sorted({l - 1, l // 2, 0}):
@@ -302,3 +314,88 @@ def test_attention_one_key_gives_v_and_far_key_is_found(ops):
                         nh, nk, hd, 1.0, window, 1280)
         hit = torch.allclose(out.cpu().view(nh, hd)[0], vc[far // 64, 0, far % 64], atol=1e-4)
         assert hit == seen
+
+
+def prefill_case(nh, nk, hd, new, start, seed):
+    """Sequences that already hold start[b] tokens and bring new[b] more; caches filled for
+    all of them (as the rotation kernel would have left them)."""
+    from minfer_amd.engine.batch import StepContext
+    rng = np.random.default_rng(seed)
+    lengths = [s + n for s, n in zip(start, new)]
+    n_cols = max((l + 63) // 64 for l in lengths)
+    n_pages = sum((l + 63) // 64 for l in lengths) + 2
+    perm = rng.permutation(n_pages)
+    table = -np.ones((len(new), n_cols), dtype=np.int32)
+    nxt = 0
+    for b, l in enumerate(lengths):
+        for c in range((l + 63) // 64):
+            table[b, c] = perm[nxt]
+            nxt += 1
+    kc, vc = make_cache(n_pages, nk, hd, torch.bfloat16, seed)
+    poison_unwritten(kc, vc, table, lengths)
+    pos = torch.cat([torch.arange(s, s + n) for s, n in zip(start, new)]).int()
+    seq = torch.repeat_interleave(torch.arange(len(new)), torch.tensor(new)).int()
+    n_tok = int(sum(new))
+    q = rnd((n_tok, nh * hd), torch.bfloat16, seed + 5)
+    cu = torch.tensor([0] + list(np.cumsum(new)), dtype=torch.int32)
+    table = torch.from_numpy(table)
+
+    def ctx_on(dev):
+        return StepContext(cache=None, n_tokens=n_tok, n_seqs=len(new), token_ids=torch.zeros(n_tok, dtype=torch.int32, device=dev),
+                           positions=pos.to(dev), seq_of_tok=seq.to(dev), cu_seqlens=cu.to(dev),
+                           start_pos=torch.tensor(start, dtype=torch.int32, device=dev),
+                           slot_ids=torch.zeros(len(new), dtype=torch.int32, device=dev), logit_rows=None,
+                           page_tables={}, max_len=max(lengths), max_new=max(new), all_decode=False,
+                           host_slots=list(range(len(new))), host_new=list(new), host_start=list(start))
+    return q, kc, vc, table, ctx_on
+
+
+@pytest.mark.parametrize("nh,nk,hd,window", [(4, 2, 16, 0), (4, 1, 32, 0), (9, 3, 48, 0), (28, 4, 128, 0),
+                                             (6, 6, 64, 0), (10, 2, 80, 0), (4, 2, 256, 0), (4, 2, 64, 40),
+                                             (7, 1, 128, 200), (4, 4, 112, 0)])
+def test_attn_prefill(ops, nh, nk, hd, window):
+    # new tokens per sequence straddle the 32/128 tiles and the 64-key pages; two sequences
+    # continue from a cache that already holds tokens
+    new = [1, 5, 31, 33, 64, 65, 127, 129, 300, 70]
+    start = [0, 0, 0, 0, 0, 0, 0, 0, 0, 150]
+    q, kc, vc, table, ctx_on = prefill_case(nh, nk, hd, new, start, 21)
+    scale = 1.0 / math.sqrt(hd)
+    ref = torch.empty(q.shape, dtype=torch.float64)
+    plain_ops.attn_prefill(q, kc, vc, table, ctx_on("cpu"), ref, nh, nk, hd, scale, window)
+    out = torch.empty(q.shape, dtype=torch.bfloat16, device=DEV)
+    ops.attn_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), ctx_on(DEV), out, nh, nk, hd, scale, window)
+    close(out, ref, 1.5e-2, 1.5e-2)
+    again = torch.empty(q.shape, dtype=torch.bfloat16, device=DEV)
+    ops.attn_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), ctx_on(DEV), again, nh, nk, hd, scale, window)
+    assert torch.equal(out, again), "two runs differ"
+    # the per-token kernel gives the same answer on the same step
+    tok = torch.empty(q.shape, dtype=torch.bfloat16, device=DEV)
+    c = ctx_on(DEV)
+    ops.attn_tokens(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), c.positions, c.seq_of_tok, tok, nh, nk, hd,
+                    scale, window, c.max_len)
+    close(out, tok.double(), 2e-2, 2e-2)
+
+
+def test_attn_prefill_far_key_and_window_edge(ops):
+    """One key's score is made to stand out for one query: the output is that key's V row
+    when the key is visible (anywhere in a long prompt, across pages), and is not when the
+    key lies just outside the window or after the query."""
+    nh, nk, hd = 2, 1, 64
+    n = 700
+    q, kc, vc, table, ctx_on = prefill_case(nh, nk, hd, [n], [0], 22)
+    kc = kc * 0.05
+    qi, far = 650, 3
+    page, row = int(table[0, far // 64]), far % 64
+    kc[page, 0, row] = q[qi, :hd] * 4.0
+    vrow = vc[page, 0, row].float()
+    for window, seen in ((0, True), (qi - far + 1, True), (qi - far, False)):
+        out = torch.empty(q.shape, dtype=torch.bfloat16, device=DEV)
+        ops.attn_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), ctx_on(DEV), out, nh, nk, hd, 1.0, window)
+        hit = torch.allclose(out[qi, :hd].float().cpu(), vrow, atol=3e-2)
+        assert hit == seen, (window, seen)
+    # a query before the key never sees it
+    out = torch.empty(q.shape, dtype=torch.bfloat16, device=DEV)
+    q2 = q.clone()
+    q2[2] = q[qi]
+    ops.attn_prefill(q2.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), ctx_on(DEV), out, nh, nk, hd, 1.0, 0)
+    assert not torch.allclose(out[2, :hd].float().cpu(), vrow, atol=3e-2)
