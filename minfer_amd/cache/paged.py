@@ -80,7 +80,9 @@ class PagePool:
 class KVGroup:
     """Storage and page bookkeeping of the entries that share one KVRequest."""
 
-    def __init__(self, request: KVRequest, entries: List[int], n_pages: int, dtype, device):
+    def __init__(self, request: KVRequest, entries: List[int], n_pages: int, dtype, device,
+                 poison: bool = False):
+        self.poison = poison
         self.request = request
         self.entries = list(entries)
         self.index_of = {e: i for i, e in enumerate(self.entries)}
@@ -88,7 +90,19 @@ class KVGroup:
         shape = (len(entries), n_pages, request.n_kv_heads, PAGE, request.head_dim)
         self.k = torch.empty(shape, dtype=dtype, device=device)
         self.v = torch.empty(shape, dtype=dtype, device=device)
+        if poison:
+            self.k.fill_(float("nan"))
+            self.v.fill_(float("nan"))
         self.pages: Dict[int, List[int]] = {}      # slot -> page id per logical page, -1 = given back
+
+    def _give(self, pages: List[int]) -> None:
+        """Back to the pool.  With `poison` (tests) the pages are overwritten with NaN, so that
+        a read of a row its sequence never wrote shows at once."""
+        self.pool.give(pages)
+        if self.poison and pages:
+            idx = torch.tensor(pages, dtype=torch.long, device=self.k.device)
+            self.k[:, idx] = float("nan")
+            self.v[:, idx] = float("nan")
 
     def first_needed_page(self, length: int) -> int:
         """Lowest logical page a query at position >= length can still read."""
@@ -108,7 +122,7 @@ class KVGroup:
         keep = (length + PAGE - 1) // PAGE
         tail = [p for p in self.pages[slot][keep:] if p >= 0]
         del self.pages[slot][keep:]
-        self.pool.give(tail)
+        self._give(tail)
 
     def drop_left_of_window(self, slot: int, length: int) -> None:
         first = self.first_needed_page(length)
@@ -116,18 +130,20 @@ class KVGroup:
         gone = [p for p in row[:first] if p >= 0]
         for i in range(min(first, len(row))):
             row[i] = -1
-        self.pool.give(gone)
+        self._give(gone)
 
     def release(self, slot: int) -> None:
-        self.pool.give([p for p in self.pages.pop(slot) if p >= 0])
+        self._give([p for p in self.pages.pop(slot) if p >= 0])
 
 
 class Cache:
     """`requests[entry]` is a KVRequest, a StateRequest or None, one per cache entry of the
     model's run order.  `max_tokens` is the most tokens all live sequences hold together,
-    each rounded up to a multiple of 64; `max_seqs` bounds the live sequences."""
+    each rounded up to a multiple of 64; `max_seqs` bounds the live sequences.  `poison`
+    (tests) fills pages with NaN when they are created and whenever they are given back."""
 
-    def __init__(self, requests: Dict[int, object], max_tokens: int, max_seqs: int, dtype, device):
+    def __init__(self, requests: Dict[int, object], max_tokens: int, max_seqs: int, dtype, device,
+                 poison: bool = False):
         if max_tokens < 1 or max_seqs < 1:
             raise CacheError("cache needs room for at least one token and one sequence")
         self.dtype, self.device = dtype, device
@@ -142,7 +158,7 @@ class Cache:
                 self.state_requests[entry] = req
             elif req is not None:
                 raise CacheError(f"cache entry {entry}: unknown request {req!r}")
-        self.groups: List[KVGroup] = [KVGroup(r, es, self.n_pages, dtype, device)
+        self.groups: List[KVGroup] = [KVGroup(r, es, self.n_pages, dtype, device, poison)
                                       for r, es in by_request.items()]
         self.group_of: Dict[int, KVGroup] = {e: g for g in self.groups for e in g.entries}
         self.states: Dict[int, torch.Tensor] = {

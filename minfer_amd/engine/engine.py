@@ -27,14 +27,16 @@ class StepError(ValueError):
 
 
 class Engine:
-    def __init__(self, model: DecoderModel, max_tokens: int, max_seqs: Optional[int] = None):
+    def __init__(self, model: DecoderModel, max_tokens: int, max_seqs: Optional[int] = None,
+                 poison_cache: bool = False):
         if not model.loaded:
             raise RuntimeError("Engine needs a model with weights")
         self.model = model
         self.device = model.rt.device
         n_pages = (max_tokens + PAGE - 1) // PAGE
         self.max_seqs = int(max_seqs) if max_seqs else max(1, min(n_pages, 1024))
-        self.cache = Cache(model.cache_requests(), max_tokens, self.max_seqs, model.rt.dtype, self.device)
+        self.cache = Cache(model.cache_requests(), max_tokens, self.max_seqs, model.rt.dtype, self.device,
+                           poison=poison_cache)
         self.vocab_size = model.spec.vocab_size
         self.max_positions = model.spec.max_positions
         self._sessions = {}

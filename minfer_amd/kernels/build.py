@@ -60,8 +60,30 @@ def source_hash(name: str) -> str:
     return h.hexdigest()
 
 
+def lib_dir() -> str:
+    """Beside the package; a per-user folder under the temporary directory when the package
+    folder cannot be written (a read-only checkout)."""
+    global LIB_DIR
+    try:
+        os.makedirs(LIB_DIR, exist_ok=True)
+        if os.access(LIB_DIR, os.W_OK):
+            return LIB_DIR
+    except OSError:
+        pass
+    import tempfile
+    alt = os.path.join(tempfile.gettempdir(), f"minfer_amd_lib_{os.getuid()}")
+    os.makedirs(alt, exist_ok=True)
+    have = os.path.join(os.path.dirname(CSRC), "_lib")
+    if os.path.isdir(have):           # built files that came with the checkout still count
+        for f in os.listdir(have):
+            if not os.path.exists(os.path.join(alt, f)):
+                shutil.copy(os.path.join(have, f), os.path.join(alt, f))
+    LIB_DIR = alt
+    return LIB_DIR
+
+
 def lib_path(name: str) -> str:
-    return os.path.join(LIB_DIR, f"libmf_{name}.so")
+    return os.path.join(lib_dir(), f"libmf_{name}.so")
 
 
 def is_current(name: str) -> bool:
@@ -78,7 +100,6 @@ def _say(msg: str) -> None:
 
 def compile_library(name: str, quiet: bool = False) -> str:
     """Compiles one library; prints a line at start and every 15 s while hipcc runs."""
-    os.makedirs(LIB_DIR, exist_ok=True)
     so = lib_path(name)
     tmp = f"{so}.{os.getpid()}.tmp"
     cmd = [_hipcc()] + HIPCC_FLAGS + ["-I", CSRC, os.path.join(CSRC, LIBRARIES[name]), "-o", tmp]
@@ -87,7 +108,7 @@ def compile_library(name: str, quiet: bool = False) -> str:
     t0 = time.time()
     env = dict(os.environ)
     env.setdefault("TMPDIR", "/tmp")
-    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env, cwd=LIB_DIR)
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env, cwd=lib_dir())
     done = threading.Event()
 
     def ticker():

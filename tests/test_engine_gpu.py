@@ -25,7 +25,7 @@ def plains(folders):
 
 def engine_for(folder, dtype, max_tokens=2048):
     from minfer_amd import Engine, load_model
-    return Engine(load_model(folder, dtype=dtype, device="cuda:0"), max_tokens=max_tokens)
+    return Engine(load_model(folder, dtype=dtype, device="cuda:0"), max_tokens=max_tokens, poison_cache=True)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -99,7 +99,7 @@ def test_first_tokens_of_a_sequence(folders, dtype):
     """Prompts of one token, the first decoded token, a prompt that ends on a page edge."""
     from minfer_amd import Engine, load_model
     plain = pq.PlainQwen2.from_folder(folders["C"])
-    eng = Engine(load_model(folders["C"], dtype=dtype), max_tokens=64 * 6)
+    eng = Engine(load_model(folders["C"], dtype=dtype), max_tokens=64 * 6, poison_cache=True)
     reqs = requests_for(777, (1, 2, 64, 65), seed=9)
     ref = plain_logits(plain, reqs)
     steps = []

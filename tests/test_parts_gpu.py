@@ -86,7 +86,7 @@ def test_attention_part_prompt_then_decode(dtype, window):
     assert specs["k.weight"].shape == (nk * hd, hidden) and specs["o.weight"].shape == (hidden, nh * hd) and "o.bias" not in specs
     w = {n: rnd(*s.shape, seed=10 + i, scale=0.15) for i, (n, s) in enumerate(sorted(specs.items()))}
     part.load(lambda name: w[name].to(DEV).to(dtype))
-    cache = Cache({0: part.cache_request()}, 64 * 8, 4, dtype, DEV)
+    cache = Cache({0: part.cache_request()}, 64 * 8, 4, dtype, DEV, poison=True)
     lens = [70, 130]
     slots = [cache.alloc_slot() for _ in lens]
     xs = [rnd(n, hidden, seed=20 + i) for i, n in enumerate(lens)]
@@ -243,7 +243,7 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
     reqs = model.cache_requests()
     assert isinstance(reqs[1], StateRequest) and reqs[0] == reqs[2] == KVRequest(1, 16, None)
     assert "l2.a.k.weight" in model.expected_tensors()        # loaded though this entry only reads a cache
-    eng = Engine(model, max_tokens=64 * 6, max_seqs=3)
+    eng = Engine(model, max_tokens=64 * 6, max_seqs=3, poison_cache=True)
     plain = PlainToy(folder)
     requests = requests_for(300, (5, 70, 33, 9), seed=4)
     ref = {r: plain.forward(t) for r, t in requests.items()}
