@@ -15,14 +15,20 @@
 // Both operands have K contiguous, which is exactly the MFMA operand layout (8 consecutive
 // k per lane), so nothing is transposed.
 //
-// Epilogues: 0 store fp32, 1 add into fp32 (residual stream), 2 store bf16.
+// Epilogues: 0 store fp32, 1 add into fp32 (residual stream), 2 store bf16, 3 SwiGLU.
+// SwiGLU (y = silu(g) * u, silu(z) = z / (1 + exp(-z)), src/graph/cpu_backend.rs:323-329):
+// the weight rows come interleaved in groups of 64, 32 gate rows then the 32 up rows of the
+// same outputs (the last group padded with zero rows), so a gate column and its up column
+// are 32 apart inside one wave's tile; the epilogue writes bfloat16 y[M][ldc], ldc = number
+// of outputs, straight from the 32-bit accumulators and the [M][2 nf] intermediate is never
+// stored.
 #include <stdlib.h>
 
 #include "common.h"
 
 namespace {
 
-enum { EPI_F32 = 0, EPI_ACC_F32 = 1, EPI_BF16 = 2 };
+enum { EPI_F32 = 0, EPI_ACC_F32 = 1, EPI_BF16 = 2, EPI_SWIGLU = 3 };
 
 __device__ __forceinline__ void store_out(void* C, int ldc, int m, int n, float v, int epi) {
   if (epi == EPI_BF16) {
@@ -33,33 +39,42 @@ __device__ __forceinline__ void store_out(void* C, int ldc, int m, int n, float 
   }
 }
 
-// 8 consecutive k of one row, zero outside the matrix; vector load when aligned.
-__device__ __forceinline__ bf16x8 load8(const bf16* __restrict__ base, int ld, int row, int rows, int k,
-                                        int K, bool vec_ok) {
-  bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-  if (row < rows && k < K) {
+__device__ __forceinline__ float swiglu_f(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
+// 8 consecutive k of one row, zero at and beyond k_end.  Rows are clamped by the caller to a
+// row that exists (results of such rows are never stored), so the fast form has no branch:
+// VEC needs 16-byte aligned rows and K a multiple of 8, so a chunk is inside or outside whole.
+template <bool VEC>
+__device__ __forceinline__ bf16x8 load8(const bf16* __restrict__ base, int ld, int row, int k, int k_end) {
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (VEC) {
+    const int kk = min(k, k_end - 8);
+    const bf16x8 v = *reinterpret_cast<const bf16x8*>(base + (size_t)row * ld + kk);
+    return k + 8 <= k_end ? v : zero;
+  } else {
+    bf16x8 v = zero;
     const bf16* p = base + (size_t)row * ld + k;
-    if (vec_ok && k + 8 <= K) {
-      v = *reinterpret_cast<const bf16x8*>(p);
-    } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        if (k + e < K) v[e] = p[e];
-    }
+    for (int e = 0; e < 8; ++e)
+      if (k + e < k_end) v[e] = p[e];
+    return v;
   }
-  return v;
+}
+
+// 8 consecutive k with no guard at all: the caller knows the chunk lies inside the row.
+__device__ __forceinline__ bf16x8 load8_inside(const bf16* __restrict__ base, int ld, int row, int k) {
+  return *reinterpret_cast<const bf16x8*>(base + (size_t)row * ld + k);
 }
 
 // ------------------------------------------------------------------ tiled kernel
 constexpr int BK = 64;
 constexpr int LDS_LD = BK + 8;   // row stride in elements: 144 bytes, conflict-free b128 reads
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, bool VEC>
 __global__ __launch_bounds__(256) void tile_kernel(const bf16* __restrict__ A, int lda,
                                                    const bf16* __restrict__ W, int ldw,
                                                    const float* __restrict__ bias, void* __restrict__ C,
-                                                   int ldc, int M, int N, int K, int epi, int vec_ok,
-                                                   int tiles_m) {
+                                                   int ldc, int M, int N, int K, int epi, int tiles_m) {
   static_assert((BM / WM) * (BN / WN) == 4, "four waves per block");
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int PA = BM / 32, PW = BN / 32;   // load passes: 32 rows x 64 k per pass
@@ -84,11 +99,29 @@ __global__ __launch_bounds__(256) void tile_kernel(const bf16* __restrict__ A, i
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   bf16x8 ra[PA], rw[PW];
+  int arow[PA], wrow[PW];                       // rows past the matrix read its last row
+#pragma unroll
+  for (int p = 0; p < PA; ++p) arow[p] = min(m0 + p * 32 + lrow, M - 1);
+#pragma unroll
+  for (int p = 0; p < PW; ++p) wrow[p] = min(n0 + p * 32 + lrow, N - 1);
   const int nkt = (K + BK - 1) / BK;
+  const int nkt_inside = VEC ? K / BK : 0;      // k tiles that need no guard (the loop's fast form:
+                                                // a guard's select would wait for the load at once)
+  auto load_tile = [&](int kt) {
+    const int k = kt * BK + lk;
+    if (kt < nkt_inside) {
 #pragma unroll
-  for (int p = 0; p < PA; ++p) ra[p] = load8(A, lda, m0 + p * 32 + lrow, M, lk, K, vec_ok);
+      for (int p = 0; p < PA; ++p) ra[p] = load8_inside(A, lda, arow[p], k);
 #pragma unroll
-  for (int p = 0; p < PW; ++p) rw[p] = load8(W, ldw, n0 + p * 32 + lrow, N, lk, K, vec_ok);
+      for (int p = 0; p < PW; ++p) rw[p] = load8_inside(W, ldw, wrow[p], k);
+    } else {
+#pragma unroll
+      for (int p = 0; p < PA; ++p) ra[p] = load8<VEC>(A, lda, arow[p], k, K);
+#pragma unroll
+      for (int p = 0; p < PW; ++p) rw[p] = load8<VEC>(W, ldw, wrow[p], k, K);
+    }
+  };
+  load_tile(0);
 #pragma unroll
   for (int p = 0; p < PA; ++p)
     *reinterpret_cast<bf16x8*>(&As[(p * 32 + lrow) * LDS_LD + lk]) = ra[p];
@@ -100,13 +133,7 @@ __global__ __launch_bounds__(256) void tile_kernel(const bf16* __restrict__ A, i
   for (int kt = 0; kt < nkt; ++kt) {
     const int cur = kt & 1;
     const bool more = kt + 1 < nkt;
-    if (more) {
-      const int k = (kt + 1) * BK + lk;
-#pragma unroll
-      for (int p = 0; p < PA; ++p) ra[p] = load8(A, lda, m0 + p * 32 + lrow, M, k, K, vec_ok);
-#pragma unroll
-      for (int p = 0; p < PW; ++p) rw[p] = load8(W, ldw, n0 + p * 32 + lrow, N, k, K, vec_ok);
-    }
+    if (more) load_tile(kt + 1);
     const bf16* as = As + cur * BM * LDS_LD;
     const bf16* ws = Ws + cur * BN * LDS_LD;
 #pragma unroll
@@ -138,6 +165,24 @@ __global__ __launch_bounds__(256) void tile_kernel(const bf16* __restrict__ A, i
   }
 
   // D[m][n]: lane holds n = lane % 32, m = 8 (r / 4) + 4 (lane / 32) + r % 4
+  if (epi == EPI_SWIGLU) {
+    if constexpr (TN % 2 == 0) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; j += 2) {
+          const int ng = n0 + wn + j * 32 + fr;            // gate column; its up column is ng + 32
+          const int col = (ng >> 6) * 32 + (ng & 63);
+          if (col >= ldc) continue;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int m = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            if (m < M) ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(acc[i][j][r], acc[i][j + 1][r]);
+          }
+        }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -153,12 +198,12 @@ __global__ __launch_bounds__(256) void tile_kernel(const bf16* __restrict__ A, i
     }
 }
 
-template <int BM, int BN, int WM, int WN>
-int launch_tile(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
-                int M, int N, int K, int epi, int vec_ok, hipStream_t stream) {
+template <int BM, int BN, int WM, int WN, bool VEC>
+int launch_tile_v(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
+                  int M, int N, int K, int epi, hipStream_t stream) {
   constexpr int smem = 2 * (BM + BN) * LDS_LD * (int)sizeof(bf16);
   static bool configured = false;
-  auto kern = tile_kernel<BM, BN, WM, WN>;
+  auto kern = tile_kernel<BM, BN, WM, WN, VEC>;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -166,9 +211,15 @@ int launch_tile(const bf16* A, int lda, const bf16* W, int ldw, const float* bia
     configured = true;
   }
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  kern<<<tiles_m * tiles_n, 256, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, vec_ok,
-                                                 tiles_m);
+  kern<<<tiles_m * tiles_n, 256, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, tiles_m);
   return mf_launch_status();
+}
+
+template <int BM, int BN, int WM, int WN>
+int launch_tile(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
+                int M, int N, int K, int epi, int vec_ok, hipStream_t stream) {
+  return vec_ok ? launch_tile_v<BM, BN, WM, WN, true>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, stream)
+                : launch_tile_v<BM, BN, WM, WN, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, stream);
 }
 
 // ------------------------------------------------------------------ skinny kernel
@@ -176,15 +227,16 @@ constexpr int KC = 256;          // k per staging step
 constexpr int SK_LD = KC + 8;    // LDS row stride in elements
 
 // Partial sums go to part[split][M][N]; with one split the epilogue runs in place.
-template <int MT>
+template <int MT, bool VEC>
 __global__ __launch_bounds__(256) void skinny_kernel(const bf16* __restrict__ A, int lda,
                                                      const bf16* __restrict__ W, int ldw,
                                                      const float* __restrict__ bias, void* __restrict__ C,
                                                      int ldc, float* __restrict__ part, int M, int N,
-                                                     int K, int k_per_split, int epi, int vec_ok) {
+                                                     int K, int k_per_split, int epi) {
   __shared__ __attribute__((aligned(16))) bf16 As[MT * 16 * SK_LD];
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int n_row = blockIdx.x * 64 + wid * 16 + (lane & 15);   // weight row of this lane
+  const int n_ld = min(n_row, N - 1);                           // the row it reads
   const int kq = (lane >> 4) * 8;                               // k offset inside a 32-step
   const int k_begin = blockIdx.y * k_per_split;
   const int k_end = min(K, k_begin + k_per_split);
@@ -196,20 +248,20 @@ __global__ __launch_bounds__(256) void skinny_kernel(const bf16* __restrict__ A,
   bf16x8 wcur[KC / 32], wnext[KC / 32];
 #pragma unroll
   for (int s = 0; s < KC / 32; ++s)
-    wcur[s] = load8(W, ldw, n_row, N, k_begin + s * 32 + kq, k_end, vec_ok);
+    wcur[s] = load8<VEC>(W, ldw, n_ld, k_begin + s * 32 + kq, k_end);
 
   for (int k0 = k_begin; k0 < k_end; k0 += KC) {
     __syncthreads();
     // stage A[0..16 MT)[k0..k0+KC): 32 chunks of 8 per row
     for (int c = tid; c < MT * 16 * (KC / 8); c += 256) {
       const int r = c / (KC / 8), kk = (c % (KC / 8)) * 8;
-      *reinterpret_cast<bf16x8*>(&As[r * SK_LD + kk]) = load8(A, lda, r, M, k0 + kk, k_end, vec_ok);
+      *reinterpret_cast<bf16x8*>(&As[r * SK_LD + kk]) = load8<VEC>(A, lda, min(r, M - 1), k0 + kk, k_end);
     }
     __syncthreads();
     if (k0 + KC < k_end) {
 #pragma unroll
       for (int s = 0; s < KC / 32; ++s)
-        wnext[s] = load8(W, ldw, n_row, N, k0 + KC + s * 32 + kq, k_end, vec_ok);
+        wnext[s] = load8<VEC>(W, ldw, n_ld, k0 + KC + s * 32 + kq, k_end);
     }
 #pragma unroll
     for (int s = 0; s < KC / 32; ++s) {
@@ -245,16 +297,19 @@ __global__ __launch_bounds__(256) void skinny_kernel(const bf16* __restrict__ A,
 // the few activation rows from L2 straight into MFMA operands, S steps (32 S k) of loads in
 // flight ahead of the matrix cores.  The waves' sums meet in LDS and wave 0 adds them in a
 // fixed order and runs the epilogue, so there is no second kernel and no atomics.
-template <int NW, int NT, int S>
+template <int NW, int NT, int S, bool VEC>
 __global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restrict__ A, int lda,
                                                            const bf16* __restrict__ W, int ldw,
                                                            const float* __restrict__ bias,
                                                            void* __restrict__ C, int ldc, int M, int N,
-                                                           int K, int k_per_wave, int epi, int vec_ok) {
+                                                           int K, int k_per_wave, int epi) {
   __shared__ float red[NW][NT][64][4];
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int n_base = blockIdx.x * 16 * NT + (lane & 15);
-  const int m_row = lane & 15;
+  const int m_row = min(lane & 15, M - 1);               // rows past M read row M - 1; never stored
+  int n_ld[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) n_ld[j] = min(n_base + 16 * j, N - 1);
   const int kq = (lane >> 4) * 8;
   const int k_begin = wid * k_per_wave;
   const int k_end = min(K, k_begin + k_per_wave);
@@ -262,26 +317,29 @@ __global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restric
 #pragma unroll
   for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
   bf16x8 wc[NT][S], ac[S], wn[NT][S], an[S];
-  if (k_begin < k_end) {
-#pragma unroll
-    for (int s = 0; s < S; ++s) {
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-        wc[j][s] = load8(W, ldw, n_base + 16 * j, N, k_begin + s * 32 + kq, k_end, vec_ok);
-      ac[s] = load8(A, lda, m_row, M, k_begin + s * 32 + kq, k_end, vec_ok);
-    }
-  }
-  for (int k0 = k_begin; k0 < k_end; k0 += S * 32) {
-    const bool more = k0 + S * 32 < k_end;
-    if (more) {
+  // a batch that lies inside [k_begin, k_end) is loaded without guards (a guard's select
+  // would make the wave wait for the load right away, and nothing would be in flight)
+  auto load_batch = [&](int k0, bf16x8 (&wd)[NT][S], bf16x8 (&ad)[S]) {
+    if (VEC && k0 + S * 32 <= k_end) {
 #pragma unroll
       for (int s = 0; s < S; ++s) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
-          wn[j][s] = load8(W, ldw, n_base + 16 * j, N, k0 + (S + s) * 32 + kq, k_end, vec_ok);
-        an[s] = load8(A, lda, m_row, M, k0 + (S + s) * 32 + kq, k_end, vec_ok);
+        for (int j = 0; j < NT; ++j) wd[j][s] = load8_inside(W, ldw, n_ld[j], k0 + s * 32 + kq);
+        ad[s] = load8_inside(A, lda, m_row, k0 + s * 32 + kq);
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < S; ++s) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) wd[j][s] = load8<VEC>(W, ldw, n_ld[j], k0 + s * 32 + kq, k_end);
+        ad[s] = load8<VEC>(A, lda, m_row, k0 + s * 32 + kq, k_end);
       }
     }
+  };
+  if (k_begin < k_end) load_batch(k_begin, wc, ac);
+  for (int k0 = k_begin; k0 < k_end; k0 += S * 32) {
+    const bool more = k0 + S * 32 < k_end;
+    if (more) load_batch(k0 + S * 32, wn, an);
 #pragma unroll
     for (int s = 0; s < S; ++s)
 #pragma unroll
@@ -302,6 +360,25 @@ __global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restric
     for (int r = 0; r < 4; ++r) red[wid][j][lane][r] = acc[j][r];
   __syncthreads();
   if (wid != 0) return;
+  if (epi == EPI_SWIGLU) {       // the block's 64 rows are one group: tiles 0,1 gate, tiles 2,3 up
+    if constexpr (NT == 4) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int col = blockIdx.x * 32 + j * 16 + (lane & 15);
+        if (col >= ldc) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = (lane >> 4) * 4 + r;
+          if (m >= M) continue;
+          float g = 0.f, u = 0.f;
+#pragma unroll
+          for (int w = 0; w < NW; ++w) { g += red[w][j][lane][r]; u += red[w][j + 2][lane][r]; }
+          ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(g, u);
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
     const int n = n_base + 16 * j;
@@ -323,8 +400,13 @@ template <int NW, int NT, int S>
 int launch_skinny16(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
                     int M, int N, int K, int epi, int vec_ok, hipStream_t stream) {
   const int k_per_wave = ((K + NW - 1) / NW + S * 32 - 1) / (S * 32) * (S * 32);
-  skinny16_kernel<NW, NT, S><<<(N + 16 * NT - 1) / (16 * NT), NW * 64, 0, stream>>>(
-      A, lda, W, ldw, bias, C, ldc, M, N, K, k_per_wave, epi, vec_ok);
+  const int blocks = (N + 16 * NT - 1) / (16 * NT);
+  if (vec_ok)
+    skinny16_kernel<NW, NT, S, true><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K,
+                                                                     k_per_wave, epi);
+  else
+    skinny16_kernel<NW, NT, S, false><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K,
+                                                                      k_per_wave, epi);
   return mf_launch_status();
 }
 
@@ -333,6 +415,17 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
                                                             void* __restrict__ C, int ldc, int M, int N,
                                                             int splits, int epi) {
   const int n = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
+  if (epi == EPI_SWIGLU) {       // n runs over the ldc outputs
+    if (n >= ldc) return;
+    const int ng = (n >> 5) * 64 + (n & 31);
+    float g = 0.f, u = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      g += part[((size_t)s * M + m) * N + ng];
+      u += part[((size_t)s * M + m) * N + ng + 32];
+    }
+    ((bf16*)C)[(size_t)m * ldc + n] = (bf16)swiglu_f(g, u);
+    return;
+  }
   if (n >= N) return;
   float v = 0.f;
   for (int s = 0; s < splits; ++s) v += part[((size_t)s * M + m) * N + n];
@@ -344,10 +437,15 @@ int launch_skinny(const bf16* A, int lda, const bf16* W, int ldw, const float* b
                   float* part, int M, int N, int K, int splits, int k_per_split, int epi, int vec_ok,
                   hipStream_t stream) {
   dim3 grid((N + 63) / 64, splits);
-  skinny_kernel<MT><<<grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, splits > 1 ? part : nullptr,
-                                              M, N, K, k_per_split, epi, vec_ok);
+  const bool two_pass = splits > 1 || epi == EPI_SWIGLU;   // gate and up columns sit in different waves
+  if (vec_ok)
+    skinny_kernel<MT, true><<<grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc,
+                                                      two_pass ? part : nullptr, M, N, K, k_per_split, epi);
+  else
+    skinny_kernel<MT, false><<<grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc,
+                                                       two_pass ? part : nullptr, M, N, K, k_per_split, epi);
   int rc = mf_launch_status();
-  if (rc == 0 && splits > 1) {
+  if (rc == 0 && two_pass) {
     dim3 g2((N + 255) / 256, M);
     skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, splits, epi);
     rc = mf_launch_status();
@@ -361,9 +459,11 @@ int launch_skinny(const bf16* A, int lda, const bf16* W, int ldw, const float* b
 MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
                         int ldc, int M, int N, int K, int epi, int variant, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || lda < K || ldw < K || ldc < N || epi < 0 || epi > 2) return (int)hipErrorInvalidValue;
+  if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > 3) return (int)hipErrorInvalidValue;
+  if (epi == EPI_SWIGLU ? (N % 64 != 0 || ldc > N / 2 || ldc <= N / 2 - 32 || bias) : ldc < N)
+    return (int)hipErrorInvalidValue;
   const int vec_ok = (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) &&
-                     ((uintptr_t)W % 16 == 0);
+                     ((uintptr_t)W % 16 == 0) && (K % 8 == 0);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   if (variant == 0) {
@@ -371,6 +471,7 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
     const long t128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     variant = (t256 >= 512) ? 1 : (t128 >= 64 || M > 64) ? 2 : 3;
   }
+  if (epi == EPI_SWIGLU && variant == 3) variant = 2;      // needs two 32-column tiles per wave
   switch (variant) {
     case 1: return launch_tile<256, 256, 128, 128>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case 2: return launch_tile<128, 128, 64, 64>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
@@ -384,11 +485,14 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
                                void* C, int ldc, float* part, int M, int N, int K, int splits,
                                int k_per_split, int epi, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || lda < K || ldw < K || ldc < N || epi < 0 || epi > 2 || splits < 1 ||
+  if (M > 64 || K <= 0 || lda < K || ldw < K || epi < 0 || epi > 3 || splits < 1 ||
       k_per_split % KC != 0 || (long)splits * k_per_split < K || (splits > 1 && !part))
     return (int)hipErrorInvalidValue;
+  if (epi == EPI_SWIGLU ? (N % 64 != 0 || ldc > N / 2 || ldc <= N / 2 - 32 || bias || (M > 16 && !part))
+                        : ldc < N)
+    return (int)hipErrorInvalidValue;
   const int vec_ok = (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) &&
-                     ((uintptr_t)W % 16 == 0);
+                     ((uintptr_t)W % 16 == 0) && (K % 8 == 0);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   static const int variant16 = getenv("MF_SKINNY16") ? atoi(getenv("MF_SKINNY16")) : 0;
@@ -397,6 +501,8 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
     // Measured at 3584..152064 weight rows: many rows -> 4 waves with two 16-row tiles each
     // (less activation traffic per weight byte); a row count that would leave a short second
     // round of 16-row blocks -> 8 waves with two tiles; otherwise 8 waves, one tile.
+    if (epi == EPI_SWIGLU)
+      return launch_skinny16<4, 4, 2>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     const int blocks16 = (N + 15) / 16;
     int v = variant16;
     if (v == 0) v = blocks16 >= 1024 ? 4 : (blocks16 > 256 && blocks16 <= 512 ? 3 : 1);

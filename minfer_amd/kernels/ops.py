@@ -16,7 +16,7 @@ from . import build
 PAGE = 64          # tokens per cache page (MF_PAGE in csrc/common.h)
 HAVE_PREFILL_ATTENTION = True
 PREFILL_BLOCK = 128     # query tokens per workgroup of the prompt attention kernel
-EPI_F32, EPI_ACC_F32, EPI_BF16 = 0, 1, 2
+EPI_F32, EPI_ACC_F32, EPI_BF16, EPI_SWIGLU = 0, 1, 2, 3
 
 
 class KernelError(RuntimeError):
@@ -268,6 +268,42 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
         return
     _check(_fn("gemm_bf16", "mf_gemm_bf16")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n, m,
                                              n, k, epi, variant, _stream()), "gemm_bf16")
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """Rows of gate and up `[nf][k]` in groups of 64: 32 gate rows, then the 32 up rows of the
+    same outputs; the last group is padded with zero rows.  The layout `linear_swiglu` reads."""
+    nf, k = gate.shape
+    groups = (nf + 31) // 32
+    pad = groups * 32 - nf
+    if pad:
+        z = torch.zeros((pad, k), dtype=gate.dtype, device=gate.device)
+        gate, up = torch.cat([gate, z]), torch.cat([up, z])
+    return torch.stack([gate.view(groups, 32, k), up.view(groups, 32, k)], dim=1).reshape(groups * 64, k).contiguous()
+
+
+def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, variant: int = 0) -> None:
+    """out = silu(x @ Wg^T) * (x @ Wu^T) in one kernel; `weight` is `interleave_gate_up(Wg, Wu)`,
+    everything bfloat16, `out` is [rows][nf]."""
+    _need(x, "linear_swiglu.x", torch.bfloat16)
+    _need(weight, "linear_swiglu.weight", torch.bfloat16)
+    m, k = x.shape
+    n = weight.shape[0]
+    nf = out.shape[1]
+    if weight.shape[1] != k or n % 64 or not n // 2 - 32 < nf <= n // 2:
+        raise KernelError(f"linear_swiglu: x {tuple(x.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+    _need(out, "linear_swiglu.out", torch.bfloat16, (m, nf))
+    if m == 0:
+        return
+    if m <= 64 and variant == 0:
+        splits, per = skinny_plan(m, n, k)
+        part = workspace("skinny", splits * m * n, x.device) if m > 16 else None
+        _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
+                                                        _ptr(part), m, n, k, splits, per, EPI_SWIGLU, _stream()),
+               "gemm_bf16_skinny(swiglu)")
+        return
+    _check(_fn("gemm_bf16", "mf_gemm_bf16")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf, m, n, k,
+                                             EPI_SWIGLU, variant, _stream()), "gemm_bf16(swiglu)")
 
 
 # ------------------------------------------------------------------ attention

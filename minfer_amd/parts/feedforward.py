@@ -1,6 +1,8 @@
 """SwiGLU feed-forward without biases: down( silu(gate x) * (up x) ), silu(z) = z/(1+e^-z)
 (src/models/qwen2/graph.rs:154-176, src/graph/cpu_backend.rs:323-329 of yusiwen/minfer).
-gate|up are one stacked matrix; the down product adds into the residual."""
+gate|up are one matrix.  In bfloat16 its rows are interleaved so that the product's epilogue
+applies SwiGLU from the 32-bit accumulators and writes y directly; in 32-bit the stacked
+product is followed by the SwiGLU kernel.  The down product adds into the residual."""
 from __future__ import annotations
 
 import torch
@@ -20,7 +22,7 @@ class SwiGLU(FeedForward):
         p = spec.params
         self.hidden, self.inter = int(p["hidden_size"]), int(p["intermediate_size"])
         self.names = {k: p[k] for k in ("gate", "up", "down")}
-        self.gate_up = self.down = None
+        self.gate_up = self.down = self.fused = None
 
     def tensor_specs(self):
         n = self.names
@@ -30,11 +32,17 @@ class SwiGLU(FeedForward):
 
     def load(self, get):
         n = self.names
-        self.gate_up = Linear.stacked([get(n["gate"] + ".weight"), get(n["up"] + ".weight")])
+        gate, up = get(n["gate"] + ".weight"), get(n["up"] + ".weight")
+        if self.rt.is_bf16 and gate.dtype == up.dtype == torch.bfloat16:
+            self.fused = ops.interleave_gate_up(gate, up)
+        else:
+            self.gate_up = Linear.stacked([gate, up])
         self.down = Linear(get(n["down"] + ".weight"))
 
     def forward(self, x, h, ctx) -> None:
-        gu = self.gate_up(x, out_dtype=torch.float32)
         y = torch.empty((x.shape[0], self.inter), dtype=self.rt.dtype, device=x.device)
-        ops.swiglu(gu, y)
+        if self.fused is not None:
+            ops.linear_swiglu(x, self.fused, y)
+        else:
+            ops.swiglu(self.gate_up(x, out_dtype=torch.float32), y)
         self.down(y, out=h, accumulate=True)

@@ -85,6 +85,25 @@ def linear(x, weight, bias, out, accumulate=False, variant=0):
     out.copy_(y.to(out.dtype))
 
 
+def interleave_gate_up(gate, up):
+    """The layout the fused kernel reads, built row by row."""
+    nf, k = gate.shape
+    groups = (nf + 31) // 32
+    out = torch.zeros(groups * 64, k, dtype=gate.dtype)
+    for i in range(nf):
+        out[(i // 32) * 64 + i % 32] = gate[i]
+        out[(i // 32) * 64 + 32 + i % 32] = up[i]
+    return out
+
+
+def linear_swiglu(x, weight, out, variant=0):
+    nf = out.shape[1]
+    idx = torch.arange(nf)
+    g = x.double() @ weight.double()[(idx // 32) * 64 + idx % 32].t()
+    u = x.double() @ weight.double()[(idx // 32) * 64 + 32 + idx % 32].t()
+    out.copy_((g / (1.0 + torch.exp(-g)) * u).to(out.dtype))
+
+
 def gather_cache_rows(cache, page_table_row, length):
     """[length][kv_heads][head_dim] rows 0..length-1 of one sequence."""
     pos = torch.arange(length)
@@ -163,7 +182,7 @@ def advance(next_ids, sampled, positions, steps):
 
 NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", "rope_table",
          "rope_kvwrite", "linear", "attn_tokens", "attn_prefill", "argmax", "sample", "penalties",
-         "top_k", "top_p", "advance"]
+         "top_k", "top_p", "advance", "interleave_gate_up", "linear_swiglu"]
 
 
 def install(monkeypatch):

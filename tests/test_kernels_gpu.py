@@ -399,3 +399,21 @@ def test_attn_prefill_far_key_and_window_edge(ops):
     q2[2] = q[qi]
     ops.attn_prefill(q2.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), ctx_on(DEV), out, nh, nk, hd, 1.0, 0)
     assert not torch.allclose(out[2, :hd].float().cpu(), vrow, atol=3e-2)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("m,nf,k", [(1, 176, 64), (8, 344, 128), (16, 32, 200), (17, 176, 64), (64, 1000, 344),
+                                    (65, 232, 200), (300, 18944, 256), (130, 31, 72)])
+def test_gemm_bf16_swiglu(ops, variant, m, nf, k):
+    x = rnd((m, k), torch.bfloat16, 30)
+    wg, wu = rnd((nf, k), torch.bfloat16, 31, 0.3), rnd((nf, k), torch.bfloat16, 32, 0.3)
+    g, u = x.double() @ wg.double().t(), x.double() @ wu.double().t()
+    ref = g / (1 + torch.exp(-g)) * u
+    w = ops.interleave_gate_up(wg.to(DEV), wu.to(DEV))
+    assert torch.equal(w.cpu(), plain_ops.interleave_gate_up(wg, wu))
+    out = torch.empty(m, nf, dtype=torch.bfloat16, device=DEV)
+    ops.linear_swiglu(x.to(DEV), w, out, variant=variant)
+    close(out, ref, 2e-5 * math.sqrt(k) + 1e-3, 1e-2)
+    again = torch.empty(m, nf, dtype=torch.bfloat16, device=DEV)
+    ops.linear_swiglu(x.to(DEV), w, again, variant=variant)
+    assert torch.equal(out, again)
