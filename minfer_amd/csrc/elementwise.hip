@@ -43,6 +43,36 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
   __shared__ float scratch[4];
   const int row = blockIdx.x;
   const float* xr = x + (size_t)(row_idx ? row_idx[row] : row) * d;
+  OT* o = out + (size_t)row * d;
+  // rows up to 256 * 4 * KEEP elements stay in registers between the sum and the scaling
+  constexpr int KEEP = 4;
+  if (d % 4 == 0 && d <= 256 * 4 * KEEP) {
+    float4 v[KEEP];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < KEEP; ++c) {
+      const int i = (c * 256 + threadIdx.x) * 4;
+      v[c] = i < d ? *reinterpret_cast<const float4*>(xr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+      ss = fmaf(v[c].x, v[c].x, ss);
+      ss = fmaf(v[c].y, v[c].y, ss);
+      ss = fmaf(v[c].z, v[c].z, ss);
+      ss = fmaf(v[c].w, v[c].w, ss);
+    }
+    ss = block_sum<256>(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+    for (int c = 0; c < KEEP; ++c) {
+      const int i = (c * 256 + threadIdx.x) * 4;
+      if (i < d) {
+        const float4 g = w ? *reinterpret_cast<const float4*>(w + i) : make_float4(1.f, 1.f, 1.f, 1.f);
+        o[i + 0] = from_f32<OT>(v[c].x * scale * g.x);
+        o[i + 1] = from_f32<OT>(v[c].y * scale * g.y);
+        o[i + 2] = from_f32<OT>(v[c].z * scale * g.z);
+        o[i + 3] = from_f32<OT>(v[c].w * scale * g.w);
+      }
+    }
+    return;
+  }
   float ss = 0.f;
   for (int i = threadIdx.x; i < d; i += 256) {
     const float v = xr[i];
@@ -50,7 +80,6 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
   }
   ss = block_sum<256>(ss, scratch);
   const float scale = 1.0f / sqrtf(ss / (float)d + eps);
-  OT* o = out + (size_t)row * d;
   for (int i = threadIdx.x; i < d; i += 256) {
     const float g = w ? w[i] : 1.0f;
     o[i] = from_f32<OT>(xr[i] * scale * g);

@@ -297,7 +297,7 @@ __global__ __launch_bounds__(256) void skinny_kernel(const bf16* __restrict__ A,
 // the few activation rows from L2 straight into MFMA operands, S steps (32 S k) of loads in
 // flight ahead of the matrix cores.  The waves' sums meet in LDS and wave 0 adds them in a
 // fixed order and runs the epilogue, so there is no second kernel and no atomics.
-template <int NW, int NT, int S, bool VEC>
+template <int NW, int NT, int S, bool VEC, bool PAIR = false>
 __global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restrict__ A, int lda,
                                                            const bf16* __restrict__ W, int ldw,
                                                            const float* __restrict__ bias,
@@ -305,11 +305,14 @@ __global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restric
                                                            int K, int k_per_wave, int epi) {
   __shared__ float red[NW][NT][64][4];
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
-  const int n_base = blockIdx.x * 16 * NT + (lane & 15);
+  // PAIR (SwiGLU, NT = 2): block b owns 16 gate rows of group b / 2 and the 16 up rows of
+  // the same outputs, 32 rows further on
+  constexpr int TSTRIDE = PAIR ? 32 : 16;
+  const int n_base = (PAIR ? (blockIdx.x >> 1) * 64 + (blockIdx.x & 1) * 16 : blockIdx.x * 16 * NT) + (lane & 15);
   const int m_row = min(lane & 15, M - 1);               // rows past M read row M - 1; never stored
   int n_ld[NT];
 #pragma unroll
-  for (int j = 0; j < NT; ++j) n_ld[j] = min(n_base + 16 * j, N - 1);
+  for (int j = 0; j < NT; ++j) n_ld[j] = min(n_base + TSTRIDE * j, N - 1);
   const int kq = (lane >> 4) * 8;
   const int k_begin = wid * k_per_wave;
   const int k_end = min(K, k_begin + k_per_wave);
@@ -360,19 +363,17 @@ __global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restric
     for (int r = 0; r < 4; ++r) red[wid][j][lane][r] = acc[j][r];
   __syncthreads();
   if (wid != 0) return;
-  if (epi == EPI_SWIGLU) {       // the block's 64 rows are one group: tiles 0,1 gate, tiles 2,3 up
-    if constexpr (NT == 4) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int col = blockIdx.x * 32 + j * 16 + (lane & 15);
-        if (col >= ldc) continue;
+  if (epi == EPI_SWIGLU) {       // tile 0 gate, tile 1 up
+    if constexpr (PAIR && NT == 2) {
+      const int col = blockIdx.x * 16 + (lane & 15);
+      if (col < ldc) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int m = (lane >> 4) * 4 + r;
           if (m >= M) continue;
           float g = 0.f, u = 0.f;
 #pragma unroll
-          for (int w = 0; w < NW; ++w) { g += red[w][j][lane][r]; u += red[w][j + 2][lane][r]; }
+          for (int w = 0; w < NW; ++w) { g += red[w][0][lane][r]; u += red[w][1][lane][r]; }
           ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(g, u);
         }
       }
@@ -396,17 +397,17 @@ __global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restric
   }
 }
 
-template <int NW, int NT, int S>
+template <int NW, int NT, int S, bool PAIR = false>
 int launch_skinny16(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
                     int M, int N, int K, int epi, int vec_ok, hipStream_t stream) {
   const int k_per_wave = ((K + NW - 1) / NW + S * 32 - 1) / (S * 32) * (S * 32);
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
   if (vec_ok)
-    skinny16_kernel<NW, NT, S, true><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K,
-                                                                     k_per_wave, epi);
+    skinny16_kernel<NW, NT, S, true, PAIR><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
+                                                                           K, k_per_wave, epi);
   else
-    skinny16_kernel<NW, NT, S, false><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K,
-                                                                      k_per_wave, epi);
+    skinny16_kernel<NW, NT, S, false, PAIR><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M,
+                                                                            N, K, k_per_wave, epi);
   return mf_launch_status();
 }
 
@@ -502,7 +503,7 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
     // (less activation traffic per weight byte); a row count that would leave a short second
     // round of 16-row blocks -> 8 waves with two tiles; otherwise 8 waves, one tile.
     if (epi == EPI_SWIGLU)
-      return launch_skinny16<4, 4, 2>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+      return launch_skinny16<4, 2, 4, true>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     const int blocks16 = (N + 15) / 16;
     int v = variant16;
     if (v == 0) v = blocks16 >= 1024 ? 4 : (blocks16 > 256 && blocks16 <= 512 ? 3 : 1);

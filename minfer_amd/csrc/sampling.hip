@@ -86,6 +86,46 @@ __global__ __launch_bounds__(NT) void argmax_kernel(const float* __restrict__ lo
   }
 }
 
+// Greedy over a large vocabulary with few rows: a row is cut into `chunks` pieces, one block
+// each, and a second pass picks among the pieces (still the first maximum).
+__global__ __launch_bounds__(NT) void argmax_part_kernel(const float* __restrict__ logits, int ld, int vocab,
+                                                         int chunks, float* __restrict__ pval,
+                                                         int* __restrict__ pidx) {
+  __shared__ float s_val[NT / 64];
+  __shared__ int s_idx[NT / 64];
+  const int per = (vocab + chunks - 1) / chunks;
+  const int lo = blockIdx.y * per, n = min(per, vocab - lo);
+  float bv = -INFINITY;
+  int bi = 0;
+  if (n > 0) {
+    block_argmax(logits + (size_t)blockIdx.x * ld + lo, n, 1.0f, s_val, s_idx, bv, bi);
+    bi += lo;
+  }
+  if (threadIdx.x == 0) {
+    pval[blockIdx.x * chunks + blockIdx.y] = n > 0 ? bv : -INFINITY;
+    pidx[blockIdx.x * chunks + blockIdx.y] = bi;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ pval,
+                                                          const int* __restrict__ pidx, int chunks,
+                                                          int* __restrict__ out) {
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += 64) {
+    const float v = pval[blockIdx.x * chunks + c];
+    const int i = pidx[blockIdx.x * chunks + c];
+    if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, MF_WAVE);
+    const int oi = __shfl_xor(bi, o, MF_WAVE);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
+}
+
 // temperature draw; temp < 1e-6 falls back to greedy (src/sampler.rs:225-227)
 __global__ __launch_bounds__(NT) void sample_kernel(const float* __restrict__ logits, int ld, int vocab,
                                                     float temp, uint64_t seed,
@@ -338,11 +378,21 @@ __global__ void advance_kernel(int* __restrict__ next_ids, const int* __restrict
 
 }  // namespace
 
-MF_API int mf_argmax(const float* logits, int ld, int rows, int vocab, int* out, float* out_val,
+// `work` (chunks * rows floats and as many ints, chunks <= 64) lets few rows of a large
+// vocabulary spread over the chip; without it a row is one block.
+MF_API int mf_argmax(const float* logits, int ld, int rows, int vocab, int* out, float* work, int chunks,
                      hipStream_t stream) {
   if (rows <= 0) return 0;
-  if (vocab <= 0 || ld < vocab) return (int)hipErrorInvalidValue;
-  argmax_kernel<<<rows, NT, 0, stream>>>(logits, ld, vocab, out, out_val);
+  if (vocab <= 0 || ld < vocab || chunks > 64) return (int)hipErrorInvalidValue;
+  if (work && chunks > 1) {
+    int* pidx = reinterpret_cast<int*>(work + (size_t)rows * chunks);
+    argmax_part_kernel<<<dim3(rows, chunks), NT, 0, stream>>>(logits, ld, vocab, chunks, work, pidx);
+    int rc = mf_launch_status();
+    if (rc) return rc;
+    argmax_final_kernel<<<rows, 64, 0, stream>>>(work, pidx, chunks, out);
+    return mf_launch_status();
+  }
+  argmax_kernel<<<rows, NT, 0, stream>>>(logits, ld, vocab, out, nullptr);
   return mf_launch_status();
 }
 

@@ -57,7 +57,7 @@ _PROTOTYPES = {
                                  c_int, c_float, c_int, _P],
     },
     "sampling": {
-        "mf_argmax": [_P, c_int, c_int, c_int, _P, _P],
+        "mf_argmax": [_P, c_int, c_int, c_int, _P, _P, c_int, _P],
         "mf_sample": [_P, c_int, c_int, c_int, c_float, c_uint64, _P, _P, _P, _P, _P],
         "mf_penalties": [_P, c_int, c_int, c_int, _P, c_int, _P, c_float, c_float, c_float, _P],
         "mf_top_k": [_P, c_int, c_int, c_int, c_int, _P],
@@ -390,8 +390,12 @@ def _logit_rows(logits: torch.Tensor, name: str):
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     rows, vocab = _logit_rows(logits, "argmax.logits")
     _need(out, "argmax.out", torch.int32, (rows,))
-    _check(_fn("sampling", "mf_argmax")(_ptr(logits), vocab, rows, vocab, _ptr(out), _ptr(None), _stream()),
-           "argmax")
+    chunks = 1
+    if vocab >= 16384 and rows < 256:          # few long rows: several blocks per row
+        chunks = max(1, min(64, 512 // rows, vocab // 4096))
+    work = workspace("argmax", 2 * rows * chunks, logits.device) if chunks > 1 else None
+    _check(_fn("sampling", "mf_argmax")(_ptr(logits), vocab, rows, vocab, _ptr(out), _ptr(work), chunks,
+                                         _stream()), "argmax")
 
 
 def sample(logits: torch.Tensor, temp: float, seed: int, keys: torch.Tensor, steps: torch.Tensor,
