@@ -226,16 +226,23 @@ int launch_tile(const bf16* A, int lda, const bf16* W, int ldw, const float* bia
 constexpr int KC = 256;          // k per staging step
 constexpr int SK_LD = KC + 8;    // LDS row stride in elements
 
-// Partial sums go to part[split][M][N]; with one split the epilogue runs in place.
+// 17 to 64 rows.  A block of 8 waves owns 128 weight rows; each wave streams its 16 rows from
+// HBM straight into MFMA operands, a chunk (256 k) ahead; the activation rows of a chunk are
+// staged in LDS once per block (double-buffered: the next chunk travels global -> registers
+// while this one is multiplied, and is written to the other buffer afterwards, so there is
+// one barrier per chunk).  Partial sums go to part[split][M][N]; with one split the epilogue
+// runs in place.
 template <int MT, bool VEC>
-__global__ __launch_bounds__(256) void skinny_kernel(const bf16* __restrict__ A, int lda,
+__global__ __launch_bounds__(512) void skinny_kernel(const bf16* __restrict__ A, int lda,
                                                      const bf16* __restrict__ W, int ldw,
                                                      const float* __restrict__ bias, void* __restrict__ C,
                                                      int ldc, float* __restrict__ part, int M, int N,
                                                      int K, int k_per_split, int epi) {
-  __shared__ __attribute__((aligned(16))) bf16 As[MT * 16 * SK_LD];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  bf16* As = reinterpret_cast<bf16*>(smem);                     // [2][MT * 16][SK_LD]
+  constexpr int ROWS = MT * 16;
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
-  const int n_row = blockIdx.x * 64 + wid * 16 + (lane & 15);   // weight row of this lane
+  const int n_row = blockIdx.x * 128 + wid * 16 + (lane & 15);  // weight row of this lane
   const int n_ld = min(n_row, N - 1);                           // the row it reads
   const int kq = (lane >> 4) * 8;                               // k offset inside a 32-step
   const int k_begin = blockIdx.y * k_per_split;
@@ -245,35 +252,56 @@ __global__ __launch_bounds__(256) void skinny_kernel(const bf16* __restrict__ A,
 #pragma unroll
   for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  bf16x8 wcur[KC / 32], wnext[KC / 32];
+  // staging slots of this thread: MT chunks of 8 k; chunk c -> row c / 32, k (c % 32) * 8
+  int srow[MT], sk[MT];
 #pragma unroll
-  for (int s = 0; s < KC / 32; ++s)
-    wcur[s] = load8<VEC>(W, ldw, n_ld, k_begin + s * 32 + kq, k_end);
-
+  for (int i = 0; i < MT; ++i) {
+    const int c = i * 512 + tid;
+    srow[i] = c / (KC / 8);
+    sk[i] = (c % (KC / 8)) * 8;
+  }
+  bf16x8 wcur[KC / 32], wnext[KC / 32], stage[MT];
+  auto load_chunk = [&](int k0, bf16x8 (&wd)[KC / 32]) {
+    if (VEC && k0 + KC <= k_end) {                     // inside: no guards, nothing waits
+#pragma unroll
+      for (int s = 0; s < KC / 32; ++s) wd[s] = load8_inside(W, ldw, n_ld, k0 + s * 32 + kq);
+#pragma unroll
+      for (int i = 0; i < MT; ++i) stage[i] = load8_inside(A, lda, min(srow[i], M - 1), k0 + sk[i]);
+    } else {
+#pragma unroll
+      for (int s = 0; s < KC / 32; ++s) wd[s] = load8<VEC>(W, ldw, n_ld, k0 + s * 32 + kq, k_end);
+#pragma unroll
+      for (int i = 0; i < MT; ++i) stage[i] = load8<VEC>(A, lda, min(srow[i], M - 1), k0 + sk[i], k_end);
+    }
+  };
+  auto store_stage = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+      *reinterpret_cast<bf16x8*>(&As[(buf * ROWS + srow[i]) * SK_LD + sk[i]]) = stage[i];
+  };
+  load_chunk(k_begin, wcur);
+  store_stage(0);
+  __syncthreads();
+  int buf = 0;
   for (int k0 = k_begin; k0 < k_end; k0 += KC) {
-    __syncthreads();
-    // stage A[0..16 MT)[k0..k0+KC): 32 chunks of 8 per row
-    for (int c = tid; c < MT * 16 * (KC / 8); c += 256) {
-      const int r = c / (KC / 8), kk = (c % (KC / 8)) * 8;
-      *reinterpret_cast<bf16x8*>(&As[r * SK_LD + kk]) = load8<VEC>(A, lda, min(r, M - 1), k0 + kk, k_end);
-    }
-    __syncthreads();
-    if (k0 + KC < k_end) {
-#pragma unroll
-      for (int s = 0; s < KC / 32; ++s)
-        wnext[s] = load8<VEC>(W, ldw, n_ld, k0 + KC + s * 32 + kq, k_end);
-    }
+    const bool more = k0 + KC < k_end;
+    if (more) load_chunk(k0 + KC, wnext);
+    const bf16* as = As + buf * ROWS * SK_LD;
 #pragma unroll
     for (int s = 0; s < KC / 32; ++s) {
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
-        const bf16x8 a =
-            *reinterpret_cast<const bf16x8*>(&As[(i * 16 + (lane & 15)) * SK_LD + s * 32 + kq]);
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&as[(i * 16 + (lane & 15)) * SK_LD + s * 32 + kq]);
         acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, wcur[s], acc[i], 0, 0, 0);
       }
     }
+    if (more) {
+      store_stage(buf ^ 1);
 #pragma unroll
-    for (int s = 0; s < KC / 32; ++s) wcur[s] = wnext[s];
+      for (int s = 0; s < KC / 32; ++s) wcur[s] = wnext[s];
+    }
+    __syncthreads();
+    buf ^= 1;
   }
 
   // D[m][n]: lane holds n = lane % 16, m = 4 (lane / 16) + r
@@ -433,25 +461,40 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
   store_out(C, ldc, m, n, v + (bias ? bias[n] : 0.f), epi);
 }
 
-template <int MT>
-int launch_skinny(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
-                  float* part, int M, int N, int K, int splits, int k_per_split, int epi, int vec_ok,
-                  hipStream_t stream) {
-  dim3 grid((N + 63) / 64, splits);
+template <int MT, bool VEC>
+int launch_skinny_v(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
+                    float* part, int M, int N, int K, int splits, int k_per_split, int epi,
+                    hipStream_t stream) {
+  constexpr int smem = 2 * MT * 16 * SK_LD * (int)sizeof(bf16);
+  static bool configured = false;
+  auto kern = skinny_kernel<MT, VEC>;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    configured = true;
+  }
+  dim3 grid((N + 127) / 128, splits);
   const bool two_pass = splits > 1 || epi == EPI_SWIGLU;   // gate and up columns sit in different waves
-  if (vec_ok)
-    skinny_kernel<MT, true><<<grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc,
-                                                      two_pass ? part : nullptr, M, N, K, k_per_split, epi);
-  else
-    skinny_kernel<MT, false><<<grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc,
-                                                       two_pass ? part : nullptr, M, N, K, k_per_split, epi);
+  kern<<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, two_pass ? part : nullptr, M, N, K,
+                                    k_per_split, epi);
   int rc = mf_launch_status();
   if (rc == 0 && two_pass) {
-    dim3 g2((N + 255) / 256, M);
+    dim3 g2(((epi == EPI_SWIGLU ? ldc : N) + 255) / 256, M);
     skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, splits, epi);
     rc = mf_launch_status();
   }
   return rc;
+}
+
+template <int MT>
+int launch_skinny(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
+                  float* part, int M, int N, int K, int splits, int k_per_split, int epi, int vec_ok,
+                  hipStream_t stream) {
+  return vec_ok ? launch_skinny_v<MT, true>(A, lda, W, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split,
+                                            epi, stream)
+                : launch_skinny_v<MT, false>(A, lda, W, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split,
+                                             epi, stream);
 }
 
 }  // namespace

@@ -228,7 +228,7 @@ def skinny_plan(m: int, n: int, k: int, target_blocks: int = 1024) -> Tuple[int,
     """(splits, k_per_split) of the decode product: enough blocks to fill the chip."""
     if m <= 16:
         return 1, (k + 255) // 256 * 256      # one kernel: K is split between the waves of a block
-    n_blocks = (n + 63) // 64
+    n_blocks = (n + 127) // 128
     chunks = (k + 255) // 256
     splits = max(1, min(chunks, target_blocks // max(1, n_blocks)))
     per = (chunks + splits - 1) // splits
