@@ -75,29 +75,51 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     for (int i = tid; i < (HDP - HD) * VT_LD; i += 256) Vt[HD * VT_LD + i] = (bf16)0.f;
   }
 
-  for (int page_i = key_lo / KT; page_i <= blk_p_hi / KT; ++page_i) {
+  // K and V of a page travel global -> registers while the page before is multiplied
+  constexpr int KCH = (KT * (HD / 8) + 255) / 256;       // K chunks of 8 elements per thread
+  constexpr int VCH = (HD / 8 + 3) / 4;                  // V chunks per thread (lane = key)
+  bf16x8 kreg[KCH], vreg[VCH];
+  auto fetch = [&](int page_i) {
     const int page = pt[page_i];
     const bf16* kp = kc + ((size_t)page * nk + hk) * KT * HD;
     const bf16* vp = vc + ((size_t)page * nk + hk) * KT * HD;
-    __syncthreads();                                     // the previous step's reads are done
-    // K as stored: thread -> (row, 8-element chunk), coalesced
-    for (int c = tid; c < KT * (HD / 8); c += 256) {
-      const int row = c / (HD / 8), ch = c % (HD / 8);
-      *reinterpret_cast<bf16x8*>(&Ks[row * K_LD + ch * 8]) =
-          *reinterpret_cast<const bf16x8*>(kp + (size_t)row * HD + ch * 8);
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = i * 256 + tid;
+      if (c < KT * (HD / 8)) kreg[i] = *reinterpret_cast<const bf16x8*>(kp + (size_t)(c / (HD / 8)) * HD + (c % (HD / 8)) * 8);
     }
-    // V transposed: lane = key, so that the 2-byte LDS writes of a wave fall side by side.
     // Rows after the block's last position were never written (a page is not cleared when
     // it is taken): they are masked out of P, but 0 * garbage could still be NaN, so they
     // enter as zeros.
     const bool v_written = page_i * KT + lane <= blk_p_hi;
-    for (int c = wid; c < HD / 8; c += 4) {
-      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (v_written) v = *reinterpret_cast<const bf16x8*>(vp + (size_t)lane * HD + c * 8);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) Vt[(c * 8 + e) * VT_LD + lane] = v[e];
+    for (int i = 0; i < VCH; ++i) {
+      const int c = i * 4 + wid;
+      vreg[i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (c < HD / 8 && v_written) vreg[i] = *reinterpret_cast<const bf16x8*>(vp + (size_t)lane * HD + c * 8);
+    }
+  };
+  const int page_first = key_lo / KT, page_last = blk_p_hi / KT;
+  fetch(page_first);
+  for (int page_i = page_first; page_i <= page_last; ++page_i) {
+    __syncthreads();                                     // the previous step's reads are done
+    // K as stored: thread -> (row, 8-element chunk)
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = i * 256 + tid;
+      if (c < KT * (HD / 8)) *reinterpret_cast<bf16x8*>(&Ks[(c / (HD / 8)) * K_LD + (c % (HD / 8)) * 8]) = kreg[i];
+    }
+    // V transposed: lane = key, so that the 2-byte LDS writes of a wave fall side by side
+#pragma unroll
+    for (int i = 0; i < VCH; ++i) {
+      const int c = i * 4 + wid;
+      if (c < HD / 8) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) Vt[(c * 8 + e) * VT_LD + lane] = vreg[i][e];
+      }
     }
     __syncthreads();
+    if (page_i < page_last) fetch(page_i + 1);
     const int key0 = page_i * KT;
     if (key0 > wave_p_hi) continue;                      // every key is later than every query here
     if (window > 0 && key0 + KT - 1 <= wave_p_lo - window) continue;   // or left of every window

@@ -67,27 +67,37 @@ __device__ __forceinline__ bf16x8 load8_inside(const bf16* __restrict__ base, in
 }
 
 // ------------------------------------------------------------------ tiled kernel
-constexpr int BK = 64;
-constexpr int LDS_LD = BK + 8;   // row stride in elements: 144 bytes, conflict-free b128 reads
-
-template <int BM, int BN, int WM, int WN, bool VEC>
-__global__ __launch_bounds__(256) void tile_kernel(const bf16* __restrict__ A, int lda,
+// LDS row stride is BK + 8 elements (144 bytes for BK 64, 80 for BK 32): conflict-free b128 reads
+template <int BM, int BN, int WM, int WN, int BK, bool VEC>
+__global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const bf16* __restrict__ A, int lda,
                                                    const bf16* __restrict__ W, int ldw,
                                                    const float* __restrict__ bias, void* __restrict__ C,
-                                                   int ldc, int M, int N, int K, int epi, int tiles_m) {
-  static_assert((BM / WM) * (BN / WN) == 4, "four waves per block");
+                                                   int ldc, int M, int N, int K, int epi, int tiles_m,
+                                                   int xcd_remap) {
+  constexpr int NTHR = 64 * (BM / WM) * (BN / WN);
+  constexpr int LDS_LD = BK + 8;
   constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int PA = BM / 32, PW = BN / 32;   // load passes: 32 rows x 64 k per pass
+  constexpr int RP = NTHR / (BK / 8);         // rows per load pass
+  constexpr int PA = BM / RP, PW = BN / RP;
+  static_assert(BM % RP == 0 && BN % RP == 0, "load passes cover the tile");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* As = reinterpret_cast<bf16*>(smem);               // [2][BM][LDS_LD]
   bf16* Ws = As + 2 * BM * LDS_LD;                        // [2][BN][LDS_LD]
 
-  // Consecutive blocks walk down M first, so blocks that run together share W tiles.
-  const int bm = blockIdx.x % tiles_m, bn = blockIdx.x / tiles_m;
+  // Workgroups go to the 8 XCDs in turn, each with an L2 of its own: give every XCD one
+  // contiguous eighth of the tiles, walking down M first, so that a W tile is fetched by one
+  // L2 only and the tiles an XCD has in flight share their W rows.
+  int tile = blockIdx.x;
+  if (xcd_remap) {
+    const int n_tiles = gridDim.x, per = n_tiles / 8, rem = n_tiles % 8;
+    const int x = blockIdx.x % 8, qq = blockIdx.x / 8;
+    tile = x * per + min(x, rem) + qq;
+  }
+  const int bm = tile % tiles_m, bn = tile / tiles_m;
   const int m0 = bm * BM, n0 = bn * BN;
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int wm = (wid % (BM / WM)) * WM, wn = (wid / (BM / WM)) * WN;
-  const int lrow = tid >> 3, lk = (tid & 7) * 8;
+  const int lrow = tid / (BK / 8), lk = (tid % (BK / 8)) * 8;
   const int fr = lane & 31, fk = (lane >> 5) * 8;
 
   floatx16 acc[TM][TN];
@@ -101,9 +111,9 @@ __global__ __launch_bounds__(256) void tile_kernel(const bf16* __restrict__ A, i
   bf16x8 ra[PA], rw[PW];
   int arow[PA], wrow[PW];                       // rows past the matrix read its last row
 #pragma unroll
-  for (int p = 0; p < PA; ++p) arow[p] = min(m0 + p * 32 + lrow, M - 1);
+  for (int p = 0; p < PA; ++p) arow[p] = min(m0 + p * RP + lrow, M - 1);
 #pragma unroll
-  for (int p = 0; p < PW; ++p) wrow[p] = min(n0 + p * 32 + lrow, N - 1);
+  for (int p = 0; p < PW; ++p) wrow[p] = min(n0 + p * RP + lrow, N - 1);
   const int nkt = (K + BK - 1) / BK;
   const int nkt_inside = VEC ? K / BK : 0;      // k tiles that need no guard (the loop's fast form:
                                                 // a guard's select would wait for the load at once)
@@ -124,10 +134,10 @@ __global__ __launch_bounds__(256) void tile_kernel(const bf16* __restrict__ A, i
   load_tile(0);
 #pragma unroll
   for (int p = 0; p < PA; ++p)
-    *reinterpret_cast<bf16x8*>(&As[(p * 32 + lrow) * LDS_LD + lk]) = ra[p];
+    *reinterpret_cast<bf16x8*>(&As[(p * RP + lrow) * LDS_LD + lk]) = ra[p];
 #pragma unroll
   for (int p = 0; p < PW; ++p)
-    *reinterpret_cast<bf16x8*>(&Ws[(p * 32 + lrow) * LDS_LD + lk]) = rw[p];
+    *reinterpret_cast<bf16x8*>(&Ws[(p * RP + lrow) * LDS_LD + lk]) = rw[p];
   __syncthreads();
 
   for (int kt = 0; kt < nkt; ++kt) {
@@ -156,10 +166,10 @@ __global__ __launch_bounds__(256) void tile_kernel(const bf16* __restrict__ A, i
       bf16* wn_ = Ws + (cur ^ 1) * BN * LDS_LD;
 #pragma unroll
       for (int p = 0; p < PA; ++p)
-        *reinterpret_cast<bf16x8*>(&an[(p * 32 + lrow) * LDS_LD + lk]) = ra[p];
+        *reinterpret_cast<bf16x8*>(&an[(p * RP + lrow) * LDS_LD + lk]) = ra[p];
 #pragma unroll
       for (int p = 0; p < PW; ++p)
-        *reinterpret_cast<bf16x8*>(&wn_[(p * 32 + lrow) * LDS_LD + lk]) = rw[p];
+        *reinterpret_cast<bf16x8*>(&wn_[(p * RP + lrow) * LDS_LD + lk]) = rw[p];
     }
     __syncthreads();
   }
@@ -198,12 +208,13 @@ __global__ __launch_bounds__(256) void tile_kernel(const bf16* __restrict__ A, i
     }
 }
 
-template <int BM, int BN, int WM, int WN, bool VEC>
+template <int BM, int BN, int WM, int WN, int BK, bool VEC>
 int launch_tile_v(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
                   int M, int N, int K, int epi, hipStream_t stream) {
-  constexpr int smem = 2 * (BM + BN) * LDS_LD * (int)sizeof(bf16);
+  constexpr int smem = 2 * (BM + BN) * (BK + 8) * (int)sizeof(bf16);
+  constexpr int NTHR = 64 * (BM / WM) * (BN / WN);
   static bool configured = false;
-  auto kern = tile_kernel<BM, BN, WM, WN, VEC>;
+  auto kern = tile_kernel<BM, BN, WM, WN, BK, VEC>;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -211,15 +222,17 @@ int launch_tile_v(const bf16* A, int lda, const bf16* W, int ldw, const float* b
     configured = true;
   }
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  kern<<<tiles_m * tiles_n, 256, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, tiles_m);
+  static const int remap = getenv("MF_NO_XCD_REMAP") ? 0 : 1;
+  kern<<<tiles_m * tiles_n, NTHR, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, tiles_m,
+                                                  remap && tiles_m * tiles_n >= 16);
   return mf_launch_status();
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int BK = 64>
 int launch_tile(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
                 int M, int N, int K, int epi, int vec_ok, hipStream_t stream) {
-  return vec_ok ? launch_tile_v<BM, BN, WM, WN, true>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, stream)
-                : launch_tile_v<BM, BN, WM, WN, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, stream);
+  return vec_ok ? launch_tile_v<BM, BN, WM, WN, BK, true>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, stream)
+                : launch_tile_v<BM, BN, WM, WN, BK, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, stream);
 }
 
 // ------------------------------------------------------------------ skinny kernel
@@ -499,7 +512,8 @@ int launch_skinny(const bf16* A, int lda, const bf16* W, int ldw, const float* b
 
 }  // namespace
 
-// `variant`: 0 picks by shape; 1: 256x256 tile, 2: 128x128, 3: 64x64 (tests name them).
+// `variant`: 0 picks by shape; 1: 256x256 tile with 4 waves, 2: 128x128, 3: 64x64, 9: 256x256
+// with 8 waves; 4..8 are other shapes kept for measurements (tests name them).
 MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
                         int ldc, int M, int N, int K, int epi, int variant, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -511,15 +525,23 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   if (variant == 0) {
+    // measured at 2048 rows: 256x256 tiles (8 waves) win once there are several tiles per CU,
+    // 128x128 otherwise; tiny problems take 64x64
     const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
     const long t128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-    variant = (t256 >= 512) ? 1 : (t128 >= 64 || M > 64) ? 2 : 3;
+    variant = (t256 >= 768) ? 9 : (t128 >= 64 || M > 64) ? 2 : 3;
   }
   if (epi == EPI_SWIGLU && variant == 3) variant = 2;      // needs two 32-column tiles per wave
   switch (variant) {
     case 1: return launch_tile<256, 256, 128, 128>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case 2: return launch_tile<128, 128, 64, 64>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case 3: return launch_tile<64, 64, 32, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case 4: return launch_tile<128, 128, 64, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case 5: return launch_tile<128, 128, 64, 64, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case 6: return launch_tile<256, 128, 64, 64, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case 7: return launch_tile<128, 256, 64, 64, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case 8: return launch_tile<256, 256, 128, 64, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case 9: return launch_tile<256, 256, 128, 64, 64>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
   }
   return (int)hipErrorInvalidValue;
 }

@@ -46,11 +46,13 @@ class StepContext:
         host's copy of the step once and kept."""
         key = ("query_tiles", block)
         if key not in self._memo:
-            seqs, starts = [], []
+            tiles = []
             for b, n in enumerate(self.host_new):
+                first = self.host_start[b] if self.host_start else 0
                 for q0 in range(0, n, block):
-                    seqs.append(b)
-                    starts.append(q0)
+                    tiles.append((first + min(q0 + block, n), b, q0))     # keys its last query sees
+            tiles.sort(key=lambda t: -t[0])                               # longest first: they finish together
+            seqs, starts = [t[1] for t in tiles], [t[2] for t in tiles]
             both = torch.tensor([seqs, starts], dtype=torch.int32).to(self.token_ids.device)
             self._memo[key] = (both[0], both[1])
         return self._memo[key]

@@ -185,7 +185,7 @@ def test_gemm_f32(ops, m, n, k):
     close(acc, ref - b.double() + base.double(), 1e-5 * math.sqrt(k) / 8, 1e-5)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 6, 9])
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(2048, 512, 256), (1, 152064, 64), (64, 3584, 3584)])
 def test_gemm_bf16(ops, variant, m, n, k):
     if variant and (m * n * k > 3e9):
@@ -401,7 +401,7 @@ def test_attn_prefill_far_key_and_window_edge(ops):
     assert not torch.allclose(out[2, :hd].float().cpu(), vrow, atol=3e-2)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("variant", [0, 1, 2, 9])
 @pytest.mark.parametrize("m,nf,k", [(1, 176, 64), (8, 344, 128), (16, 32, 200), (17, 176, 64), (64, 1000, 344),
                                     (65, 232, 200), (300, 18944, 256), (130, 31, 72)])
 def test_gemm_bf16_swiglu(ops, variant, m, nf, k):
