@@ -40,6 +40,7 @@ def parse():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--only", choices=["decode", "prefill"], help="run one part (for profiles); prints no JSON line")
     return ap.parse_args()
 
 
@@ -144,10 +145,18 @@ def main() -> int:
     cfg = dict(QWEN25_7B, num_hidden_layers=a.layers)
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[a.dtype]
     elem = 2 if a.dtype == "bf16" else 4
-    batches = [a.batch] + ([] if a.no_points else [1, 64])
+    batches = [a.batch] + ([] if (a.no_points or a.only) else [1, 64])
     max_tokens = max(batches) * a.context
     llm = LLM(config=cfg, random_weights=True, weight_seed=0, dtype=dtype, n_ctx=a.context,
               n_slots=max(batches), max_tokens=max_tokens)
+    if a.only == "decode":
+        r = run_decode(llm, cfg, a.batch, a.prompt_max, a.steps, a.warmup, not a.no_graph, elem)
+        print(f"decode batch {a.batch}: {r['tok_s']:.1f} tok/s, {r['ms']:.3f} ms/step, {r['gbs']:.0f} GB/s")
+        return 0
+    if a.only == "prefill":
+        s = run_prefill(llm, cfg, a.prefill_tokens)
+        print(f"prefill {a.prefill_tokens} tokens: {s * 1e3:.2f} ms, {a.prefill_tokens / s:.0f} tok/s")
+        return 0
     main_run = run_decode(llm, cfg, a.batch, a.prompt_max, a.steps, a.warmup, not a.no_graph, elem)
     pre_s = run_prefill(llm, cfg, a.prefill_tokens)
     points = {}

@@ -6,9 +6,14 @@ import numpy as np
 
 from tiny import random_tokens
 
-# tolerance of bfloat16 logits, as a fraction of the logits' standard deviation: bfloat16
-# keeps 8 bits, the run rounds activations a few times per layer
-BF16_REL = 0.04
+# bfloat16 logits, as fractions of the logits' standard deviation over the vocabulary.
+# bfloat16 keeps 8 bits (relative rounding error 2^-9/sqrt(3) = 0.11 % rms) and a run rounds
+# activations about eight times per layer, so the error of a logit is a sum of many small
+# independent terms: its rms over the vocabulary is what the size of the model fixes (measured
+# 0.3..0.8 % from 64 to 3584 wide), while its maximum grows with the number of entries looked
+# at (4.9 sigma at 152064).  Both are bounded: rms 1 %, maximum 5.5 %.
+BF16_RMS = 0.01
+BF16_MAX = 0.055
 F32_ABS = 1e-4
 
 
@@ -98,10 +103,16 @@ def compare(rows, ref, dtype: str, what: str):
     worst = 0.0
     for (rid, p), got in sorted(rows.items()):
         want = ref[rid][p]
-        err = float(np.abs(got.astype(np.float64) - want).max())
-        tol = F32_ABS if dtype == "float32" else BF16_REL * float(want.std())
+        diff = got.astype(np.float64) - want
+        err = float(np.abs(diff).max())
+        tol = F32_ABS if dtype == "float32" else BF16_MAX * float(want.std())
         assert np.isfinite(got).all(), f"{what}: non-finite logits at request {rid} position {p}"
         assert err <= tol, (f"{what} [{dtype}]: request {rid} position {p} (of {len(ref[rid])}): "
                             f"max abs err {err:.3e} > {tol:.3e}")
+        if dtype != "float32":
+            rms = float(np.sqrt(np.mean(diff * diff)))
+            assert rms <= BF16_RMS * float(want.std()), (
+                f"{what} [{dtype}]: request {rid} position {p}: rms err {rms:.3e} > "
+                f"{BF16_RMS * float(want.std()):.3e}")
         worst = max(worst, err)
     return worst

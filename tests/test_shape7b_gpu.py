@@ -1,0 +1,42 @@
+"""One layer at the widths of Qwen2.5-7B (hidden 3584, 28 heads over 4 kv heads of 128,
+feed-forward 18944, vocabulary 152064) with random weights: 32-bit logits against the plain
+implementation under the three ways of cutting, and bfloat16 within its tolerance.  The
+sums here are as long as in the full model (18944 terms in the down product)."""
+import numpy as np
+import pytest
+
+from plain_qwen2 import PlainQwen2
+from replays import batch_steps, compare, plain_logits, requests_for, run_steps, tail_steps, whole_steps
+
+pytestmark = pytest.mark.gpu
+
+SHAPE_7B_ONE_LAYER = dict(
+    architectures=["Qwen2ForCausalLM"], model_type="qwen2", hidden_act="silu",
+    num_hidden_layers=1, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+    intermediate_size=18944, vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-6,
+    max_position_embeddings=32768, tie_word_embeddings=True, use_sliding_window=False)
+
+
+@pytest.fixture(scope="module")
+def folder(tmp_path_factory):
+    from minfer_amd import config_from_dict, write_random_model
+    return write_random_model(str(tmp_path_factory.mktemp("shape7b") / "m"), config_from_dict(SHAPE_7B_ONE_LAYER), seed=5)
+
+
+@pytest.fixture(scope="module")
+def reference(folder):
+    plain = PlainQwen2.from_folder(folder, dtype=np.float64)
+    reqs = requests_for(152064, (3, 20, 9, 37), seed=6)
+    return reqs, plain_logits(plain, reqs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_layer_at_7b_widths(folder, reference, dtype):
+    from minfer_amd import Engine, load_model
+    reqs, ref = reference
+    ids = list(reqs)
+    eng = Engine(load_model(folder, dtype=dtype), max_tokens=64 * 4, poison_cache=True)
+    worst = max(compare(run_steps(eng, whole_steps(reqs)), ref, dtype, "7B widths whole"),
+                compare(run_steps(eng, tail_steps(reqs, tail=8)), ref, dtype, "7B widths one by one"),
+                compare(run_steps(eng, batch_steps(reqs, [ids[:3], ids[3:]])), ref, dtype, "7B widths batches"))
+    print(f"{dtype}: worst abs err {worst:.3e}")
