@@ -4,8 +4,12 @@
 // yusiwen/minfer; the reference's own matrix kernels are quantised and are not followed.)
 //
 // Three kernels:
-//  * `tile_kernel`: many rows (prompts).  A BM x BN block tile per 256 threads, K walked
-//    in steps of 64 through double-buffered LDS, 32x32x16 MFMA, each wave a WM x WN tile.
+//  * `tile_kernel`: many rows (prompts).  A BM x BN block tile per 4 or 8 waves, K walked in
+//    steps of BK through double-buffered LDS, 32x32x16 MFMA, each wave a WM x WN tile.
+//    Measured on MI355X at 2048 rows: what bounds it is operand delivery into the CU (the
+//    same loop without its global loads runs a third faster, without its LDS reads a tenth),
+//    so the largest tile that still leaves two waves per SIMD wins where there are enough
+//    tiles; prefetching two tiles ahead in registers changed nothing and was dropped.
 //  * `skinny16_kernel`: at most 16 rows (decode).  The time is the weight stream: the waves
 //    of a block split K, each reads weights and activations straight into MFMA operands
 //    (16x16x32) and the partial sums meet in LDS.
@@ -512,8 +516,8 @@ int launch_skinny(const bf16* A, int lda, const bf16* W, int ldw, const float* b
 
 }  // namespace
 
-// `variant`: 0 picks by shape; 1: 256x256 tile with 4 waves, 2: 128x128, 3: 64x64, 9: 256x256
-// with 8 waves; 4..8 are other shapes kept for measurements (tests name them).
+// `variant`: 0 picks by shape; 1: 256x256 tile with 4 waves, 2: 128x128, 3: 64x64, 6: 256x128
+// with 8 waves, 9: 256x256 with 8 waves (tests name them).
 MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
                         int ldc, int M, int N, int K, int epi, int variant, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -536,11 +540,7 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
     case 1: return launch_tile<256, 256, 128, 128>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case 2: return launch_tile<128, 128, 64, 64>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case 3: return launch_tile<64, 64, 32, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    case 4: return launch_tile<128, 128, 64, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    case 5: return launch_tile<128, 128, 64, 64, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case 6: return launch_tile<256, 128, 64, 64, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    case 7: return launch_tile<128, 256, 64, 64, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    case 8: return launch_tile<256, 256, 128, 64, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case 9: return launch_tile<256, 256, 128, 64, 64>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
   }
   return (int)hipErrorInvalidValue;
