@@ -3,14 +3,16 @@
 // (out[t][o] = dot(W[o][:], x[t][:]) + b[o], src/graph/cpu_backend.rs:214-248 of
 // yusiwen/minfer; the reference's own matrix kernels are quantised and are not followed.)
 //
-// Three kernels:
+// Four kernels:
 //  * `tile_kernel`: many rows (prompts).  A BM x BN block tile per 4 or 8 waves, K walked in
 //    steps of BK through double-buffered LDS, 32x32x16 MFMA, each wave a WM x WN tile.
 //    Measured on MI355X at 2048 rows: what bounds it is operand delivery into the CU (the
 //    same loop without its global loads runs a third faster, without its LDS reads a tenth),
 //    so the largest tile that still leaves two waves per SIMD wins where there are enough
 //    tiles; prefetching two tiles ahead in registers changed nothing and was dropped.
-//  * `skinny16_kernel`: at most 16 rows (decode).  The time is the weight stream: the waves
+//  * `stationary16_kernel`: at most 16 rows and K of 1536, 2048, 3584 or 4096 (decode): one
+//    block per CU keeps the activations in registers and walks over weight tiles.
+//  * `skinny16_kernel`: at most 16 rows, any K (decode).  The time is the weight stream: the waves
 //    of a block split K, each reads weights and activations straight into MFMA operands
 //    (16x16x32) and the partial sums meet in LDS.
 //  * `skinny_kernel`: 17 to 64 rows.  Each wave owns 16 weight rows and reads them from HBM
@@ -456,6 +458,120 @@ int launch_skinny16(const bf16* A, int lda, const bf16* W, int ldw, const float*
   return mf_launch_status();
 }
 
+// At most 16 rows and K = 256 NS (NS steps of 32 k for each of 8 waves): the activations are
+// read once per block and stay in registers.  The grid is one block per CU; a block walks
+// over its share of the 16-row weight tiles (items), and the load of the next item's
+// weights is issued right behind the MFMA that frees the register, so the weight stream
+// never pauses between items.  After an item the waves' sums meet in LDS (two buffers, one
+// barrier per item) and the waves take turns at adding them and running the epilogue.
+// Against the kernel above this removes the per-tile re-read of the activations (which
+// cost a quarter of the time at 8 rows) and the start-up of a block per tile.
+template <int NS, int NT, bool PAIR>
+__global__ __launch_bounds__(512) void stationary16_kernel(const bf16* __restrict__ A, int lda,
+                                                           const bf16* __restrict__ W, int ldw,
+                                                           const float* __restrict__ bias,
+                                                           void* __restrict__ C, int ldc, int M, int N,
+                                                           int n_items, int epi) {
+  constexpr int NW = 8;
+  constexpr int COLS = 16 * NT;            // weight rows (output columns) of an item
+  constexpr int RS = COLS + 4;             // row stride of the sums in LDS: conflict-free writes
+  __shared__ float red[2][NW][16][RS];     // [buffer][wave][activation row][weight row of the item]
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int r16 = lane & 15;
+  const int k0 = wid * NS * 32 + (lane >> 4) * 8;         // this lane's k in step 0 of its slice
+  const bf16* arow = A + (size_t)min(r16, M - 1) * lda + k0;
+  bf16x8 afr[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) afr[s] = *reinterpret_cast<const bf16x8*>(arow + s * 32);
+
+  // first weight row of tile j of an item (before the lane's own row is added)
+  auto tile_row = [&](int item, int j) {
+    return PAIR ? (item >> 1) * 64 + (item & 1) * 16 + j * 32 : (item * NT + j) * 16;
+  };
+  bf16x8 w[NT][NS];
+  const bf16* wrow[NT];
+  int item = blockIdx.x;
+  if (item < n_items) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      wrow[j] = W + (size_t)min(tile_row(item, j) + r16, N - 1) * ldw + k0;
+#pragma unroll
+      for (int s = 0; s < NS; ++s) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32);
+    }
+  }
+  for (int it = 0; item < n_items; item += gridDim.x, ++it) {
+    const int next = item + gridDim.x;
+    const bool has_next = next < n_items;
+    if (has_next) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) wrow[j] = W + (size_t)min(tile_row(next, j) + r16, N - 1) * ldw + k0;
+    }
+    floatx4 acc[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afr[s], w[j][s], acc[j], 0, 0, 0);
+        if (has_next) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32);
+      }
+    }
+    // D[m][n]: n = lane % 16, m = 4 (lane / 16) + r
+    const int buf = it & 1;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[buf][wid][(lane >> 4) * 4 + r][j * 16 + r16] = acc[j][r];
+    __syncthreads();
+    // The buffer is written again two items on, behind the next barrier, which this wave
+    // reaches only after it has read its sums here.
+    if (wid != (it & (NW - 1))) continue;
+    if (epi == EPI_SWIGLU) {
+      if constexpr (PAIR && NT == 2) {
+        const int col = item * 16 + r16;
+        if (col < ldc) {
+          for (int m = lane >> 4; m < M; m += 4) {
+            float g = 0.f, u = 0.f;
+#pragma unroll
+            for (int ww = 0; ww < NW; ++ww) { g += red[buf][ww][m][r16]; u += red[buf][ww][m][16 + r16]; }
+            ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(g, u);
+          }
+        }
+      }
+      continue;
+    }
+    // a pass of the wave covers 64 / COLS activation rows of COLS adjacent outputs each
+    const int c = lane % COLS;
+    const int n = tile_row(item, c >> 4) + (c & 15);
+    if (n >= N) continue;
+    const float b = bias ? bias[n] : 0.f;
+    for (int m = lane / COLS; m < M; m += 64 / COLS) {
+      float v = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < NW; ++ww) v += red[buf][ww][m][c];
+      store_out(C, ldc, m, n, v + b, epi);
+    }
+  }
+}
+
+// true when the shape is one the register-resident kernel is built for
+template <int NS, int NT, bool PAIR>
+int launch_stationary16(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
+                        int M, int N, int epi, hipStream_t stream) {
+  const int n_items = PAIR ? N / 32 : (N + 16 * NT - 1) / (16 * NT);
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return (int)hipErrorUnknown;
+    n_cu = prop.multiProcessorCount;
+  }
+  const int grid = n_items < n_cu ? n_items : n_cu;
+  stationary16_kernel<NS, NT, PAIR><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, n_items, epi);
+  return mf_launch_status();
+}
+
 __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restrict__ part,
                                                             const float* __restrict__ bias,
                                                             void* __restrict__ C, int ldc, int M, int N,
@@ -567,6 +683,23 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
     // Measured at 3584..152064 weight rows: many rows -> 4 waves with two 16-row tiles each
     // (less activation traffic per weight byte); a row count that would leave a short second
     // round of 16-row blocks -> 8 waves with two tiles; otherwise 8 waves, one tile.
+    // K = 256 NS with enough tiles to go round: the register-resident kernel
+    static const int stationary = getenv("MF_NO_STATIONARY") ? 0 : 1;
+    if (stationary && vec_ok && K % 256 == 0 && (N + 15) / 16 >= 128) {
+      // two tiles an item where there are enough of them: 128-byte rows of 32-bit output
+      static const int nt_env = getenv("MF_STATIONARY_NT") ? atoi(getenv("MF_STATIONARY_NT")) : 0;
+      const bool two = nt_env ? nt_env == 2 : (N + 31) / 32 >= 128;
+#define MF_STATIONARY(NS_)                                                                                  \
+  case NS_:                                                                                                 \
+    return epi == EPI_SWIGLU                                                                                \
+               ? launch_stationary16<NS_, 2, true>(a, lda, w, ldw, bias, C, ldc, M, N, epi, stream)         \
+           : two ? launch_stationary16<NS_, 2, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, stream)      \
+                 : launch_stationary16<NS_, 1, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, stream);
+      switch (K / 256) {
+        MF_STATIONARY(6) MF_STATIONARY(8) MF_STATIONARY(14) MF_STATIONARY(16)
+      }
+#undef MF_STATIONARY
+    }
     if (epi == EPI_SWIGLU)
       return launch_skinny16<4, 2, 4, true>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     const int blocks16 = (N + 15) / 16;
