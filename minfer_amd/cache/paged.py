@@ -11,7 +11,9 @@ context.  The same rule makes reuse safe: a page's old rows are never read, beca
 sequence reads positions below its own length only and writes each before reading it.
 
 Layers with the same needs (kv heads, head size, window) form a group with storage of its
-own: one K and one V tensor `[entries][pages][kv_heads][64][head_dim]` and one page pool.
+own: one K tensor `[entries][pages][kv_heads][64][head_dim]`, one V tensor (the same shape in
+32-bit, `[entries][pages][kv_heads][head_dim][64]` in bfloat16, see `v_page_shape`) and one
+page pool.
 A group with a window gives pages back as soon as every position in them has left the
 window of all later queries.
 """
@@ -23,6 +25,15 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import torch
 
 PAGE = 64
+
+
+def v_page_shape(n_kv_heads: int, head_dim: int, dtype) -> Tuple[int, int, int]:
+    """One page of V: like K, `[kv_heads][64][head_dim]`, in 32-bit; transposed inside the page,
+    `[kv_heads][head_dim][64]`, in bfloat16, where the attention kernels feed V^T rows to the
+    matrix cores as they are stored."""
+    if dtype == torch.bfloat16:
+        return (n_kv_heads, head_dim, PAGE)
+    return (n_kv_heads, PAGE, head_dim)
 
 
 class CacheError(RuntimeError):
@@ -87,9 +98,10 @@ class KVGroup:
         self.entries = list(entries)
         self.index_of = {e: i for i, e in enumerate(self.entries)}
         self.pool = PagePool(n_pages)
-        shape = (len(entries), n_pages, request.n_kv_heads, PAGE, request.head_dim)
-        self.k = torch.empty(shape, dtype=dtype, device=device)
-        self.v = torch.empty(shape, dtype=dtype, device=device)
+        self.k = torch.empty((len(entries), n_pages, request.n_kv_heads, PAGE, request.head_dim),
+                             dtype=dtype, device=device)
+        self.v = torch.empty((len(entries), n_pages) + v_page_shape(request.n_kv_heads, request.head_dim, dtype),
+                             dtype=dtype, device=device)
         if poison:
             self.k.fill_(float("nan"))
             self.v.fill_(float("nan"))
@@ -238,7 +250,7 @@ class Cache:
 
     # ------------------------------------------------------------ views
     def kv(self, entry: int):
-        """(K, V) of one entry: `[pages][kv_heads][64][head_dim]` each, and its group."""
+        """(K, V) of one entry, `[pages]` + page shape each, and its group."""
         g = self.group_of[entry]
         i = g.index_of[entry]
         return g.k[i], g.v[i], g

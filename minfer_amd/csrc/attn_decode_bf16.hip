@@ -1,0 +1,249 @@
+// Attention of single query tokens over the paged cache in bfloat16 on the gfx950 matrix
+// cores (decode), split along the keys.
+//
+// For a query token t of sequence b at position p and kv head hk, the G = nh/nk query heads
+// of the group read the same keys: cache rows j with lo <= j <= p, lo = 0 or p - window + 1.
+// s_j = dot(q, K_j) * scale; softmax over j; o = sum_j p_j V_j (src/graph/cpu_backend.rs:
+// 437-494 of yusiwen/minfer; the causal rule "rows 0..=pos" is its `vl = pos + 1`, :462).
+// The softmax is the online form of the reference's CUDA kernel (running max, running sum,
+// rescaled accumulator, src/cuda_kernels.cu:673-790), in 32-bit; probabilities are rounded to
+// bfloat16 for the second product, as in the prompt kernel.
+//
+// The heads of a group share every key, so up to 16 of them are the second matrix of one
+// product: a wave takes 32 keys at a time and computes, with 16x16x32 MFMAs,
+//   S^T[key][head] = K Q^T      A = K rows straight from the cache, B = Q held in registers
+//   O^T[col][head] += V^T P^T   A = V^T rows straight from the cache, B = P^T
+// The cache keeps V transposed inside a page ([head_dim][64 keys]) in bfloat16, so V^T rows
+// are contiguous over the keys like K rows are over head_dim, and neither operand passes
+// through LDS.  In both results a lane owns one head (lane % 16): the softmax statistics are
+// per-lane scalars, and the scores a lane holds (8 consecutive keys, by the choice of which
+// key each K row of a tile is) are exactly the 8 k-slots of its B operand in the second
+// product, so P never leaves its registers.
+//
+// A block is (token, kv head, chunk of 16 heads, key split); its 4 waves take the 32-key steps
+// of the split in turn and merge through LDS.  The split length follows the token's own
+// length, so every split has work.  With several splits each block writes an unnormalised
+// partial (acc, max, sum) and attn_combine_kernel merges them in a fixed order.
+#include "attn_tokens_impl.h"
+
+namespace {
+
+constexpr int STEP = 32;       // keys per wave step
+
+template <int HD>
+__global__ __launch_bounds__(256) void attn_decode_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vt,
+    const int* __restrict__ page_table, int pt_stride, const int* __restrict__ positions,
+    const int* __restrict__ seq_of_tok, bf16* __restrict__ out, float* __restrict__ part, int nh, int nk,
+    float scale, int window, int n_splits) {
+  constexpr int KS = (HD + 31) / 32;      // 32-wide steps over head_dim in the first product
+  constexpr int CT = HD / 16;             // 16-wide column tiles of the output
+  constexpr int O_LD = HD + 4;
+  __shared__ float sm_o[4][16][O_LD];
+  __shared__ float sm_ml[4][16][2];
+
+  const int t = blockIdx.x;
+  const int G = nh / nk;
+  const int n_gc = (G + 15) / 16;
+  const int hk = blockIdx.y / n_gc;
+  const int g0 = (blockIdx.y % n_gc) * 16;
+  const int gcount = min(16, G - g0);
+  const int h0 = hk * G + g0;
+  const int split = blockIdx.z;
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, q4 = lane >> 4;
+
+  const int p = positions[t];
+  const int* pt = page_table + (size_t)seq_of_tok[t] * pt_stride;
+  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  // split length: this token's keys over the splits, in whole block rounds of 4 steps
+  const int per = (p + 1 - lo + n_splits - 1) / n_splits;
+  const int split_len = (per + 4 * STEP - 1) / (4 * STEP) * (4 * STEP);
+  const int j_begin = lo + split * split_len;
+  const int j_end = min(p + 1, j_begin + split_len);
+
+  // B operand of the first product: row = head r16, 8 elements of head_dim at 32 ks + 8 q4
+  bf16x8 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    qf[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    const int d = ks * 32 + q4 * 8;
+    if (r16 < gcount && d < HD)
+      qf[ks] = *reinterpret_cast<const bf16x8*>(q + ((size_t)t * nh + h0 + r16) * HD + d);
+  }
+
+  floatx4 oacc[CT];                       // O^T: head r16, columns 16 c + 4 q4 + r
+#pragma unroll
+  for (int c = 0; c < CT; ++c) oacc[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;   // of head r16 (the same in the four lanes that share it)
+
+  // Steps are 32-key blocks of the cache, so a step lies in one page.  Row r16 of K tile a is
+  // key 8 (r16 / 4) + 4 a + r16 % 4 of the step: the scores of lane (r16, q4) then belong to
+  // keys 8 q4 + 4 a + r, r = 0..3, eight consecutive keys over the two tiles.
+  const int step0 = j_begin / STEP;
+  const int n_steps = j_begin < j_end ? (j_end - 1) / STEP - step0 + 1 : 0;
+  const int krow = 8 * (r16 >> 2) + (r16 & 3);
+  bf16x8 kn[2][KS], vn[CT];
+  auto issue = [&](int i) {
+    const int jb = (step0 + i) * STEP;
+    const int page = pt[jb / MF_PAGE];
+    const int off = jb % MF_PAGE;
+    const bf16* kp = kc + (((size_t)page * nk + hk) * MF_PAGE + off + krow) * HD + q4 * 8;
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        kn[a][ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (ks * 32 + q4 * 8 < HD) kn[a][ks] = *reinterpret_cast<const bf16x8*>(kp + (size_t)(4 * a) * HD + ks * 32);
+      }
+    const bf16* vp = vt + (((size_t)page * nk + hk) * HD + r16) * MF_PAGE + off + q4 * 8;
+#pragma unroll
+    for (int c = 0; c < CT; ++c) vn[c] = *reinterpret_cast<const bf16x8*>(vp + (size_t)(16 * c) * MF_PAGE);
+  };
+  if (w < n_steps) issue(w);
+  for (int i = w; i < n_steps; i += 4) {
+    bf16x8 kf[2][KS], vf[CT];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) kf[a][ks] = kn[a][ks];
+#pragma unroll
+    for (int c = 0; c < CT; ++c) vf[c] = vn[c];
+    if (i + 4 < n_steps) issue(i + 4);
+
+    const int jb = (step0 + i) * STEP;
+    const int key0 = jb + 8 * q4;                  // this lane's eight keys: key0 .. key0 + 7
+    const bool edge = jb < j_begin || jb + STEP > j_end;
+    if (edge) {
+      // Keys outside the split are masked out of P below, but their V may never have been
+      // written (a page is not cleared when it is taken) and 0 * garbage could be NaN:
+      // they enter as zeros.
+#pragma unroll
+      for (int c = 0; c < CT; ++c)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (key0 + e < j_begin || key0 + e >= j_end) vf[c][e] = (bf16)0.f;
+    }
+    floatx4 s[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      s[a] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        s[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[a][ks], qf[ks], s[a], 0, 0, 0);
+    }
+    float sc[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = key0 + e;
+      const float v = s[e >> 2][e & 3] * scale;
+      sc[e] = (!edge || (j >= j_begin && j < j_end)) ? v : -INFINITY;
+      mx = fmaxf(mx, sc[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, MF_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, MF_WAVE));
+    const float m_new = fmaxf(m_run, mx);
+    const float corr = (m_new == -INFINITY) ? 1.f : __expf(m_run - m_new);
+    float lsum = 0.f;
+    bf16x8 pf;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float pe = (sc[e] == -INFINITY) ? 0.f : __expf(sc[e] - m_new);
+      lsum += pe;
+      pf[e] = (bf16)pe;
+    }
+    lsum += __shfl_xor(lsum, 16, MF_WAVE);
+    lsum += __shfl_xor(lsum, 32, MF_WAVE);
+    l_run = l_run * corr + lsum;
+    m_run = m_new;
+#pragma unroll
+    for (int c = 0; c < CT; ++c) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) oacc[c][r] *= corr;
+      oacc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[c], pf, oacc[c], 0, 0, 0);
+    }
+  }
+
+  // merge the 4 waves
+#pragma unroll
+  for (int c = 0; c < CT; ++c)
+    *reinterpret_cast<floatx4*>(&sm_o[w][r16][16 * c + 4 * q4]) = oacc[c];
+  if (q4 == 0) { sm_ml[w][r16][0] = m_run; sm_ml[w][r16][1] = l_run; }
+  __syncthreads();
+  // thread -> (head g, 16 threads over the columns)
+  const int g = threadIdx.x >> 4;
+  if (g >= gcount) return;
+  const int sub = threadIdx.x & 15;
+  float mm = -INFINITY;
+#pragma unroll
+  for (int ww = 0; ww < 4; ++ww) mm = fmaxf(mm, sm_ml[ww][g][0]);
+  float cw[4], L = 0.f;
+#pragma unroll
+  for (int ww = 0; ww < 4; ++ww) {
+    cw[ww] = (mm == -INFINITY) ? 0.f : __expf(sm_ml[ww][g][0] - mm);
+    L += sm_ml[ww][g][1] * cw[ww];
+  }
+  const int h = h0 + g;
+  if (n_splits == 1) {
+    bf16* o = out + ((size_t)t * nh + h) * HD;
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    for (int d = sub; d < HD; d += 16) {
+      float a = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) a += sm_o[ww][g][d] * cw[ww];
+      o[d] = (bf16)(a * inv);
+    }
+  } else {
+    float* o = part + (((size_t)t * nh + h) * n_splits + split) * (HD + 2);
+    for (int d = sub; d < HD; d += 16) {
+      float a = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) a += sm_o[ww][g][d] * cw[ww];
+      o[d] = a;
+    }
+    if (sub == 0) { o[HD] = mm; o[HD + 1] = L; }
+  }
+}
+
+template <int HD>
+int launch(const bf16* q, const bf16* kc, const bf16* vt, const int* page_table, int pt_stride,
+           const int* positions, const int* seq_of_tok, bf16* out, float* part, int n_tok, int nh, int nk,
+           float scale, int window, int n_splits, hipStream_t stream) {
+  const int G = nh / nk;
+  dim3 grid(n_tok, nk * ((G + 15) / 16), n_splits);
+  attn_decode_kernel<HD><<<grid, 256, 0, stream>>>(q, kc, vt, page_table, pt_stride, positions, seq_of_tok, out,
+                                                   part, nh, nk, scale, window, n_splits);
+  int rc = mf_launch_status();
+  if (rc == 0 && n_splits > 1) {
+    attn_tokens::attn_combine_kernel<bf16><<<n_tok * nh, 64, 0, stream>>>(part, out, HD, n_splits);
+    rc = mf_launch_status();
+  }
+  return rc;
+}
+
+}  // namespace
+
+// q, out: [n_tok][nh][hd]; kc: [pages][nk][64][hd]; vt: [pages][nk][hd][64] (V transposed inside
+// a page); part: n_tok * nh * n_splits * (hd + 2) floats when n_splits > 1 (at most 64 splits).
+MF_API int mf_attn_decode_bf16(const void* q, const void* kc, const void* vt, const int* page_table,
+                               int pt_stride, const int* positions, const int* seq_of_tok, void* out,
+                               float* part, int n_tok, int nh, int nk, int hd, float scale, int window,
+                               int n_splits, hipStream_t stream) {
+  if (n_tok <= 0) return 0;
+  if (hd % 16 != 0 || hd < 16 || hd > 256 || nk <= 0 || nh % nk != 0 || n_splits < 1 || n_splits > 64 ||
+      (n_splits > 1 && part == nullptr))
+    return (int)hipErrorInvalidValue;
+#define MF_CASE(E)                                                                                          \
+  case E:                                                                                                   \
+    return launch<16 * E>((const bf16*)q, (const bf16*)kc, (const bf16*)vt, page_table, pt_stride,          \
+                          positions, seq_of_tok, (bf16*)out, part, n_tok, nh, nk, scale, window, n_splits,  \
+                          stream);
+  switch (hd / 16) {
+    MF_CASE(1) MF_CASE(2) MF_CASE(3) MF_CASE(4) MF_CASE(5) MF_CASE(6) MF_CASE(7) MF_CASE(8)
+    MF_CASE(9) MF_CASE(10) MF_CASE(11) MF_CASE(12) MF_CASE(13) MF_CASE(14) MF_CASE(15) MF_CASE(16)
+  }
+#undef MF_CASE
+  return (int)hipErrorInvalidValue;
+}

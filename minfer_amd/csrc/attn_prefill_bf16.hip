@@ -9,7 +9,8 @@
 // 32-bit, probabilities are rounded to bfloat16 for the second product.
 //
 // A block (4 waves) owns 128 consecutive query tokens of one sequence and one query head;
-// each wave 32 of them.  Per cache page (64 keys): K goes to LDS as stored, V transposed.
+// each wave 32 of them.  Per cache page (64 keys): K and V^T go to LDS as stored (the cache
+// keeps a page of V transposed, [head_dim][64 keys]).
 //   S^T[key][q] = K Q^T      32x32x16 MFMA, A = K rows from LDS, B = Q held in registers
 //   lane <-> query column, so the row statistics of the softmax are per-lane scalars
 //   O^T[d][q]  += V^T P^T    A = V^T from LDS, B = P^T, which is S^T's own register layout
@@ -77,26 +78,33 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 
   // K and V of a page travel global -> registers while the page before is multiplied
   constexpr int KCH = (KT * (HD / 8) + 255) / 256;       // K chunks of 8 elements per thread
-  constexpr int VCH = (HD / 8 + 3) / 4;                  // V chunks per thread (lane = key)
+  constexpr int VCH = (HD * (KT / 8) + 255) / 256;       // V^T chunks of 8 keys per thread
   bf16x8 kreg[KCH], vreg[VCH];
   auto fetch = [&](int page_i) {
     const int page = pt[page_i];
     const bf16* kp = kc + ((size_t)page * nk + hk) * KT * HD;
-    const bf16* vp = vc + ((size_t)page * nk + hk) * KT * HD;
+    const bf16* vp = vc + ((size_t)page * nk + hk) * HD * KT;     // a page of V is [HD][KT]
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
       const int c = i * 256 + tid;
       if (c < KT * (HD / 8)) kreg[i] = *reinterpret_cast<const bf16x8*>(kp + (size_t)(c / (HD / 8)) * HD + (c % (HD / 8)) * 8);
     }
-    // Rows after the block's last position were never written (a page is not cleared when
+    // Keys after the block's last position were never written (a page is not cleared when
     // it is taken): they are masked out of P, but 0 * garbage could still be NaN, so they
     // enter as zeros.
-    const bool v_written = page_i * KT + lane <= blk_p_hi;
+    const int n_written = blk_p_hi - page_i * KT + 1;    // keys of this page that exist
 #pragma unroll
     for (int i = 0; i < VCH; ++i) {
-      const int c = i * 4 + wid;
-      vreg[i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (c < HD / 8 && v_written) vreg[i] = *reinterpret_cast<const bf16x8*>(vp + (size_t)lane * HD + c * 8);
+      const int c = i * 256 + tid;                       // chunk: column c / 8, keys 8 (c % 8) ..
+      if (c < HD * (KT / 8)) {
+        vreg[i] = *reinterpret_cast<const bf16x8*>(vp + (size_t)c * 8);
+        if (n_written < KT) {
+          const int k0 = (c % (KT / 8)) * 8;
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (k0 + e >= n_written) vreg[i][e] = (bf16)0.f;
+        }
+      }
     }
   };
   const int page_first = key_lo / KT, page_last = blk_p_hi / KT;
@@ -109,13 +117,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       const int c = i * 256 + tid;
       if (c < KT * (HD / 8)) *reinterpret_cast<bf16x8*>(&Ks[(c / (HD / 8)) * K_LD + (c % (HD / 8)) * 8]) = kreg[i];
     }
-    // V transposed: lane = key, so that the 2-byte LDS writes of a wave fall side by side
+    // V^T as stored: thread -> (column, 8-key chunk); the row stride keeps 8-byte alignment only
 #pragma unroll
     for (int i = 0; i < VCH; ++i) {
-      const int c = i * 4 + wid;
-      if (c < HD / 8) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) Vt[(c * 8 + e) * VT_LD + lane] = vreg[i][e];
+      const int c = i * 256 + tid;
+      if (c < HD * (KT / 8)) {
+        bf16* dst = &Vt[(c / (KT / 8)) * VT_LD + (c % (KT / 8)) * 8];
+        *reinterpret_cast<bf16x4*>(dst) = bf16x4{vreg[i][0], vreg[i][1], vreg[i][2], vreg[i][3]};
+        *reinterpret_cast<bf16x4*>(dst + 4) = bf16x4{vreg[i][4], vreg[i][5], vreg[i][6], vreg[i][7]};
       }
     }
     __syncthreads();

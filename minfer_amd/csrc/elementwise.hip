@@ -194,7 +194,9 @@ MF_API int mf_rope_table(float* cs, float* sn, int n_pos, int half, double theta
 // token's position before attention reads it (src/graph/cpu_backend.rs:118-149).
 // qkv is [T][(nh + 2 nk) hd] in 32-bit with biases already added.  One block per
 // (token, head of q|k|v).
-template <typename OT>
+// In bfloat16 a page of V is stored transposed, [hd][64 keys], the layout the attention
+// kernels read as a matrix-core operand; in 32-bit it lies like K, [64 keys][hd].
+template <typename OT, bool V_TRANSPOSED>
 __global__ __launch_bounds__(64) void rope_kvwrite_kernel(
     const float* __restrict__ qkv, const float* __restrict__ cs, const float* __restrict__ sn,
     const int* __restrict__ positions, const int* __restrict__ seq_of_tok,
@@ -219,15 +221,19 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(
   if (page < 0) return;
   const bool is_k = head < nh + nk;
   const int hk = is_k ? head - nh : head - nh - nk;
-  OT* dst = (is_k ? kcache : vcache) + (((size_t)page * nk + hk) * MF_PAGE + pos % MF_PAGE) * hd;
   if (is_k) {
+    OT* dst = kcache + (((size_t)page * nk + hk) * MF_PAGE + pos % MF_PAGE) * hd;
     for (int i = threadIdx.x; i < half; i += 64) {
       const float c = cs[(size_t)pos * half + i], s = sn[(size_t)pos * half + i];
       const float x0 = src[i], x1 = src[i + half];
       dst[i] = from_f32<OT>(x0 * c - x1 * s);
       dst[i + half] = from_f32<OT>(x0 * s + x1 * c);
     }
+  } else if (V_TRANSPOSED) {      // a page of V is [hd][64 keys]
+    OT* dst = vcache + ((size_t)page * nk + hk) * hd * MF_PAGE + pos % MF_PAGE;
+    for (int i = threadIdx.x; i < hd; i += 64) dst[(size_t)i * MF_PAGE] = from_f32<OT>(src[i]);
   } else {
+    OT* dst = vcache + (((size_t)page * nk + hk) * MF_PAGE + pos % MF_PAGE) * hd;
     for (int i = threadIdx.x; i < hd; i += 64) dst[i] = from_f32<OT>(src[i]);
   }
 }
@@ -239,11 +245,11 @@ MF_API int mf_rope_kvwrite(const float* qkv, const float* cs, const float* sn, c
   if (n_tok <= 0) return 0;
   dim3 grid(n_tok, write_kv ? nh + 2 * nk : nh);
   if (is_bf16)
-    rope_kvwrite_kernel<bf16><<<grid, 64, 0, stream>>>(qkv, cs, sn, positions, seq_of_tok, page_table,
+    rope_kvwrite_kernel<bf16, true><<<grid, 64, 0, stream>>>(qkv, cs, sn, positions, seq_of_tok, page_table,
                                                        pt_stride, (bf16*)q_out, (bf16*)kcache,
                                                        (bf16*)vcache, nh, nk, hd, write_kv);
   else
-    rope_kvwrite_kernel<float><<<grid, 64, 0, stream>>>(qkv, cs, sn, positions, seq_of_tok, page_table,
+    rope_kvwrite_kernel<float, false><<<grid, 64, 0, stream>>>(qkv, cs, sn, positions, seq_of_tok, page_table,
                                                         pt_stride, (float*)q_out, (float*)kcache,
                                                         (float*)vcache, nh, nk, hd, write_kv);
   return mf_launch_status();

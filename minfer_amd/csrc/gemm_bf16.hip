@@ -378,11 +378,19 @@ __global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restric
         ad[s] = load8_inside(A, lda, m_row, k0 + s * 32 + kq);
       }
     } else {
+      // the slice's last batch: whole steps still go unguarded, the rest is guarded or zero
 #pragma unroll
       for (int s = 0; s < S; ++s) {
+        const int k = k0 + s * 32;
+        if (VEC && k + 32 <= k_end) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j) wd[j][s] = load8<VEC>(W, ldw, n_ld[j], k0 + s * 32 + kq, k_end);
-        ad[s] = load8<VEC>(A, lda, m_row, k0 + s * 32 + kq, k_end);
+          for (int j = 0; j < NT; ++j) wd[j][s] = load8_inside(W, ldw, n_ld[j], k + kq);
+          ad[s] = load8_inside(A, lda, m_row, k + kq);
+        } else {
+#pragma unroll
+          for (int j = 0; j < NT; ++j) wd[j][s] = load8<VEC>(W, ldw, n_ld[j], k + kq, k_end);
+          ad[s] = load8<VEC>(A, lda, m_row, k + kq, k_end);
+        }
       }
     }
   };
@@ -444,10 +452,136 @@ __global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restric
   }
 }
 
+// The same split of the work as skinny16_kernel (a block owns 16 NT weight rows, its waves split
+// K), for aligned operands and K a multiple of 32, with the loads rolling: a wave holds S steps
+// of weights and activations in registers, and the refill of a register is issued right behind
+// the MFMA that read it, so S steps of loads stay in flight the whole time in half the
+// registers of the two-buffer scheme above.  With K of many thousands and few weight rows
+// (the down projection) the chip is filled by loads in flight, not by blocks, and this is
+// what the time depends on.
+template <int NW, int NT, int S, bool PAIR>
+__global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restrict__ A, int lda,
+                                                            const bf16* __restrict__ W, int ldw,
+                                                            const float* __restrict__ bias,
+                                                            void* __restrict__ C, int ldc, int M, int N,
+                                                            int K, int steps_per_wave, int epi) {
+  constexpr int COLS = 16 * NT;
+  constexpr int RS = COLS + 4;
+  __shared__ float red[NW][16][RS];
+  const int lane = threadIdx.x & 63;
+  const int wid = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // the same in the whole wave
+  const int r16 = lane & 15;
+  auto tile_row = [&](int j) {
+    return PAIR ? (blockIdx.x >> 1) * 64 + (blockIdx.x & 1) * 16 + j * 32 : (blockIdx.x * NT + j) * 16;
+  };
+  const int total = K / 32;
+  const int first = min(wid * steps_per_wave, total);
+  const int T = min(steps_per_wave, total - first);       // steps of this wave
+  const int kq = first * 32 + (lane >> 4) * 8;
+  const bf16* arow = A + (size_t)min(r16, M - 1) * lda + kq;
+  const bf16* wrow[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) wrow[j] = W + (size_t)min(tile_row(j) + r16, N - 1) * ldw + kq;
+  floatx4 acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int R = T / S, rem = T % S;
+  if (R == 0) {       // a slice shorter than the registers hold: step by step
+    for (int s = 0; s < T; ++s) {
+      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(arow + s * 32);
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            a1, *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32), acc[j], 0, 0, 0);
+    }
+  } else {
+    bf16x8 a[S], w[NT][S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      a[s] = *reinterpret_cast<const bf16x8*>(arow + s * 32);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32);
+    }
+    // rounds whose refills all exist: no branch in the body
+    int base = 0;
+    for (int i = 0; i + 1 < R; ++i, base += S) {
+#pragma unroll
+      for (int s = 0; s < S; ++s) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s], w[j][s], acc[j], 0, 0, 0);
+          w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + (base + S + s) * 32);
+        }
+        a[s] = *reinterpret_cast<const bf16x8*>(arow + (base + S + s) * 32);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // the last whole round refills only what the remainder needs
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s], w[j][s], acc[j], 0, 0, 0);
+      if (s < rem) {
+        a[s] = *reinterpret_cast<const bf16x8*>(arow + (base + S + s) * 32);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + (base + S + s) * 32);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      if (s < rem) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s], w[j][s], acc[j], 0, 0, 0);
+      }
+    }
+  }
+  // D[m][n]: n = lane % 16, m = 4 (lane / 16) + r
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wid][(lane >> 4) * 4 + r][j * 16 + r16] = acc[j][r];
+  __syncthreads();
+  if (wid != 0) return;
+  if (epi == EPI_SWIGLU) {
+    if constexpr (PAIR && NT == 2) {
+      const int col = blockIdx.x * 16 + r16;
+      if (col < ldc) {
+        for (int m = lane >> 4; m < M; m += 4) {
+          float g = 0.f, u = 0.f;
+#pragma unroll
+          for (int ww = 0; ww < NW; ++ww) { g += red[ww][m][r16]; u += red[ww][m][16 + r16]; }
+          ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(g, u);
+        }
+      }
+    }
+    return;
+  }
+  const int c = lane % COLS;
+  const int n = tile_row(c >> 4) + (c & 15);
+  if (n >= N) return;
+  const float b = bias ? bias[n] : 0.f;
+  for (int m = lane / COLS; m < M; m += 64 / COLS) {
+    float v = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) v += red[ww][m][c];
+    store_out(C, ldc, m, n, v + b, epi);
+  }
+}
+
+template <int NW, int NT, int S, bool PAIR = false>
+int launch_rolling16(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
+                     int M, int N, int K, int epi, hipStream_t stream) {
+  const int steps_per_wave = (K / 32 + NW - 1) / NW;
+  const int blocks = PAIR ? N / 32 : (N + 16 * NT - 1) / (16 * NT);
+  rolling16_kernel<NW, NT, S, PAIR><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K,
+                                                                    steps_per_wave, epi);
+  return mf_launch_status();
+}
+
 template <int NW, int NT, int S, bool PAIR = false>
 int launch_skinny16(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
                     int M, int N, int K, int epi, int vec_ok, hipStream_t stream) {
-  const int k_per_wave = ((K + NW - 1) / NW + S * 32 - 1) / (S * 32) * (S * 32);
+  const int k_per_wave = ((K + NW - 1) / NW + 31) / 32 * 32;      // even shares; a slice's last batch may be short
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
   if (vec_ok)
     skinny16_kernel<NW, NT, S, true, PAIR><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
@@ -466,24 +600,34 @@ int launch_skinny16(const bf16* A, int lda, const bf16* W, int ldw, const float*
 // barrier per item) and the waves take turns at adding them and running the epilogue.
 // Against the kernel above this removes the per-tile re-read of the activations (which
 // cost a quarter of the time at 8 rows) and the start-up of a block per tile.
-template <int NS, int NT, bool PAIR>
-__global__ __launch_bounds__(512) void stationary16_kernel(const bf16* __restrict__ A, int lda,
+//
+// NORM: the activations are rows of the 32-bit residual stream, to be RMS-normalised on the way
+// in (y = x / sqrt(mean(x^2) + eps) * g, src/vec_ops.rs:500-522).  The 1 / sqrt(..) is one
+// number per row, so it can wait for the epilogue: the matrix cores get bf16(x * g), every
+// wave sums x^2 over its own slice of K while it converts, and the epilogue multiplies the
+// row's sums by 1 / sqrt(total / K + eps).  No pass over the row beforehand, no kernel and no
+// activation buffer between the norm and the product.
+struct NormArgs {
+  const float* g;          // [K] norm weight
+  const int* row_idx;      // activation row m is residual row row_idx[m] (null: m)
+  float eps;
+};
+
+template <int NS, int NT, bool PAIR, bool NORM>
+__global__ __launch_bounds__(512) void stationary16_kernel(const void* __restrict__ Av, int lda,
                                                            const bf16* __restrict__ W, int ldw,
                                                            const float* __restrict__ bias,
                                                            void* __restrict__ C, int ldc, int M, int N,
-                                                           int n_items, int epi) {
+                                                           int n_items, int epi, NormArgs norm) {
   constexpr int NW = 8;
   constexpr int COLS = 16 * NT;            // weight rows (output columns) of an item
   constexpr int RS = COLS + 4;             // row stride of the sums in LDS: conflict-free writes
   __shared__ float red[2][NW][16][RS];     // [buffer][wave][activation row][weight row of the item]
+  __shared__ float ssq[NW][16];            // NORM: sum of x^2 over a wave's slice, per activation row
+  __shared__ __attribute__((aligned(16))) float gs[NORM ? NW * NS * 32 : 4];   // NORM: the norm's weight
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int r16 = lane & 15;
   const int k0 = wid * NS * 32 + (lane >> 4) * 8;         // this lane's k in step 0 of its slice
-  const bf16* arow = A + (size_t)min(r16, M - 1) * lda + k0;
-  bf16x8 afr[NS];
-#pragma unroll
-  for (int s = 0; s < NS; ++s) afr[s] = *reinterpret_cast<const bf16x8*>(arow + s * 32);
-
   // first weight row of tile j of an item (before the lane's own row is added)
   auto tile_row = [&](int item, int j) {
     return PAIR ? (item >> 1) * 64 + (item & 1) * 16 + j * 32 : (item * NT + j) * 16;
@@ -491,21 +635,77 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const bf16* __restric
   bf16x8 w[NT][NS];
   const bf16* wrow[NT];
   int item = blockIdx.x;
+  auto first_loads = [&](int j) {
+    wrow[j] = W + (size_t)min(tile_row(item, j) + r16, N - 1) * ldw + k0;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32);
+  };
+  bf16x8 afr[NS];
+  float ss = 0.f;
+  if constexpr (NORM) {
+    // Everything the prologue needs is asked for at once, oldest first in the order it is
+    // used: the norm's weight (staged in LDS for all waves), this lane's x, and the first
+    // item's tile 0, which keeps HBM at work while the activations are converted.  The order is
+    // pinned: left alone, the compiler asks for the weights first and then waits for them
+    // before it stages g.
+    static_assert(NW * NS * 32 <= 2 * NW * 64 * 4, "two float4 of g per thread cover K");
+    const int ge0 = min((int)threadIdx.x * 4, NW * NS * 32 - 4);                 // the last ones twice
+    const int ge1 = min((NW * 64 + (int)threadIdx.x) * 4, NW * NS * 32 - 4);
+    const float4 gt0 = *reinterpret_cast<const float4*>(norm.g + ge0);
+    const float4 gt1 = *reinterpret_cast<const float4*>(norm.g + ge1);
+    const int m_src = min(r16, M - 1);
+    const float* xrow = (const float*)Av + (size_t)(norm.row_idx ? norm.row_idx[m_src] : m_src) * lda + k0;
+    float4 x[NS][2];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      x[s][0] = *reinterpret_cast<const float4*>(xrow + s * 32);
+      x[s][1] = *reinterpret_cast<const float4*>(xrow + s * 32 + 4);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (item < n_items) first_loads(0);
+    __builtin_amdgcn_sched_barrier(0);
+    *reinterpret_cast<float4*>(&gs[ge0]) = gt0;
+    *reinterpret_cast<float4*>(&gs[ge1]) = gt1;
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const float4 x0 = x[s][0], x1 = x[s][1];
+      const float4 g0 = *reinterpret_cast<const float4*>(&gs[k0 + s * 32]);
+      const float4 g1 = *reinterpret_cast<const float4*>(&gs[k0 + s * 32 + 4]);
+      ss = fmaf(x0.x, x0.x, ss); ss = fmaf(x0.y, x0.y, ss); ss = fmaf(x0.z, x0.z, ss); ss = fmaf(x0.w, x0.w, ss);
+      ss = fmaf(x1.x, x1.x, ss); ss = fmaf(x1.y, x1.y, ss); ss = fmaf(x1.z, x1.z, ss); ss = fmaf(x1.w, x1.w, ss);
+      afr[s][0] = (bf16)(x0.x * g0.x); afr[s][1] = (bf16)(x0.y * g0.y);
+      afr[s][2] = (bf16)(x0.z * g0.z); afr[s][3] = (bf16)(x0.w * g0.w);
+      afr[s][4] = (bf16)(x1.x * g1.x); afr[s][5] = (bf16)(x1.y * g1.y);
+      afr[s][6] = (bf16)(x1.z * g1.z); afr[s][7] = (bf16)(x1.w * g1.w);
+      // the packed value is wanted here and now (left alone, the compiler keeps x and g
+      // alive and converts in front of the first MFMA, at twice the registers)
+      asm volatile("" : "+v"(afr[s]));
+    }
+    ss += __shfl_xor(ss, 16);
+    ss += __shfl_xor(ss, 32);
+    if (lane < 16) ssq[wid][lane] = ss;    // read behind the first item's barrier
+    __builtin_amdgcn_sched_barrier(0);
+  } else {
+    const bf16* arow = (const bf16*)Av + (size_t)min(r16, M - 1) * lda + k0;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) afr[s] = *reinterpret_cast<const bf16x8*>(arow + s * 32);
+    if (item < n_items) first_loads(0);
+  }
   if (item < n_items) {
 #pragma unroll
-    for (int j = 0; j < NT; ++j) {
-      wrow[j] = W + (size_t)min(tile_row(item, j) + r16, N - 1) * ldw + k0;
-#pragma unroll
-      for (int s = 0; s < NS; ++s) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32);
-    }
+    for (int j = 1; j < NT; ++j) first_loads(j);
   }
   for (int it = 0; item < n_items; item += gridDim.x, ++it) {
+    // The loop body has no branch, so that the compiler can count the loads in flight and wait
+    // for the oldest one only: behind the last item the loads go to the head of the matrix,
+    // the same few lines for every lane, and their values are dropped.
     const int next = item + gridDim.x;
     const bool has_next = next < n_items;
-    if (has_next) {
 #pragma unroll
-      for (int j = 0; j < NT; ++j) wrow[j] = W + (size_t)min(tile_row(next, j) + r16, N - 1) * ldw + k0;
-    }
+    for (int j = 0; j < NT; ++j)
+      wrow[j] = W + (has_next ? (size_t)min(tile_row(next, j) + r16, N - 1) * ldw : (size_t)0) + k0;
     floatx4 acc[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -514,7 +714,8 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const bf16* __restric
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
         acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afr[s], w[j][s], acc[j], 0, 0, 0);
-        if (has_next) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32);
+        w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32);
+        __builtin_amdgcn_sched_barrier(0);      // keep "use a register, then refill it" in this order
       }
     }
     // D[m][n]: n = lane % 16, m = 4 (lane / 16) + r
@@ -527,6 +728,12 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const bf16* __restric
     // The buffer is written again two items on, behind the next barrier, which this wave
     // reaches only after it has read its sums here.
     if (wid != (it & (NW - 1))) continue;
+    auto row_scale = [&](int m) {          // NORM: 1 / sqrt(mean(x^2) + eps) of activation row m
+      float t = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < NW; ++ww) t += ssq[ww][m];
+      return 1.0f / sqrtf(t / (float)(NW * NS * 32) + norm.eps);
+    };
     if (epi == EPI_SWIGLU) {
       if constexpr (PAIR && NT == 2) {
         const int col = item * 16 + r16;
@@ -535,6 +742,11 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const bf16* __restric
             float g = 0.f, u = 0.f;
 #pragma unroll
             for (int ww = 0; ww < NW; ++ww) { g += red[buf][ww][m][r16]; u += red[buf][ww][m][16 + r16]; }
+            if constexpr (NORM) {
+              const float sc = row_scale(m);
+              g *= sc;
+              u *= sc;
+            }
             ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(g, u);
           }
         }
@@ -550,6 +762,7 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const bf16* __restric
       float v = 0.f;
 #pragma unroll
       for (int ww = 0; ww < NW; ++ww) v += red[buf][ww][m][c];
+      if constexpr (NORM) v *= row_scale(m);
       store_out(C, ldc, m, n, v + b, epi);
     }
   }
@@ -557,8 +770,8 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const bf16* __restric
 
 // true when the shape is one the register-resident kernel is built for
 template <int NS, int NT, bool PAIR>
-int launch_stationary16(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
-                        int M, int N, int epi, hipStream_t stream) {
+int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
+                        int M, int N, int epi, const NormArgs* norm, hipStream_t stream) {
   const int n_items = PAIR ? N / 32 : (N + 16 * NT - 1) / (16 * NT);
   static int n_cu = 0;
   if (n_cu == 0) {
@@ -568,7 +781,12 @@ int launch_stationary16(const bf16* A, int lda, const bf16* W, int ldw, const fl
     n_cu = prop.multiProcessorCount;
   }
   const int grid = n_items < n_cu ? n_items : n_cu;
-  stationary16_kernel<NS, NT, PAIR><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, n_items, epi);
+  if (norm)
+    stationary16_kernel<NS, NT, PAIR, true><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, n_items,
+                                                                      epi, *norm);
+  else
+    stationary16_kernel<NS, NT, PAIR, false><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, n_items,
+                                                                       epi, NormArgs{nullptr, nullptr, 0.f});
   return mf_launch_status();
 }
 
@@ -662,6 +880,29 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
   return (int)hipErrorInvalidValue;
 }
 
+// The register-resident kernel for the shapes it is built for (K = 256 NS with enough tiles to
+// go round); MF_NOT_BUILT for any other, and nothing is launched.
+constexpr int MF_NOT_BUILT = -2;
+static int stationary16(const void* a, int lda, const bf16* w, int ldw, const float* bias, void* C, int ldc, int M,
+                 int N, int K, int epi, const NormArgs* norm, hipStream_t stream) {
+  static const int off = getenv("MF_NO_STATIONARY") ? 1 : 0;
+  if (off || M > 16 || K % 256 != 0 || (N + 15) / 16 < 128) return MF_NOT_BUILT;
+  if (epi == EPI_SWIGLU && N % 64 != 0) return MF_NOT_BUILT;
+  // two tiles an item where there are enough of them: 128-byte rows of 32-bit output
+  const bool two = (N + 31) / 32 >= 128;
+#define MF_STATIONARY(NS_)                                                                                  \
+  case NS_:                                                                                                 \
+    return epi == EPI_SWIGLU                                                                                \
+               ? launch_stationary16<NS_, 2, true>(a, lda, w, ldw, bias, C, ldc, M, N, epi, norm, stream)   \
+           : two ? launch_stationary16<NS_, 2, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, norm, stream) \
+                 : launch_stationary16<NS_, 1, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, norm, stream);
+  switch (K / 256) {
+    MF_STATIONARY(6) MF_STATIONARY(8) MF_STATIONARY(14) MF_STATIONARY(16)
+  }
+#undef MF_STATIONARY
+  return MF_NOT_BUILT;
+}
+
 // M <= 64.  `part` holds splits*M*N floats when splits > 1; k_per_split is a multiple of 256.
 MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, const float* bias,
                                void* C, int ldc, float* part, int M, int N, int K, int splits,
@@ -683,22 +924,20 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
     // Measured at 3584..152064 weight rows: many rows -> 4 waves with two 16-row tiles each
     // (less activation traffic per weight byte); a row count that would leave a short second
     // round of 16-row blocks -> 8 waves with two tiles; otherwise 8 waves, one tile.
-    // K = 256 NS with enough tiles to go round: the register-resident kernel
-    static const int stationary = getenv("MF_NO_STATIONARY") ? 0 : 1;
-    if (stationary && vec_ok && K % 256 == 0 && (N + 15) / 16 >= 128) {
-      // two tiles an item where there are enough of them: 128-byte rows of 32-bit output
-      static const int nt_env = getenv("MF_STATIONARY_NT") ? atoi(getenv("MF_STATIONARY_NT")) : 0;
-      const bool two = nt_env ? nt_env == 2 : (N + 31) / 32 >= 128;
-#define MF_STATIONARY(NS_)                                                                                  \
-  case NS_:                                                                                                 \
-    return epi == EPI_SWIGLU                                                                                \
-               ? launch_stationary16<NS_, 2, true>(a, lda, w, ldw, bias, C, ldc, M, N, epi, stream)         \
-           : two ? launch_stationary16<NS_, 2, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, stream)      \
-                 : launch_stationary16<NS_, 1, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, stream);
-      switch (K / 256) {
-        MF_STATIONARY(6) MF_STATIONARY(8) MF_STATIONARY(14) MF_STATIONARY(16)
+    if (vec_ok) {
+      const int rc = stationary16(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, nullptr, stream);
+      if (rc != MF_NOT_BUILT) return rc;
+    }
+    static const int rolling = getenv("MF_ROLLING16") ? atoi(getenv("MF_ROLLING16")) : 1;
+    if (rolling && vec_ok && K % 32 == 0 && epi != EPI_SWIGLU) {
+      switch (rolling) {
+        case 1: return launch_rolling16<8, 1, 16>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+        case 2: return launch_rolling16<8, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+        case 3: return launch_rolling16<16, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+        case 4: return launch_rolling16<8, 2, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+        case 5: return launch_rolling16<16, 1, 12>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+        case 6: return launch_rolling16<8, 1, 24>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
       }
-#undef MF_STATIONARY
     }
     if (epi == EPI_SWIGLU)
       return launch_skinny16<4, 2, 4, true>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
@@ -717,4 +956,19 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
     case 4: return launch_skinny<4>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
   }
   return (int)hipErrorInvalidValue;
+}
+
+// RMS norm of rows of the 32-bit residual stream x (row m of the product is x[row_idx[m]]), then
+// the product with W, in one kernel.  Returns MF_NOT_BUILT (-2), having launched nothing, for
+// shapes the register-resident kernel does not cover: the caller then runs the norm and the
+// product one after the other.
+MF_API int mf_gemm_bf16_normed(const float* x, int ldx, const int* row_idx, const float* g, float eps,
+                               const void* W, int ldw, const float* bias, void* C, int ldc, int M, int N, int K,
+                               int epi, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || epi < 0 || epi > EPI_SWIGLU) return (int)hipErrorInvalidValue;
+  if (ldx % 4 != 0 || ldw % 8 != 0 || (uintptr_t)x % 16 != 0 || (uintptr_t)g % 16 != 0 || (uintptr_t)W % 16 != 0)
+    return MF_NOT_BUILT;
+  const NormArgs norm{g, row_idx, eps};
+  return stationary16(x, ldx, (const bf16*)W, ldw, bias, C, ldc, M, N, K, epi, &norm, stream);
 }

@@ -13,7 +13,7 @@ from typing import Callable, Dict, List, Optional
 import torch
 
 from ..kernels import ops
-from ..parts.base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Runtime, make_part)
+from ..parts.base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Normed, Runtime, make_part)
 from ..parts.linear import Linear
 from ..parts.spec import BlockSpec, ModelSpec
 from ..weights.loader import TensorSpec
@@ -97,8 +97,7 @@ class DecoderModel:
             kept = torch.empty((rows.numel(), s.hidden_size), dtype=torch.float32, device=h.device)
             ops.gather_rows(h, rows, kept)
             h = kept
-        x = self.final_norm.forward(h)
-        return self.head(x, out_dtype=torch.float32)
+        return self.head(Normed(self.final_norm, h), out_dtype=torch.float32)
 
 
 def expected_tensors(spec: ModelSpec) -> Dict[str, TensorSpec]:

@@ -26,12 +26,12 @@ LIBRARIES: Dict[str, str] = {
     "gemm_f32": "gemm_f32.hip",
     "gemm_bf16": "gemm_bf16.hip",
     "attn_tokens_f32": "attn_tokens_f32.hip",
-    "attn_tokens_bf16": "attn_tokens_bf16.hip",
+    "attn_decode_bf16": "attn_decode_bf16.hip",
     "attn_prefill_bf16": "attn_prefill_bf16.hip",
     "sampling": "sampling.hip",
 }
 HEADERS = {"attn_tokens_f32": ["common.h", "attn_tokens_impl.h"],
-           "attn_tokens_bf16": ["common.h", "attn_tokens_impl.h"]}
+           "attn_decode_bf16": ["common.h", "attn_tokens_impl.h"]}
 
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-shared", "-std=c++17",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -5,6 +5,8 @@ cached workspaces below.
 """
 from __future__ import annotations
 
+import os
+
 import ctypes
 from ctypes import c_double, c_float, c_int, c_size_t, c_uint64, c_void_p
 from typing import Dict, Optional, Tuple
@@ -12,6 +14,7 @@ from typing import Dict, Optional, Tuple
 import torch
 
 from . import build
+from ..cache.paged import v_page_shape
 
 PAGE = 64          # tokens per cache page (MF_PAGE in csrc/common.h)
 HAVE_PREFILL_ATTENTION = True
@@ -43,14 +46,16 @@ _PROTOTYPES = {
         "mf_gemm_bf16": [_P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_gemm_bf16_skinny": [_P, c_int, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int,
                                 c_int, c_int, _P],
+        "mf_gemm_bf16_normed": [_P, c_int, _P, _P, c_float, _P, c_int, _P, _P, c_int, c_int, c_int, c_int,
+                                c_int, _P],
     },
     "attn_tokens_f32": {
         "mf_attn_tokens_f32": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
                                c_float, c_int, c_int, c_int, _P],
     },
-    "attn_tokens_bf16": {
-        "mf_attn_tokens_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
-                                c_float, c_int, c_int, c_int, _P],
+    "attn_decode_bf16": {
+        "mf_attn_decode_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
+                                c_float, c_int, c_int, _P],
     },
     "attn_prefill_bf16": {
         "mf_attn_prefill_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int,
@@ -201,6 +206,8 @@ def rope_kvwrite(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positi
                  seq_of_tok: torch.Tensor, page_table: torch.Tensor, q_out: torch.Tensor,
                  kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor], n_heads: int,
                  n_kv_heads: int, head_dim: int, write_kv: bool = True) -> None:
+    """Rotates q and k, and stores k and v of the tokens at their positions in the cache pages
+    (`v_page_shape` says how V lies in a page)."""
     n_tok = positions.numel()
     _need(qkv, "rope.qkv", torch.float32, (n_tok, (n_heads + 2 * n_kv_heads) * head_dim))
     _need(cos, "rope.cos", torch.float32)
@@ -212,10 +219,7 @@ def rope_kvwrite(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positi
     _need(page_table, "rope.page_table", torch.int32)
     _need(q_out, "rope.q_out", _FLOATS, (n_tok, n_heads * head_dim))
     if write_kv:
-        for name, c in (("rope.kcache", kcache), ("rope.vcache", vcache)):
-            _need(c, name, q_out.dtype)
-            if tuple(c.shape[1:]) != (n_kv_heads, PAGE, head_dim):
-                raise KernelError(f"{name}: shape {tuple(c.shape)}, expected [pages, {n_kv_heads}, {PAGE}, {head_dim}]")
+        _need_caches("rope", kcache, vcache, q_out.dtype, n_kv_heads, head_dim)
     _check(_fn("elementwise", "mf_rope_kvwrite")(
         _ptr(qkv), _ptr(cos), _ptr(sin), _ptr(positions), _ptr(seq_of_tok), _ptr(page_table),
         page_table.shape[1], _ptr(q_out), _ptr(kcache if write_kv else None),
@@ -306,6 +310,54 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, vari
                                              EPI_SWIGLU, variant, _stream()), "gemm_bf16(swiglu)")
 
 
+NOT_BUILT = -2      # an entry point's answer for a shape it has no kernel for; nothing was launched
+
+
+def linear_normed(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, row_idx: Optional[torch.Tensor],
+                  weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                  accumulate: bool = False, swiglu: bool = False) -> bool:
+    """out (+)= rmsnorm(x[row_idx]) @ weight^T (+ bias) in one kernel, for the few-row shapes
+    the register-resident decode product covers; with `swiglu`, `weight` is
+    `interleave_gate_up(Wg, Wu)` and out = silu(gate) * up.  x is the float32 residual stream,
+    weight bfloat16.  Returns False, having done nothing, when there is no such kernel for
+    the shape: the caller then norms and multiplies in two steps."""
+    _need(x, "linear_normed.x", torch.float32)
+    _need(weight, "linear_normed.weight", torch.bfloat16)
+    k = x.shape[1]
+    n = weight.shape[0]
+    m = x.shape[0] if row_idx is None else row_idx.numel()
+    if weight.shape[1] != k:
+        raise KernelError(f"linear_normed: x is {tuple(x.shape)}, weight is {tuple(weight.shape)}")
+    _need(norm_weight, "linear_normed.norm_weight", torch.float32, (k,))
+    if row_idx is not None:
+        _need(row_idx, "linear_normed.row_idx", torch.int32)
+    if bias is not None:
+        _need(bias, "linear_normed.bias", torch.float32, (n,))
+    if swiglu:
+        nf = out.shape[1]
+        if n % 64 or not n // 2 - 32 < nf <= n // 2 or bias is not None or accumulate:
+            raise KernelError(f"linear_normed(swiglu): weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+        _need(out, "linear_normed.out", torch.bfloat16, (m, nf))
+        epi, ldc = EPI_SWIGLU, nf
+    else:
+        _need(out, "linear_normed.out", _FLOATS, (m, n))
+        if accumulate and out.dtype != torch.float32:
+            raise KernelError("linear_normed: accumulation needs a float32 output")
+        epi = EPI_BF16 if out.dtype == torch.bfloat16 else (EPI_ACC_F32 if accumulate else EPI_F32)
+        ldc = n
+    if m == 0:
+        return True
+    if m > 16 or os.environ.get("MF_NO_FOLD"):
+        return False
+    rc = _fn("gemm_bf16", "mf_gemm_bf16_normed")(_ptr(x), k, _ptr(row_idx), _ptr(norm_weight), float(eps),
+                                                 _ptr(weight), k, _ptr(bias), _ptr(out), ldc, m, n, k, epi,
+                                                 _stream())
+    if rc == NOT_BUILT:
+        return False
+    _check(rc, "gemm_bf16_normed")
+    return True
+
+
 # ------------------------------------------------------------------ attention
 def split_plan(n_tok: int, n_kv_heads: int, group: int, head_dim: int, max_len: int,
                target_blocks: int = 1024) -> Tuple[int, int]:
@@ -319,18 +371,37 @@ def split_plan(n_tok: int, n_kv_heads: int, group: int, head_dim: int, max_len: 
     return (max_len + split_len - 1) // split_len, split_len
 
 
+def _need_caches(what: str, kcache: torch.Tensor, vcache: torch.Tensor, dtype, n_kv_heads: int,
+                 head_dim: int) -> None:
+    _need(kcache, what + ".kcache", dtype)
+    _need(vcache, what + ".vcache", dtype)
+    if tuple(kcache.shape[1:]) != (n_kv_heads, PAGE, head_dim):
+        raise KernelError(f"{what}.kcache: shape {tuple(kcache.shape)}, expected "
+                          f"[pages, {n_kv_heads}, {PAGE}, {head_dim}]")
+    want = v_page_shape(n_kv_heads, head_dim, dtype)
+    if tuple(vcache.shape[1:]) != want or vcache.shape[0] != kcache.shape[0]:
+        raise KernelError(f"{what}.vcache: shape {tuple(vcache.shape)}, expected "
+                          f"[{kcache.shape[0]}, {want[0]}, {want[1]}, {want[2]}]")
+
+
+def decode_split_plan(n_tok: int, n_kv_heads: int, group: int, max_len: int, target_blocks: int = 512) -> int:
+    """Key splits of the bfloat16 decode attention: enough blocks to fill the chip, at least
+    128 keys of the longest possible sequence per split, at most 64.  The kernel divides each
+    token's own length by this number, so every split has work."""
+    blocks = n_tok * n_kv_heads * ((group + 15) // 16)
+    return max(1, min(target_blocks // max(1, blocks), (max_len + 127) // 128, 64))
+
+
 def attn_tokens(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
                 positions: torch.Tensor, seq_of_tok: torch.Tensor, out: torch.Tensor, n_heads: int,
                 n_kv_heads: int, head_dim: int, scale: float, window: int, max_len: int) -> None:
     """Each query token attends to its sequence's cache rows lo..position.  `max_len` bounds
-    position + 1 for every token (it only shapes the launch)."""
+    position + 1 for every token (it only shapes the launch).  bfloat16 runs on the matrix
+    cores, 32-bit on plain FMA."""
     n_tok = positions.numel()
     _need(q, "attn.q", _FLOATS, (n_tok, n_heads * head_dim))
     _need(out, "attn.out", q.dtype, (n_tok, n_heads * head_dim))
-    for name, c in (("attn.kcache", kcache), ("attn.vcache", vcache)):
-        _need(c, name, q.dtype)
-        if tuple(c.shape[1:]) != (n_kv_heads, PAGE, head_dim):
-            raise KernelError(f"{name}: shape {tuple(c.shape)}, expected [pages, {n_kv_heads}, {PAGE}, {head_dim}]")
+    _need_caches("attn", kcache, vcache, q.dtype, n_kv_heads, head_dim)
     _need(page_table, "attn.page_table", torch.int32)
     _need(positions, "attn.positions", torch.int32, (n_tok,))
     _need(seq_of_tok, "attn.seq_of_tok", torch.int32, (n_tok,))
@@ -340,13 +411,20 @@ def attn_tokens(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
         raise KernelError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
     if max_len > page_table.shape[1] * PAGE:
         raise KernelError(f"attention: max_len {max_len} exceeds the page table ({page_table.shape[1]} pages)")
+    if q.dtype == torch.bfloat16:
+        n_splits = decode_split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, max_len)
+        part = workspace("attn", n_tok * n_heads * n_splits * (head_dim + 2), q.device) if n_splits > 1 else None
+        _check(_fn("attn_decode_bf16", "mf_attn_decode_bf16")(
+            _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions),
+            _ptr(seq_of_tok), _ptr(out), _ptr(part), n_tok, n_heads, n_kv_heads, head_dim, float(scale),
+            int(window or 0), n_splits, _stream()), "attn_decode_bf16")
+        return
     n_splits, split_len = split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, head_dim, max_len)
     part = workspace("attn", n_tok * n_heads * n_splits * (head_dim + 2), q.device) if n_splits > 1 else None
-    name = "attn_tokens_bf16" if q.dtype == torch.bfloat16 else "attn_tokens_f32"
-    _check(_fn(name, "mf_" + name)(
+    _check(_fn("attn_tokens_f32", "mf_attn_tokens_f32")(
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions),
         _ptr(seq_of_tok), _ptr(out), _ptr(part), n_tok, n_heads, n_kv_heads, head_dim, float(scale),
-        int(window or 0), n_splits, split_len, _stream()), name)
+        int(window or 0), n_splits, split_len, _stream()), "attn_tokens_f32")
 
 
 def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
@@ -358,10 +436,7 @@ def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pa
     n_tok = ctx.n_tokens
     _need(q, "attn_prefill.q", torch.bfloat16, (n_tok, n_heads * head_dim))
     _need(out, "attn_prefill.out", torch.bfloat16, (n_tok, n_heads * head_dim))
-    for name, c in (("attn_prefill.kcache", kcache), ("attn_prefill.vcache", vcache)):
-        _need(c, name, torch.bfloat16)
-        if tuple(c.shape[1:]) != (n_kv_heads, PAGE, head_dim):
-            raise KernelError(f"{name}: shape {tuple(c.shape)}, expected [pages, {n_kv_heads}, {PAGE}, {head_dim}]")
+    _need_caches("attn_prefill", kcache, vcache, torch.bfloat16, n_kv_heads, head_dim)
     _need(page_table, "attn_prefill.page_table", torch.int32)
     _need(ctx.cu_seqlens, "attn_prefill.cu_seqlens", torch.int32, (ctx.n_seqs + 1,))
     _need(ctx.start_pos, "attn_prefill.start_pos", torch.int32, (ctx.n_seqs,))

@@ -65,6 +65,8 @@ class GQAttention(Mixer):
     def prepare(self, max_len: int) -> None:
         self.position.prepare(max_len)
 
+    takes_normed = True
+
     def forward(self, x, h, ctx, entry: int, writes_cache: bool) -> None:
         kc, vc, group = ctx.cache.kv(entry)
         table = ctx.page_table(group)

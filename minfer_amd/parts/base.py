@@ -55,6 +55,42 @@ class Norm(Part):
         """float32 rows in, run-type rows out; row r reads h[row_idx[r]] when given."""
         raise NotImplementedError
 
+    def rms_scale(self):
+        """(weight, eps) if this norm is y = x / sqrt(mean(x^2) + eps) * weight with a float32
+        weight vector, else None.  A product that follows such a norm may fold it in."""
+        return None
+
+
+class Normed:
+    """The rows `norm(h[row_idx])` before anyone has computed them.  A block hands this to a
+    mixer or feed-forward that declares `takes_normed = True`; such a part passes it to its
+    first `Linear`, which folds the norm into the product where a kernel for that exists, or
+    calls `tensor()` (computed once, then kept) like any part that needs the rows themselves."""
+
+    def __init__(self, norm: "Norm", h: torch.Tensor, row_idx: Optional[torch.Tensor] = None):
+        self.norm, self.h, self.row_idx = norm, h, row_idx
+        self._rows: Optional[torch.Tensor] = None
+
+    @property
+    def shape(self):
+        return (self.h.shape[0] if self.row_idx is None else self.row_idx.numel(), self.h.shape[1])
+
+    @property
+    def device(self):
+        return self.h.device
+
+    def tensor(self) -> torch.Tensor:
+        if self._rows is None:
+            self._rows = self.norm.forward(self.h, row_idx=self.row_idx)
+        return self._rows
+
+
+def normed_input(norm: "Norm", part, h: torch.Tensor, row_idx: Optional[torch.Tensor] = None):
+    """What a block gives `part` as its input: the lazy form if the part takes it."""
+    if getattr(part, "takes_normed", False):
+        return Normed(norm, h, row_idx)
+    return norm.forward(h, row_idx=row_idx)
+
 
 class PositionEncoding(Part):
     def rotate_and_store(self, qkv: torch.Tensor, ctx, q_out: torch.Tensor, kcache, vcache,
@@ -69,6 +105,8 @@ class Mixer(Part):
         """A `KVRequest`, a `StateRequest` or None."""
         return None
 
+    takes_normed = False     # True: `x` may arrive as a `Normed` (see there)
+
     def forward(self, x: torch.Tensor, h: torch.Tensor, ctx, entry: int, writes_cache: bool) -> None:
         """Adds the mixer's output for the step's tokens into h.  `entry` is the cache entry
         (`ctx.cache.kv(entry)` / `ctx.cache.state(entry)`)."""
@@ -76,6 +114,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    takes_normed = False     # True: `x` may arrive as a `Normed`
+
     def forward(self, x: torch.Tensor, h: torch.Tensor, ctx) -> None:
         """Adds the feed-forward's output into h (h may hold fewer rows than the step)."""
         raise NotImplementedError

@@ -8,18 +8,18 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import Block, register_block
+from .base import Block, normed_input, register_block
 
 
 @register_block("prenorm")
 class PreNormBlock(Block):
     def forward(self, h, ctx, entry: int, writes_cache: bool, keep_rows=None):
-        x = self.mixer_norm.forward(h)
+        x = normed_input(self.mixer_norm, self.mixer, h)
         self.mixer.forward(x, h, ctx, entry, writes_cache)
         if keep_rows is not None:
             kept = torch.empty((keep_rows.numel(), h.shape[1]), dtype=h.dtype, device=h.device)
             ops.gather_rows(h, keep_rows, kept)
             h = kept
-        x = self.feed_forward_norm.forward(h)
+        x = normed_input(self.feed_forward_norm, self.feed_forward, h)
         self.feed_forward.forward(x, h, ctx)
         return h

@@ -9,7 +9,7 @@ import torch
 
 from ..kernels import ops
 from ..weights.loader import TensorSpec
-from .base import FeedForward, register_feed_forward
+from .base import FeedForward, Normed, register_feed_forward
 from .linear import Linear
 
 
@@ -39,10 +39,15 @@ class SwiGLU(FeedForward):
             self.gate_up = Linear.stacked([gate, up])
         self.down = Linear(get(n["down"] + ".weight"))
 
+    takes_normed = True
+
     def forward(self, x, h, ctx) -> None:
         y = torch.empty((x.shape[0], self.inter), dtype=self.rt.dtype, device=x.device)
         if self.fused is not None:
-            ops.linear_swiglu(x, self.fused, y)
+            fold = x.norm.rms_scale() if isinstance(x, Normed) else None
+            if fold is None or not ops.linear_normed(x.h, fold[0], fold[1], x.row_idx, self.fused, None, y,
+                                                     swiglu=True):
+                ops.linear_swiglu(x.tensor() if isinstance(x, Normed) else x, self.fused, y)
         else:
             ops.swiglu(self.gate_up(x, out_dtype=torch.float32), y)
         self.down(y, out=h, accumulate=True)

@@ -12,6 +12,7 @@ from typing import List, Optional
 import torch
 
 from ..kernels import ops
+from .base import Normed
 
 
 def common_matrix_dtype(tensors: List[torch.Tensor]) -> torch.dtype:
@@ -39,11 +40,17 @@ class Linear:
                            else x.to(torch.float32) for t, x in zip(weights, biases)])
         return cls(w, b)
 
-    def __call__(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
+    def __call__(self, x, out: Optional[torch.Tensor] = None,
                  out_dtype: torch.dtype = torch.float32, accumulate: bool = False) -> torch.Tensor:
         rows = x.shape[0]
         if out is None:
             out = torch.empty((rows, self.out_features), dtype=out_dtype, device=x.device)
+        if isinstance(x, Normed):
+            fold = x.norm.rms_scale() if self.weight.dtype == torch.bfloat16 else None
+            if fold is not None and ops.linear_normed(x.h, fold[0], fold[1], x.row_idx, self.weight, self.bias,
+                                                      out, accumulate=accumulate):
+                return out
+            x = x.tensor()
         if self.weight.dtype == torch.float32 and x.dtype != torch.float32:
             wide = torch.empty(x.shape, dtype=torch.float32, device=x.device)
             ops.convert(x, wide)

@@ -27,6 +27,9 @@ class RMSNorm(Norm):
     def load(self, get):
         self.weight = get(self.name).to(torch.float32).contiguous()
 
+    def rms_scale(self):
+        return self.weight, self.eps
+
     def forward(self, h, out: Optional[torch.Tensor] = None, row_idx: Optional[torch.Tensor] = None):
         rows = h.shape[0] if row_idx is None else row_idx.numel()
         if out is None:

@@ -27,6 +27,12 @@ def rmsnorm(x, weight, eps, out, row_idx=None):
     out.copy_(y.to(out.dtype))
 
 
+def rmsnorm_reference(x, weight, eps):
+    """The norm alone, float64, unrounded."""
+    s = x.double()
+    return s * (1.0 / torch.sqrt((s * s).mean(dim=-1, keepdim=True) + eps)) * weight.double()
+
+
 def gather_rows(x, idx, out):
     out.copy_(x[idx.long()])
 
@@ -73,7 +79,10 @@ def rope_kvwrite(qkv, cos, sin, positions, seq_of_tok, page_table, q_out, kcache
     page = page_table.long()[seq_of_tok.long(), pos // PAGE]
     assert (page >= 0).all(), "token written to a page that was not reserved"
     kcache[page, :, pos % PAGE, :] = k
-    vcache[page, :, pos % PAGE, :] = v
+    if v_transposed(vcache):
+        vcache[page, :, :, pos % PAGE] = v
+    else:
+        vcache[page, :, pos % PAGE, :] = v
 
 
 def linear(x, weight, bias, out, accumulate=False, variant=0):
@@ -104,11 +113,39 @@ def linear_swiglu(x, weight, out, variant=0):
     out.copy_((g / (1.0 + torch.exp(-g)) * u).to(out.dtype))
 
 
-def gather_cache_rows(cache, page_table_row, length):
+def linear_normed(x, norm_weight, eps, row_idx, weight, bias, out, accumulate=False, swiglu=False):
+    """The stand-in has no folded kernel: the caller norms and multiplies in two steps."""
+    return False
+
+
+def linear_normed_reference(x, norm_weight, eps, row_idx, weight, bias, swiglu=False):
+    """What the folded kernel computes, in float64, with its one rounding of the activations:
+    bf16(x * g) goes to the matrix cores and 1 / sqrt(mean(x^2) + eps) is applied to the sums."""
+    rows = x if row_idx is None else x[row_idx.long()]
+    a = (rows.float() * norm_weight.float()).to(torch.bfloat16).double()
+    inv = 1.0 / torch.sqrt((rows.double() ** 2).mean(dim=1, keepdim=True) + eps)
+    y = a @ weight.double().t() * inv
+    if bias is not None:
+        y = y + bias.double()
+    return y
+
+
+def v_transposed(vcache):
+    """A bfloat16 cache keeps a page of V as [kv_heads][head_dim][64], a 32-bit one as
+    [kv_heads][64][head_dim] (the product's `v_page_shape`)."""
+    return vcache.dtype == torch.bfloat16
+
+
+def v_rows(vcache, page, off):
+    """[n][kv_heads][head_dim] rows of V at (page[i], off[i])."""
+    return vcache[page, :, :, off] if v_transposed(vcache) else vcache[page, :, off, :]
+
+
+def gather_cache_rows(cache, page_table_row, length, is_v=False):
     """[length][kv_heads][head_dim] rows 0..length-1 of one sequence."""
     pos = torch.arange(length)
     page = page_table_row.long()[pos // PAGE]
-    return cache[page, :, pos % PAGE, :]
+    return v_rows(cache, page, pos % PAGE) if is_v else cache[page, :, pos % PAGE, :]
 
 
 def attn_tokens(q, kcache, vcache, page_table, positions, seq_of_tok, out, n_heads, n_kv_heads,
@@ -125,7 +162,7 @@ def attn_tokens(q, kcache, vcache, page_table, positions, seq_of_tok, out, n_hea
         page = row.long()[pos // PAGE]
         assert (page >= 0).all(), "attention reads a page that was given back"
         k = kcache[page, :, pos % PAGE, :].double()      # [n][nk][hd]
-        v = vcache[page, :, pos % PAGE, :].double()
+        v = v_rows(vcache, page, pos % PAGE).double()
         for h in range(n_heads):
             s = (k[:, h // g, :] @ qh[i, h]) * scale
             res[i, h] = torch.softmax(s, dim=0) @ v[:, h // g, :]
@@ -182,7 +219,7 @@ def advance(next_ids, sampled, positions, steps):
 
 NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", "rope_table",
          "rope_kvwrite", "linear", "attn_tokens", "attn_prefill", "argmax", "sample", "penalties",
-         "top_k", "top_p", "advance", "interleave_gate_up", "linear_swiglu"]
+         "top_k", "top_p", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed"]
 
 
 def install(monkeypatch):

@@ -117,9 +117,16 @@ def test_rope_table(ops, theta, half):
 
 
 def make_cache(n_pages, nk, hd, dtype, seed=0):
+    """K and V as [pages][kv_heads][64][head_dim]: for V this is the logical view, `stored_v`
+    gives what the kernels take."""
     k = rnd((n_pages, nk, 64, hd), dtype, seed)
     v = rnd((n_pages, nk, 64, hd), dtype, seed + 1)
     return k, v
+
+
+def stored_v(v):
+    """A bfloat16 cache keeps a page of V transposed, [kv_heads][head_dim][64]."""
+    return v.transpose(2, 3).contiguous() if v.dtype == torch.bfloat16 else v
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -133,6 +140,7 @@ def test_rope_kvwrite(ops, dtype, nh, nk, hd):
     qkv = rnd((t, (nh + 2 * nk) * hd), seed=6)
     cs, sn = plain_ops.rope_table(256, hd // 2, 1e4, 1.0, "cpu")
     kc, vc = make_cache(10, nk, hd, dtype, 7)
+    vc = stored_v(vc)
     q_ref = torch.empty(t, nh * hd, dtype=dtype)
     kr, vr = kc.clone(), vc.clone()
     plain_ops.rope_kvwrite(qkv, cs, sn, pos, seq, table, q_ref, kr, vr, nh, nk, hd)
@@ -258,7 +266,7 @@ def build_attention_case(nh, nk, hd, lengths, dtype, seed, n_pages_extra=3):
     pos = torch.tensor(pos, dtype=torch.int32)
     seq = torch.tensor(seq, dtype=torch.int32)
     q = rnd((pos.numel(), nh * hd), dtype, seed + 5)
-    return q, kc, vc, torch.from_numpy(table), pos, seq
+    return q, kc, stored_v(vc), torch.from_numpy(table), pos, seq
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -349,7 +357,7 @@ def prefill_case(nh, nk, hd, new, start, seed):
                            slot_ids=torch.zeros(len(new), dtype=torch.int32, device=dev), logit_rows=None,
                            page_tables={}, max_len=max(lengths), max_new=max(new), all_decode=False,
                            host_slots=list(range(len(new))), host_new=list(new), host_start=list(start))
-    return q, kc, vc, table, ctx_on
+    return q, kc, stored_v(vc), table, ctx_on
 
 
 @pytest.mark.parametrize("nh,nk,hd,window", [(4, 2, 16, 0), (4, 1, 32, 0), (9, 3, 48, 0), (28, 4, 128, 0),
@@ -389,7 +397,7 @@ def test_attn_prefill_far_key_and_window_edge(ops):
     qi, far = 650, 3
     page, row = int(table[0, far // 64]), far % 64
     kc[page, 0, row] = q[qi, :hd] * 4.0
-    vrow = vc[page, 0, row].float()
+    vrow = vc[page, 0, :, row].float()             # a bfloat16 page of V is [kv_heads][head_dim][64]
     for window, seen in ((0, True), (qi - far + 1, True), (qi - far, False)):
         out = torch.empty(q.shape, dtype=torch.bfloat16, device=DEV)
         ops.attn_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), ctx_on(DEV), out, nh, nk, hd, 1.0, window)
@@ -420,3 +428,64 @@ def test_gemm_bf16_swiglu(ops, variant, m, nf, k):
     again = torch.empty(m, nf, dtype=torch.bfloat16, device=DEV)
     ops.linear_swiglu(x.to(DEV), w, again, variant=variant)
     assert torch.equal(out, again)
+
+
+@pytest.mark.parametrize("m,n,k,idx", [(1, 2100, 1536, False), (5, 4608, 2048, True), (8, 4001, 3584, False),
+                                       (16, 2048, 4096, True), (3, 152064, 3584, True)])
+def test_gemm_bf16_normed(ops, m, n, k, idx):
+    """RMS norm folded into the few-row product: against the same formula in float64 with the
+    kernel's one rounding (tight), and against norm-then-product as the two kernels do it."""
+    h = rnd((m + 3, k), seed=40, scale=3.0)
+    h[0, 5] = 40.0                                    # one large element: the row's scale must see it
+    g = 1.0 + rnd((k,), seed=41, scale=0.2)
+    w, b = rnd((n, k), torch.bfloat16, 42, 0.05), rnd((n,), seed=43)
+    eps = 1e-5
+    row_idx = torch.tensor([(3 * i + 1) % (m + 3) for i in range(m)], dtype=torch.int32) if idx else None
+    src = h if idx else h[:m].contiguous()
+    ref = plain_ops.linear_normed_reference(src, g, eps, row_idx, w, b)
+    out = torch.empty(m, n, device=DEV)
+    done = ops.linear_normed(src.to(DEV), g.to(DEV), eps, None if row_idx is None else row_idx.to(DEV),
+                             w.to(DEV), b.to(DEV), out)
+    assert done, "this shape is one the folded kernel is built for"
+    close(out, ref, 2e-5 * math.sqrt(k), 1e-5)
+    # the two-kernel path rounds x / rms * g instead of x * g: same size of error, not the same bits
+    x = torch.empty(m, k, dtype=torch.bfloat16, device=DEV)
+    ops.rmsnorm(src.to(DEV), g.to(DEV), eps, x, None if row_idx is None else row_idx.to(DEV))
+    two = torch.empty(m, n, device=DEV)
+    ops.linear(x, w.to(DEV), b.to(DEV), two)
+    exact = plain_ops.rmsnorm_reference(src if row_idx is None else src[row_idx.long()], g, eps) @ w.double().t() + b.double()
+    e_fold, e_two = (out.cpu().double() - exact).abs().max().item(), (two.cpu().double() - exact).abs().max().item()
+    assert e_fold <= 1.5 * e_two + 1e-4, (e_fold, e_two)
+    base = rnd((m, n), seed=44)
+    acc = base.to(DEV).clone()
+    assert ops.linear_normed(src.to(DEV), g.to(DEV), eps, None if row_idx is None else row_idx.to(DEV),
+                             w.to(DEV), None, acc, accumulate=True)
+    close(acc, ref - b.double() + base.double(), 2e-5 * math.sqrt(k), 1e-5)
+
+
+@pytest.mark.parametrize("m,nf,k", [(8, 1100, 1536), (3, 2100, 3584), (16, 1030, 4096), (1, 18944, 3584)])
+def test_gemm_bf16_normed_swiglu(ops, m, nf, k):
+    h = rnd((m, k), seed=50, scale=2.0)
+    g = 1.0 + rnd((k,), seed=51, scale=0.2)
+    wg, wu = rnd((nf, k), torch.bfloat16, 52, 0.05), rnd((nf, k), torch.bfloat16, 53, 0.05)
+    eps = 1e-6
+    gate = plain_ops.linear_normed_reference(h, g, eps, None, wg, None)
+    up = plain_ops.linear_normed_reference(h, g, eps, None, wu, None)
+    ref = gate / (1 + torch.exp(-gate)) * up
+    w = ops.interleave_gate_up(wg.to(DEV), wu.to(DEV))
+    out = torch.empty(m, nf, dtype=torch.bfloat16, device=DEV)
+    assert ops.linear_normed(h.to(DEV), g.to(DEV), eps, None, w, None, out, swiglu=True)
+    close(out, ref, 2e-5 * math.sqrt(k) + 1e-3, 1e-2)
+
+
+def test_gemm_bf16_normed_declines(ops):
+    """Shapes without a folded kernel: nothing is written and the caller is told."""
+    h, g = rnd((4, 200), seed=60), rnd((200,), seed=61)
+    w = rnd((300, 200), torch.bfloat16, 62)
+    out = torch.full((4, 300), 7.0, device=DEV)
+    assert not ops.linear_normed(h.to(DEV), g.to(DEV), 1e-6, None, w.to(DEV), None, out)
+    assert not ops.linear_normed(rnd((17, 2048), seed=63).to(DEV), rnd((2048,), seed=64).to(DEV), 1e-6, None,
+                                 rnd((4096, 2048), torch.bfloat16, 65).to(DEV), None,
+                                 torch.full((17, 4096), 7.0, device=DEV))
+    torch.cuda.synchronize()
+    assert torch.all(out == 7.0)
