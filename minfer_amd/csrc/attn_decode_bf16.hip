@@ -30,12 +30,50 @@ namespace {
 
 constexpr int STEP = 32;       // keys per wave step
 
+// ROPE: the step's q|k|v come as the 32-bit output of their product, [(nh + 2 nk) hd] per token,
+// not yet rotated and not yet in the cache.  The kernel rotates q on the way into its operand
+// (half-split pairs i, i + hd/2; x0' = x0 c - x1 s, x1' = x0 s + x1 c; src/graph/
+// cpu_backend.rs:421-431), and the blocks of the last split, which holds the token's own
+// position, rotate k, take v, put both into their operands in place of what the cache row
+// holds, and (one block per kv head, when write_kv) store them into the cache for later
+// steps: no rotation kernel and no q buffer between the product and the attention.
+struct RopeArgs {
+  const float* qkv;      // [n_tok][(nh + 2 nk) hd]
+  const float* cs;       // [positions][hd / 2]
+  const float* sn;
+  int write_kv;
+};
+
+// 8 rotated elements d .. d + 7 of one head (src, hd floats) at position pos
 template <int HD>
+__device__ __forceinline__ bf16x8 rotated8(const float* __restrict__ src, const float* __restrict__ cs,
+                                           const float* __restrict__ sn, int pos, int d) {
+  constexpr int HALF = HD / 2;
+  const bool upper = d >= HALF;
+  const int i = upper ? d - HALF : d;               // index into the table and of the lower partner
+  const float4 a0 = *reinterpret_cast<const float4*>(src + i), a1 = *reinterpret_cast<const float4*>(src + i + 4);
+  const float4 b0 = *reinterpret_cast<const float4*>(src + i + HALF);
+  const float4 b1 = *reinterpret_cast<const float4*>(src + i + HALF + 4);
+  const float4 c0 = *reinterpret_cast<const float4*>(cs + (size_t)pos * HALF + i);
+  const float4 c1 = *reinterpret_cast<const float4*>(cs + (size_t)pos * HALF + i + 4);
+  const float4 s0 = *reinterpret_cast<const float4*>(sn + (size_t)pos * HALF + i);
+  const float4 s1 = *reinterpret_cast<const float4*>(sn + (size_t)pos * HALF + i + 4);
+  const float x0[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+  const float x1[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+  const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+  const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+  bf16x8 r;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) r[e] = (bf16)(upper ? x0[e] * sv[e] + x1[e] * c[e] : x0[e] * c[e] - x1[e] * sv[e]);
+  return r;
+}
+
+template <int HD, bool ROPE>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
-    const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vt,
+    const bf16* __restrict__ q, bf16* kc, bf16* vt,
     const int* __restrict__ page_table, int pt_stride, const int* __restrict__ positions,
     const int* __restrict__ seq_of_tok, bf16* __restrict__ out, float* __restrict__ part, int nh, int nk,
-    float scale, int window, int n_splits) {
+    float scale, int window, int n_splits, RopeArgs rope) {
   constexpr int KS = (HD + 31) / 32;      // 32-wide steps over head_dim in the first product
   constexpr int CT = HD / 16;             // 16-wide column tiles of the output
   constexpr int O_LD = HD + 4;
@@ -63,14 +101,63 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int j_begin = lo + split * split_len;
   const int j_end = min(p + 1, j_begin + split_len);
 
-  // B operand of the first product: row = head r16, 8 elements of head_dim at 32 ks + 8 q4
+  // B operand of the first product: row = head r16, 8 elements of head_dim at 32 ks + 8 q4.
+  // ROPE: the block rotates its 16 heads once, one 8-element chunk per thread, into LDS.
+  __shared__ __attribute__((aligned(16))) bf16 sm_q[ROPE ? 16 * KS * 32 : 8];
+  if constexpr (ROPE) {
+    for (int c = threadIdx.x; c < 16 * KS * 4; c += 256) {
+      const int head = c / (KS * 4), d = (c % (KS * 4)) * 8;
+      bf16x8 q8 = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (head < gcount && d < HD)
+        q8 = rotated8<HD>(rope.qkv + ((size_t)t * (nh + 2 * nk) + h0 + head) * HD, rope.cs, rope.sn, p, d);
+      *reinterpret_cast<bf16x8*>(&sm_q[head * KS * 32 + d]) = q8;
+    }
+  }
+  // ROPE: the token's own key and value, for the blocks whose split ends at its position:
+  // rotated (k) and rounded once here, kept in LDS until the step that holds position p.
+  // Key p is row `krow + 4 a` of tile a in its step for exactly one a, in the four lanes of one
+  // r16; value p is element p % 8 of the lanes with q4 = (p % 32) / 8.
+  const int krow = 8 * (r16 >> 2) + (r16 & 3);
+  const bool own_split = ROPE && rope.write_kv && j_end == p + 1 && j_begin <= p;
+  const int po = p % STEP;
+  const int own_a = (po - krow) >> 2;                      // 0 or 1 where this lane holds key p
+  const bool own_k = own_split && (po - krow == 0 || po - krow == 4);
+  const bool own_v = own_split && q4 == (po >> 3);
+  __shared__ __attribute__((aligned(16))) bf16 sm_k[ROPE ? KS * 32 : 8];
+  __shared__ bf16 sm_v[ROPE ? HD : 8];
+  if constexpr (ROPE) {
+    if (own_split) {
+      const int tid = threadIdx.x;
+      const float* row = rope.qkv + (size_t)t * (nh + 2 * nk) * HD;
+      const bool store = blockIdx.y % n_gc == 0;           // one block per kv head fills the cache
+      const int page = pt[p / MF_PAGE];
+      if (tid < KS * 4) {
+        bf16x8 k8 = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (tid * 8 < HD) {
+          k8 = rotated8<HD>(row + (size_t)(nh + hk) * HD, rope.cs, rope.sn, p, tid * 8);
+          if (store)
+            *reinterpret_cast<bf16x8*>(kc + (((size_t)page * nk + hk) * MF_PAGE + p % MF_PAGE) * HD + tid * 8) = k8;
+        }
+        *reinterpret_cast<bf16x8*>(&sm_k[tid * 8]) = k8;
+      }
+      for (int d = tid; d < HD; d += 256) {
+        const bf16 v = (bf16)row[(size_t)(nh + nk + hk) * HD + d];
+        sm_v[d] = v;
+        if (store) vt[(((size_t)page * nk + hk) * HD + d) * MF_PAGE + p % MF_PAGE] = v;
+      }
+    }
+    __syncthreads();
+  }
   bf16x8 qf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
-    qf[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
     const int d = ks * 32 + q4 * 8;
-    if (r16 < gcount && d < HD)
-      qf[ks] = *reinterpret_cast<const bf16x8*>(q + ((size_t)t * nh + h0 + r16) * HD + d);
+    if constexpr (ROPE) {
+      qf[ks] = *reinterpret_cast<const bf16x8*>(&sm_q[r16 * KS * 32 + d]);
+    } else {
+      qf[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (r16 < gcount && d < HD) qf[ks] = *reinterpret_cast<const bf16x8*>(q + ((size_t)t * nh + h0 + r16) * HD + d);
+    }
   }
 
   floatx4 oacc[CT];                       // O^T: head r16, columns 16 c + 4 q4 + r
@@ -83,7 +170,6 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   // keys 8 q4 + 4 a + r, r = 0..3, eight consecutive keys over the two tiles.
   const int step0 = j_begin / STEP;
   const int n_steps = j_begin < j_end ? (j_end - 1) / STEP - step0 + 1 : 0;
-  const int krow = 8 * (r16 >> 2) + (r16 & 3);
   bf16x8 kn[2][KS], vn[CT];
   auto issue = [&](int i) {
     const int jb = (step0 + i) * STEP;
@@ -115,6 +201,27 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const int jb = (step0 + i) * STEP;
     const int key0 = jb + 8 * q4;                  // this lane's eight keys: key0 .. key0 + 7
     const bool edge = jb < j_begin || jb + STEP > j_end;
+    if constexpr (ROPE) {
+      if (own_split && jb + po == p) {             // the step of the token's own position
+        if (own_k) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            const bf16x8 k8 = *reinterpret_cast<const bf16x8*>(&sm_k[ks * 32 + q4 * 8]);
+            if (own_a == 0) kf[0][ks] = k8;
+            else kf[1][ks] = k8;
+          }
+        }
+        if (own_v) {
+#pragma unroll
+          for (int c = 0; c < CT; ++c) {
+            const bf16 v = sm_v[16 * c + r16];
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (e == (po & 7)) vf[c][e] = v;
+          }
+        }
+      }
+    }
     if (edge) {
       // Keys outside the split are masked out of P below, but their V may never have been
       // written (a page is not cleared when it is taken) and 0 * garbage could be NaN:
@@ -208,19 +315,43 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 }
 
 template <int HD>
-int launch(const bf16* q, const bf16* kc, const bf16* vt, const int* page_table, int pt_stride,
-           const int* positions, const int* seq_of_tok, bf16* out, float* part, int n_tok, int nh, int nk,
-           float scale, int window, int n_splits, hipStream_t stream) {
+int launch(const bf16* q, bf16* kc, bf16* vt, const int* page_table, int pt_stride, const int* positions,
+           const int* seq_of_tok, bf16* out, float* part, int n_tok, int nh, int nk, float scale, int window,
+           int n_splits, const RopeArgs* rope, hipStream_t stream) {
   const int G = nh / nk;
   dim3 grid(n_tok, nk * ((G + 15) / 16), n_splits);
-  attn_decode_kernel<HD><<<grid, 256, 0, stream>>>(q, kc, vt, page_table, pt_stride, positions, seq_of_tok, out,
-                                                   part, nh, nk, scale, window, n_splits);
+  if (rope)
+    attn_decode_kernel<HD, true><<<grid, 256, 0, stream>>>(q, kc, vt, page_table, pt_stride, positions, seq_of_tok,
+                                                           out, part, nh, nk, scale, window, n_splits, *rope);
+  else
+    attn_decode_kernel<HD, false><<<grid, 256, 0, stream>>>(q, kc, vt, page_table, pt_stride, positions,
+                                                            seq_of_tok, out, part, nh, nk, scale, window, n_splits,
+                                                            RopeArgs{nullptr, nullptr, nullptr, 0});
   int rc = mf_launch_status();
   if (rc == 0 && n_splits > 1) {
     attn_tokens::attn_combine_kernel<bf16><<<n_tok * nh, 64, 0, stream>>>(part, out, HD, n_splits);
     rc = mf_launch_status();
   }
   return rc;
+}
+
+int dispatch(const void* q, void* kc, void* vt, const int* page_table, int pt_stride, const int* positions,
+             const int* seq_of_tok, void* out, float* part, int n_tok, int nh, int nk, int hd, float scale,
+             int window, int n_splits, const RopeArgs* rope, hipStream_t stream) {
+  if (n_tok <= 0) return 0;
+  if (hd % 16 != 0 || hd < 16 || hd > 256 || nk <= 0 || nh % nk != 0 || n_splits < 1 || n_splits > 64 ||
+      (n_splits > 1 && part == nullptr))
+    return (int)hipErrorInvalidValue;
+#define MF_CASE(E)                                                                                          \
+  case E:                                                                                                   \
+    return launch<16 * E>((const bf16*)q, (bf16*)kc, (bf16*)vt, page_table, pt_stride, positions,           \
+                          seq_of_tok, (bf16*)out, part, n_tok, nh, nk, scale, window, n_splits, rope, stream);
+  switch (hd / 16) {
+    MF_CASE(1) MF_CASE(2) MF_CASE(3) MF_CASE(4) MF_CASE(5) MF_CASE(6) MF_CASE(7) MF_CASE(8)
+    MF_CASE(9) MF_CASE(10) MF_CASE(11) MF_CASE(12) MF_CASE(13) MF_CASE(14) MF_CASE(15) MF_CASE(16)
+  }
+#undef MF_CASE
+  return (int)hipErrorInvalidValue;
 }
 
 }  // namespace
@@ -231,19 +362,21 @@ MF_API int mf_attn_decode_bf16(const void* q, const void* kc, const void* vt, co
                                int pt_stride, const int* positions, const int* seq_of_tok, void* out,
                                float* part, int n_tok, int nh, int nk, int hd, float scale, int window,
                                int n_splits, hipStream_t stream) {
-  if (n_tok <= 0) return 0;
-  if (hd % 16 != 0 || hd < 16 || hd > 256 || nk <= 0 || nh % nk != 0 || n_splits < 1 || n_splits > 64 ||
-      (n_splits > 1 && part == nullptr))
-    return (int)hipErrorInvalidValue;
-#define MF_CASE(E)                                                                                          \
-  case E:                                                                                                   \
-    return launch<16 * E>((const bf16*)q, (const bf16*)kc, (const bf16*)vt, page_table, pt_stride,          \
-                          positions, seq_of_tok, (bf16*)out, part, n_tok, nh, nk, scale, window, n_splits,  \
-                          stream);
-  switch (hd / 16) {
-    MF_CASE(1) MF_CASE(2) MF_CASE(3) MF_CASE(4) MF_CASE(5) MF_CASE(6) MF_CASE(7) MF_CASE(8)
-    MF_CASE(9) MF_CASE(10) MF_CASE(11) MF_CASE(12) MF_CASE(13) MF_CASE(14) MF_CASE(15) MF_CASE(16)
-  }
-#undef MF_CASE
-  return (int)hipErrorInvalidValue;
+  return dispatch(q, const_cast<void*>(kc), const_cast<void*>(vt), page_table, pt_stride, positions, seq_of_tok,
+                  out, part, n_tok, nh, nk, hd, scale, window, n_splits, nullptr, stream);
+}
+
+// The same with the rotation and the cache write of the step's own q|k|v folded in: qkv is the
+// 32-bit [n_tok][(nh + 2 nk) hd] output of their product, cs/sn the [positions][hd / 2] tables.
+// Each token must be the last position of its sequence (a decode step); hd must be a multiple
+// of 16 so that 8-element chunks do not straddle the half.  With write_kv = 0 nothing is
+// stored and k, v come from the cache (a layer that reads another layer's cache).
+MF_API int mf_attn_decode_rope_bf16(const float* qkv, const float* cs, const float* sn, void* kc, void* vt,
+                                    const int* page_table, int pt_stride, const int* positions,
+                                    const int* seq_of_tok, void* out, float* part, int n_tok, int nh, int nk,
+                                    int hd, float scale, int window, int n_splits, int write_kv,
+                                    hipStream_t stream) {
+  const RopeArgs rope{qkv, cs, sn, write_kv};
+  return dispatch(nullptr, kc, vt, page_table, pt_stride, positions, seq_of_tok, out, part, n_tok, nh, nk, hd,
+                  scale, window, n_splits, &rope, stream);
 }

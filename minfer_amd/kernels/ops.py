@@ -56,6 +56,8 @@ _PROTOTYPES = {
     "attn_decode_bf16": {
         "mf_attn_decode_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
                                 c_float, c_int, c_int, _P],
+        "mf_attn_decode_rope_bf16": [_P, _P, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int,
+                                     c_int, c_float, c_int, c_int, c_int, _P],
     },
     "attn_prefill_bf16": {
         "mf_attn_prefill_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int,
@@ -425,6 +427,39 @@ def attn_tokens(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions),
         _ptr(seq_of_tok), _ptr(out), _ptr(part), n_tok, n_heads, n_kv_heads, head_dim, float(scale),
         int(window or 0), n_splits, split_len, _stream()), "attn_tokens_f32")
+
+
+def attn_decode_rope(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, kcache: torch.Tensor,
+                     vcache: torch.Tensor, page_table: torch.Tensor, positions: torch.Tensor,
+                     seq_of_tok: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
+                     scale: float, window: int, max_len: int, write_kv: bool = True) -> None:
+    """A bfloat16 decode step's rotation, cache write and attention in one kernel: qkv is the
+    float32 `[tokens][(heads + 2 kv_heads) head_dim]` output of the q|k|v product; every token is
+    the next position of its sequence.  Same result as `rope_kvwrite` then `attn_tokens`."""
+    n_tok = positions.numel()
+    _need(qkv, "attn_decode_rope.qkv", torch.float32, (n_tok, (n_heads + 2 * n_kv_heads) * head_dim))
+    _need(cos, "attn_decode_rope.cos", torch.float32)
+    _need(sin, "attn_decode_rope.sin", torch.float32, tuple(cos.shape))
+    if cos.shape[1] != head_dim // 2:
+        raise KernelError(f"rope: table has {cos.shape[1]} frequencies, head_dim {head_dim} needs {head_dim // 2}")
+    _need(out, "attn_decode_rope.out", torch.bfloat16, (n_tok, n_heads * head_dim))
+    _need_caches("attn_decode_rope", kcache, vcache, torch.bfloat16, n_kv_heads, head_dim)
+    _need(page_table, "attn_decode_rope.page_table", torch.int32)
+    _need(positions, "attn_decode_rope.positions", torch.int32, (n_tok,))
+    _need(seq_of_tok, "attn_decode_rope.seq_of_tok", torch.int32, (n_tok,))
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise KernelError(f"attention: head_dim {head_dim} is not a multiple of 16 in [16, 256]")
+    if n_heads % n_kv_heads:
+        raise KernelError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
+    if max_len > page_table.shape[1] * PAGE or max_len > cos.shape[0]:
+        raise KernelError(f"attention: max_len {max_len} exceeds the page table ({page_table.shape[1]} pages) "
+                          f"or the rotation table ({cos.shape[0]} positions)")
+    n_splits = decode_split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, max_len)
+    part = workspace("attn", n_tok * n_heads * n_splits * (head_dim + 2), qkv.device) if n_splits > 1 else None
+    _check(_fn("attn_decode_bf16", "mf_attn_decode_rope_bf16")(
+        _ptr(qkv), _ptr(cos), _ptr(sin), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1],
+        _ptr(positions), _ptr(seq_of_tok), _ptr(out), _ptr(part), n_tok, n_heads, n_kv_heads, head_dim,
+        float(scale), int(window or 0), n_splits, 1 if write_kv else 0, _stream()), "attn_decode_rope_bf16")
 
 
 def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,

@@ -71,10 +71,16 @@ class GQAttention(Mixer):
         kc, vc, group = ctx.cache.kv(entry)
         table = ctx.page_table(group)
         qkv = self.qkv(x, out_dtype=torch.float32)
-        q = torch.empty((x.shape[0], self.nh * self.hd), dtype=self.rt.dtype, device=x.device)
-        self.position.rotate_and_store(qkv, ctx, q, kc, vc, table, self.nh, self.nk, writes_cache)
-        o = torch.empty_like(q)
         window = 0 if self.window is None else int(self.window)
+        o = torch.empty((x.shape[0], self.nh * self.hd), dtype=self.rt.dtype, device=x.device)
+        tables = self.position.rotation_tables(ctx.max_len) if self.rt.is_bf16 and ctx.all_decode else None
+        if tables is not None:         # decode: rotation, cache write and attention in one kernel
+            ops.attn_decode_rope(qkv, tables[0], tables[1], kc, vc, table, ctx.positions, ctx.seq_of_tok, o,
+                                 self.nh, self.nk, self.hd, self.scale, window, ctx.max_len, writes_cache)
+            self.o(o, out=h, accumulate=True)
+            return
+        q = torch.empty_like(o)
+        self.position.rotate_and_store(qkv, ctx, q, kc, vc, table, self.nh, self.nk, writes_cache)
         if self.rt.is_bf16 and not ctx.all_decode and ops.HAVE_PREFILL_ATTENTION:
             ops.attn_prefill(q, kc, vc, table, ctx, o, self.nh, self.nk, self.hd, self.scale, window)
         else:

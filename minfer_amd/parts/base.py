@@ -99,6 +99,11 @@ class PositionEncoding(Part):
         step's tokens into the cache pages."""
         raise NotImplementedError
 
+    def rotation_tables(self, max_len: int):
+        """(cos, sin) `[positions][head_dim / 2]` float32 tables if this encoding is the
+        half-split rotation the decode attention kernel can apply itself, else None."""
+        return None
+
 
 class Mixer(Part):
     def cache_request(self):

@@ -35,6 +35,10 @@ class RotaryNeoX(PositionEncoding):
             self.cos, self.sin = ops.rope_table(n, self.head_dim // 2, self.theta, self.freq_scale,
                                                 self.rt.device)
 
+    def rotation_tables(self, max_len: int):
+        self.prepare(max_len)
+        return self.cos, self.sin
+
     def rotate_and_store(self, qkv, ctx, q_out, kcache, vcache, page_table, n_heads, n_kv_heads,
                          write_kv: bool) -> None:
         self.prepare(ctx.max_len)

@@ -169,6 +169,15 @@ def attn_tokens(q, kcache, vcache, page_table, positions, seq_of_tok, out, n_hea
     out.copy_(res.view(t, n_heads * head_dim).to(out.dtype))
 
 
+def attn_decode_rope(qkv, cos, sin, kcache, vcache, page_table, positions, seq_of_tok, out, n_heads,
+                     n_kv_heads, head_dim, scale, window, max_len, write_kv=True):
+    q = torch.empty(positions.numel(), n_heads * head_dim, dtype=out.dtype)
+    rope_kvwrite(qkv, cos, sin, positions, seq_of_tok, page_table, q, kcache, vcache, n_heads, n_kv_heads,
+                 head_dim, write_kv)
+    attn_tokens(q, kcache, vcache, page_table, positions, seq_of_tok, out, n_heads, n_kv_heads, head_dim, scale,
+                window, max_len)
+
+
 def attn_prefill(q, kcache, vcache, page_table, ctx, out, n_heads, n_kv_heads, head_dim, scale, window):
     attn_tokens(q, kcache, vcache, page_table, ctx.positions, ctx.seq_of_tok, out, n_heads, n_kv_heads,
                 head_dim, scale, window, ctx.max_len)
@@ -219,7 +228,7 @@ def advance(next_ids, sampled, positions, steps):
 
 NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", "rope_table",
          "rope_kvwrite", "linear", "attn_tokens", "attn_prefill", "argmax", "sample", "penalties",
-         "top_k", "top_p", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed"]
+         "top_k", "top_p", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed", "attn_decode_rope"]
 
 
 def install(monkeypatch):

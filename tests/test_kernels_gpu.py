@@ -294,6 +294,54 @@ def test_attn_tokens(ops, dtype, nh, nk, hd, window):
     assert torch.equal(again, outs[0]), "two runs differ"
 
 
+@pytest.mark.parametrize("write_kv", [True, False])
+@pytest.mark.parametrize("nh,nk,hd,window", [(4, 2, 16, 0), (9, 3, 48, 0), (28, 4, 128, 0), (20, 1, 80, 0),
+                                             (4, 2, 256, 0), (4, 2, 64, 40), (36, 2, 128, 0)])
+def test_attn_decode_rope(ops, nh, nk, hd, window, write_kv):
+    """Rotation + cache write + attention of a decode step in one kernel against the two-step
+    plain path.  The row of the token's own position is poisoned beforehand when the kernel
+    is to write it: it must take k and v from the product's output, not from the cache."""
+    lengths = [1, 2, 31, 32, 33, 64, 65, 129, 500, 1000]
+    rng = np.random.default_rng(31)
+    n_cols = max((l + 63) // 64 for l in lengths)
+    n_pages = sum((l + 63) // 64 for l in lengths) + 3
+    perm = rng.permutation(n_pages)
+    table = -np.ones((len(lengths), n_cols), dtype=np.int32)
+    nxt = 0
+    for b, l in enumerate(lengths):
+        for c in range((l + 63) // 64):
+            table[b, c] = perm[nxt]
+            nxt += 1
+    kc, vc = make_cache(n_pages, nk, hd, torch.bfloat16, 32)
+    # rows from the token's own position on are unwritten; with write_kv False the own row exists
+    poison_unwritten(kc, vc, table, [l - 1 if write_kv else l for l in lengths])
+    vc = stored_v(vc)
+    table = torch.from_numpy(table)
+    pos = torch.tensor([l - 1 for l in lengths], dtype=torch.int32)
+    seq = torch.arange(len(lengths), dtype=torch.int32)
+    qkv = rnd((len(lengths), (nh + 2 * nk) * hd), seed=33)
+    cs, sn = plain_ops.rope_table(1024, hd // 2, 1e4, 1.0, "cpu")
+    scale = 1.0 / math.sqrt(hd)
+    kr, vr = kc.clone(), vc.clone()
+    ref = torch.empty(len(lengths), nh * hd, dtype=torch.float64)
+    plain_ops.attn_decode_rope(qkv, cs, sn, kr, vr, table, pos, seq, ref, nh, nk, hd, scale, window, 1000, write_kv)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    out = torch.empty(len(lengths), nh * hd, dtype=torch.bfloat16, device=DEV)
+    ops.attn_decode_rope(qkv.to(DEV), cs.to(DEV), sn.to(DEV), kd, vd, table.to(DEV), pos.to(DEV), seq.to(DEV),
+                         out, nh, nk, hd, scale, window, 1000, write_kv)
+    close(out, ref, 1.5e-2, 1.5e-2)
+    # the cache afterwards: the own rows written (or nothing touched), everything else as before
+    same = lambda a, b: torch.equal(torch.nan_to_num(a.float(), nan=7e7), torch.nan_to_num(b.float(), nan=7e7))
+    if write_kv:
+        close(torch.nan_to_num(kd.float(), nan=7e7), torch.nan_to_num(kr.float(), nan=7e7), 2e-2, 2e-2)
+        close(torch.nan_to_num(vd.float(), nan=7e7), torch.nan_to_num(vr.float(), nan=7e7), 2e-2, 2e-2)
+        for b, l in enumerate(lengths):
+            page, off = int(table[b, (l - 1) // 64]), (l - 1) % 64
+            assert not torch.isnan(kd[page, :, off].float()).any() and not torch.isnan(vd[page, :, :, off].float()).any()
+    else:
+        assert same(kd.cpu(), kc) and same(vd.cpu(), vc)
+
+
 def test_attention_one_key_gives_v_and_far_key_is_found(ops):
     # one key -> output = V exactly (src/graph/cpu_backend.rs:640-682), broadcast over the group
     nh, nk, hd = 4, 2, 16
