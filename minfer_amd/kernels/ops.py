@@ -386,12 +386,15 @@ def _need_caches(what: str, kcache: torch.Tensor, vcache: torch.Tensor, dtype, n
                           f"[{kcache.shape[0]}, {want[0]}, {want[1]}, {want[2]}]")
 
 
-def decode_split_plan(n_tok: int, n_kv_heads: int, group: int, max_len: int, target_blocks: int = 512) -> int:
-    """Key splits of the bfloat16 decode attention: enough blocks to fill the chip, at least
-    128 keys of the longest possible sequence per split, at most 64.  The kernel divides each
-    token's own length by this number, so every split has work."""
+def decode_split_plan(n_tok: int, n_kv_heads: int, group: int, max_len: int, target_blocks: int = 256) -> int:
+    """Key splits of the bfloat16 decode attention: about one block per CU (measured best at
+    1, 8 and 64 sequences of 4 kv heads), at least 128 keys of the longest possible sequence
+    per split, at most 16.  The kernel divides each token's own length by this number, so
+    every split has work."""
     blocks = n_tok * n_kv_heads * ((group + 15) // 16)
-    return max(1, min(target_blocks // max(1, blocks), (max_len + 127) // 128, 64))
+    if os.environ.get("MF_ATTN_SPLITS"):
+        return int(os.environ["MF_ATTN_SPLITS"])
+    return max(1, min(target_blocks // max(1, blocks), (max_len + 127) // 128, 16))
 
 
 def attn_tokens(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
