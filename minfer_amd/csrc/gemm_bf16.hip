@@ -452,6 +452,18 @@ __global__ __launch_bounds__(NW * 64) void skinny16_kernel(const bf16* __restric
   }
 }
 
+// compute units of the current device (0 on error)
+static int cu_count() {
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
+    n_cu = prop.multiProcessorCount;
+  }
+  return n_cu;
+}
+
 // The same split of the work as skinny16_kernel (a block owns 16 NT weight rows, its waves split
 // K), for aligned operands and K a multiple of 32, with the loads rolling: a wave holds S steps
 // of weights and activations in registers, and the refill of a register is issued right behind
@@ -464,15 +476,21 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
                                                             const bf16* __restrict__ W, int ldw,
                                                             const float* __restrict__ bias,
                                                             void* __restrict__ C, int ldc, int M, int N,
-                                                            int K, int steps_per_wave, int epi) {
+                                                            int K, int steps_per_wave, int epi, int rpb) {
   constexpr int COLS = 16 * NT;
   constexpr int RS = COLS + 4;
   __shared__ float red[NW][16][RS];
   const int lane = threadIdx.x & 63;
   const int wid = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // the same in the whole wave
   const int r16 = lane & 15;
+  // rpb: weight rows per block (at most 16 NT; fewer when that spreads the rows over every CU:
+  // a CU draws only so much from memory, so an idle CU is bandwidth lost).  Lanes past the
+  // block's rows read its last row again, from the CU's own cache.
   auto tile_row = [&](int j) {
-    return PAIR ? (blockIdx.x >> 1) * 64 + (blockIdx.x & 1) * 16 + j * 32 : (blockIdx.x * NT + j) * 16;
+    return PAIR ? (blockIdx.x >> 1) * 64 + (blockIdx.x & 1) * 16 + j * 32 : blockIdx.x * rpb + j * 16;
+  };
+  auto lane_row = [&](int j) {           // the weight row this lane reads in tile j
+    return PAIR ? tile_row(j) + r16 : blockIdx.x * rpb + min(j * 16 + r16, rpb - 1);
   };
   const int total = K / 32;
   const int first = min(wid * steps_per_wave, total);
@@ -481,7 +499,7 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
   const bf16* arow = A + (size_t)min(r16, M - 1) * lda + kq;
   const bf16* wrow[NT];
 #pragma unroll
-  for (int j = 0; j < NT; ++j) wrow[j] = W + (size_t)min(tile_row(j) + r16, N - 1) * ldw + kq;
+  for (int j = 0; j < NT; ++j) wrow[j] = W + (size_t)min(lane_row(j), N - 1) * ldw + kq;
   floatx4 acc[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -558,7 +576,7 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
   }
   const int c = lane % COLS;
   const int n = tile_row(c >> 4) + (c & 15);
-  if (n >= N) return;
+  if (n >= N || (!PAIR && c >= rpb)) return;
   const float b = bias ? bias[n] : 0.f;
   for (int m = lane / COLS; m < M; m += 64 / COLS) {
     float v = 0.f;
@@ -572,9 +590,16 @@ template <int NW, int NT, int S, bool PAIR = false>
 int launch_rolling16(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
                      int M, int N, int K, int epi, hipStream_t stream) {
   const int steps_per_wave = (K / 32 + NW - 1) / NW;
-  const int blocks = PAIR ? N / 32 : (N + 16 * NT - 1) / (16 * NT);
+  int rpb = 16 * NT, blocks = N / 32;
+  if (!PAIR) {
+    const int n_cu = cu_count();
+    if (n_cu <= 0) return (int)hipErrorUnknown;
+    rpb = (N + n_cu - 1) / n_cu;                 // one block per CU when the rows are few
+    rpb = rpb < 1 ? 1 : (rpb > 16 * NT ? 16 * NT : rpb);
+    blocks = (N + rpb - 1) / rpb;
+  }
   rolling16_kernel<NW, NT, S, PAIR><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K,
-                                                                    steps_per_wave, epi);
+                                                                    steps_per_wave, epi, rpb);
   return mf_launch_status();
 }
 
@@ -618,7 +643,7 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
                                                            const bf16* __restrict__ W, int ldw,
                                                            const float* __restrict__ bias,
                                                            void* __restrict__ C, int ldc, int M, int N,
-                                                           int n_items, int epi, NormArgs norm) {
+                                                           int cols_total, int unit, int epi, NormArgs norm) {
   constexpr int NW = 8;
   constexpr int COLS = 16 * NT;            // weight rows (output columns) of an item
   constexpr int RS = COLS + 4;             // row stride of the sums in LDS: conflict-free writes
@@ -628,15 +653,28 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int r16 = lane & 15;
   const int k0 = wid * NS * 32 + (lane >> 4) * 8;         // this lane's k in step 0 of its slice
-  // first weight row of tile j of an item (before the lane's own row is added)
-  auto tile_row = [&](int item, int j) {
-    return PAIR ? (item >> 1) * 64 + (item & 1) * 16 + j * 32 : (item * NT + j) * 16;
+  // The block's share: output columns [c_begin, c_end), the same number for every block up to
+  // one `unit`, so that every CU streams the same bytes (a CU draws only so much from memory;
+  // whole items per block would leave some with a fifth more than others).  PAIR: a column is
+  // a gate row and the up row 32 further on, in groups of 64 weight rows.  An item is CH
+  // columns; lanes past c_end read the share's last row again, from the CU's own cache.
+  constexpr int CH = PAIR ? 16 : COLS;
+  const int units = (cols_total + unit - 1) / unit;
+  const int c_begin = (int)((long)blockIdx.x * units / gridDim.x) * unit;
+  const int c_end = min((int)((long)(blockIdx.x + 1) * units / gridDim.x) * unit, cols_total);
+  const int n_items = (c_end - c_begin + CH - 1) / CH;
+  auto lane_wrow = [&](int c0, int j) {      // weight row of this lane in tile j of the item at c0
+    if (PAIR) {
+      const int col = min(c0 + r16, c_end - 1);
+      return (col >> 5) * 64 + (col & 31) + 32 * j;
+    }
+    return min(c0 + 16 * j + r16, c_end - 1);
   };
   bf16x8 w[NT][NS];
   const bf16* wrow[NT];
-  int item = blockIdx.x;
+  const int item = 0;
   auto first_loads = [&](int j) {
-    wrow[j] = W + (size_t)min(tile_row(item, j) + r16, N - 1) * ldw + k0;
+    wrow[j] = W + (size_t)lane_wrow(c_begin, j) * ldw + k0;
 #pragma unroll
     for (int s = 0; s < NS; ++s) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32);
   };
@@ -697,15 +735,15 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
 #pragma unroll
     for (int j = 1; j < NT; ++j) first_loads(j);
   }
-  for (int it = 0; item < n_items; item += gridDim.x, ++it) {
+  for (int it = 0; it < n_items; ++it) {
     // The loop body has no branch, so that the compiler can count the loads in flight and wait
     // for the oldest one only: behind the last item the loads go to the head of the matrix,
     // the same few lines for every lane, and their values are dropped.
-    const int next = item + gridDim.x;
-    const bool has_next = next < n_items;
+    const int c0 = c_begin + it * CH;
+    const bool has_next = it + 1 < n_items;
 #pragma unroll
     for (int j = 0; j < NT; ++j)
-      wrow[j] = W + (has_next ? (size_t)min(tile_row(next, j) + r16, N - 1) * ldw : (size_t)0) + k0;
+      wrow[j] = W + (has_next ? (size_t)lane_wrow(c0 + CH, j) * ldw : (size_t)0) + k0;
     floatx4 acc[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -736,8 +774,8 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
     };
     if (epi == EPI_SWIGLU) {
       if constexpr (PAIR && NT == 2) {
-        const int col = item * 16 + r16;
-        if (col < ldc) {
+        const int col = c0 + r16;
+        if (col < c_end && col < ldc) {
           for (int m = lane >> 4; m < M; m += 4) {
             float g = 0.f, u = 0.f;
 #pragma unroll
@@ -755,8 +793,8 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
     }
     // a pass of the wave covers 64 / COLS activation rows of COLS adjacent outputs each
     const int c = lane % COLS;
-    const int n = tile_row(item, c >> 4) + (c & 15);
-    if (n >= N) continue;
+    const int n = c0 + c;
+    if (n >= c_end) continue;
     const float b = bias ? bias[n] : 0.f;
     for (int m = lane / COLS; m < M; m += 64 / COLS) {
       float v = 0.f;
@@ -772,21 +810,21 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
 template <int NS, int NT, bool PAIR>
 int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
                         int M, int N, int epi, const NormArgs* norm, hipStream_t stream) {
-  const int n_items = PAIR ? N / 32 : (N + 16 * NT - 1) / (16 * NT);
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return (int)hipErrorUnknown;
-    n_cu = prop.multiProcessorCount;
-  }
-  const int grid = n_items < n_cu ? n_items : n_cu;
+  const int n_cu = cu_count();
+  if (n_cu <= 0) return (int)hipErrorUnknown;
+  const int cols_total = PAIR ? N / 2 : N;
+  // shares in whole 128-byte lines of 32-bit output where the output is large enough for the
+  // cost of partial lines to show; else in pairs of columns
+  const int unit = (!PAIR && cols_total / 32 >= 8 * n_cu) ? 32 : 2;
+  const int units = (cols_total + unit - 1) / unit;
+  const int grid = units < n_cu ? units : n_cu;
   if (norm)
-    stationary16_kernel<NS, NT, PAIR, true><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, n_items,
-                                                                      epi, *norm);
+    stationary16_kernel<NS, NT, PAIR, true><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
+                                                                      cols_total, unit, epi, *norm);
   else
-    stationary16_kernel<NS, NT, PAIR, false><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, n_items,
-                                                                       epi, NormArgs{nullptr, nullptr, 0.f});
+    stationary16_kernel<NS, NT, PAIR, false><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
+                                                                       cols_total, unit, epi,
+                                                                       NormArgs{nullptr, nullptr, 0.f});
   return mf_launch_status();
 }
 
@@ -888,8 +926,10 @@ static int stationary16(const void* a, int lda, const bf16* w, int ldw, const fl
   static const int off = getenv("MF_NO_STATIONARY") ? 1 : 0;
   if (off || M > 16 || K % 256 != 0 || (N + 15) / 16 < 128) return MF_NOT_BUILT;
   if (epi == EPI_SWIGLU && N % 64 != 0) return MF_NOT_BUILT;
-  // two tiles an item where there are enough of them: 128-byte rows of 32-bit output
-  const bool two = (N + 31) / 32 >= 128;
+  // two tiles an item where a block's share is more than one: 128-byte rows of 32-bit output
+  const int n_cu = cu_count();
+  if (n_cu <= 0) return (int)hipErrorUnknown;
+  const bool two = (N + n_cu - 1) / n_cu > 16;
 #define MF_STATIONARY(NS_)                                                                                  \
   case NS_:                                                                                                 \
     return epi == EPI_SWIGLU                                                                                \
