@@ -95,12 +95,20 @@ class DecodeSession:
         new_len = {s: cache.length(s) + 1 for s in self.slots}
         if max(new_len.values()) > self.max_len:
             raise ValueError(f"decode session was sized for {self.max_len} positions")
-        cache.reserve(new_len)
-        for g in cache.groups:
-            rows = cache.page_rows(g, self.slots, self.n_cols)
-            if self._host_tables.get(id(g)) != rows:
-                self.tables[id(g)].copy_(torch.tensor(rows, dtype=torch.int32))
-                self._host_tables[id(g)] = rows
+        # A page table row changes only when its sequence starts a new page (or, in a windowed
+        # group, gives one back): that is the only time the host touches the tables.
+        grows = [s for s, n in new_len.items() if (n - 1) % PAGE == 0]
+        windowed = any(g.request.window is not None for g in cache.groups)
+        if grows:
+            cache.reserve({s: new_len[s] for s in grows})
+        if grows or windowed or not self._host_tables:
+            for g in cache.groups:
+                if self._host_tables and not grows and g.request.window is None:
+                    continue
+                rows = cache.page_rows(g, self.slots, self.n_cols)
+                if self._host_tables.get(id(g)) != rows:
+                    self.tables[id(g)].copy_(torch.tensor(rows, dtype=torch.int32))
+                    self._host_tables[id(g)] = rows
         if not self.use_graph:
             self._run()
         elif self.graph is not None:
