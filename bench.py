@@ -100,13 +100,22 @@ def run_decode(llm, cfg, batch, prompt_max, steps, warmup, use_graph, elem):
     sampler = Sampler(SamplingParams.greedy())
     sess = eng.decode_session(batch, prompt_max + warmup + steps + 8, sampler, use_graph=use_graph)
     sess.bind(slots, first, list(range(batch)), [1] * batch)
-    for _ in range(warmup):
-        sess.step()
+    def run(n):
+        """n decode steps the way the generation loop runs them: the next step is started before
+        the tokens of the one before are read."""
+        pending = sess.launch()
+        for _ in range(n - 1):
+            ahead = sess.launch()
+            sess.collect(pending)
+            pending = ahead
+        sess.collect(pending)
+
+    if warmup:
+        run(warmup)
     ctx_start = sum(eng.length(s) for s in slots)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        sess.step()
+    run(steps)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ctx_end = sum(eng.length(s) for s in slots)

@@ -366,14 +366,26 @@ __global__ __launch_bounds__(NT) void top_p_kernel(float* __restrict__ logits, i
   }
 }
 
-// after a decode step: feed the sampled token back, move every sequence on by one
+// after a decode step: feed the sampled token back, move every sequence on by one, and (when
+// prev is given) put the token into the sequence's window of recent tokens: prev[i] holds the
+// last n_prev[i] <= max_prev tokens in no particular order (the penalties count, they do not
+// look at the order), cursor[i] is where the next one goes, the oldest once the window is full.
 __global__ void advance_kernel(int* __restrict__ next_ids, const int* __restrict__ sampled,
-                               int* __restrict__ positions, int* __restrict__ steps, int n) {
+                               int* __restrict__ positions, int* __restrict__ steps, int n,
+                               int* __restrict__ prev, int max_prev, int* __restrict__ n_prev,
+                               int* __restrict__ cursor) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  next_ids[i] = sampled[i];
+  const int tok = sampled[i];
+  next_ids[i] = tok;
   positions[i] += 1;
   steps[i] += 1;
+  if (prev) {
+    const int c = cursor[i];
+    prev[(size_t)i * max_prev + c] = tok;
+    cursor[i] = c + 1 == max_prev ? 0 : c + 1;
+    if (n_prev[i] < max_prev) n_prev[i] += 1;
+  }
 }
 
 }  // namespace
@@ -429,9 +441,11 @@ MF_API int mf_top_p(float* logits, int ld, int rows, int vocab, float p, hipStre
   return mf_launch_status();
 }
 
-MF_API int mf_advance(int* next_ids, const int* sampled, int* positions, int* steps, int n,
-                      hipStream_t stream) {
+MF_API int mf_advance(int* next_ids, const int* sampled, int* positions, int* steps, int n, int* prev,
+                      int max_prev, int* n_prev, int* cursor, hipStream_t stream) {
   if (n <= 0) return 0;
-  advance_kernel<<<(n + 255) / 256, 256, 0, stream>>>(next_ids, sampled, positions, steps, n);
+  if (prev && (max_prev <= 0 || !n_prev || !cursor)) return (int)hipErrorInvalidValue;
+  advance_kernel<<<(n + 255) / 256, 256, 0, stream>>>(next_ids, sampled, positions, steps, n, prev, max_prev,
+                                                      n_prev, cursor);
   return mf_launch_status();
 }

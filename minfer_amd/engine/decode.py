@@ -6,7 +6,8 @@ The reference reuses its built graph across decode steps because positions are d
 structure (src/graph/params.rs:39-52, src/graph/cache.rs:37-54 of yusiwen/minfer), and its
 CUDA path captures the step as a CUDA graph (src/cuda.rs:480-527).  Here token ids,
 positions, page tables, sampler counters and the recent-token windows live in buffers of a
-fixed size per batch size; the host only reserves pages ahead and reads the sampled tokens.
+fixed size per batch size; the host only reserves pages ahead and reads the sampled tokens,
+and it may start the next step before it has read them (`launch` / `collect`).
 """
 from __future__ import annotations
 
@@ -43,6 +44,14 @@ class DecodeSession:
         self.sampled = torch.zeros(n_seqs, **i32)
         self.prev = torch.zeros((n_seqs, REPEAT_LAST_N), **i32)
         self.n_prev = torch.zeros(n_seqs, **i32)
+        self.cursor = torch.zeros(n_seqs, **i32)
+        # results of the two steps that may be in flight travel to pinned host memory
+        self._pinned = self._events = None
+        if dev.type == "cuda":
+            self._pinned = [torch.empty(n_seqs, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+            self._events = [torch.cuda.Event() for _ in range(2)]
+        self._host_out: List[Optional[List[int]]] = [None, None]
+        self._launched = self._collected = 0
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.warm = False
         self.slots: List[int] = []
@@ -64,6 +73,8 @@ class DecodeSession:
         self.keys.copy_(torch.tensor(list(keys), dtype=torch.int64))
         self.steps.copy_(torch.tensor(list(steps), dtype=torch.int32))
         self._host_tables = {}
+        if self._launched != self._collected:
+            raise RuntimeError("decode session bound while a step is in flight")
 
     def set_windows(self, windows: Sequence[Sequence[int]]) -> None:
         """Recent tokens of each sequence for the penalties (at most the last 64)."""
@@ -74,6 +85,7 @@ class DecodeSession:
                 flat[i, :len(r)] = torch.tensor(r, dtype=torch.int32)
         self.prev.copy_(flat)
         self.n_prev.copy_(torch.tensor([len(r) for r in rows], dtype=torch.int32))
+        self.cursor.copy_(torch.tensor([len(r) % REPEAT_LAST_N for r in rows], dtype=torch.int32))
 
     # ------------------------------------------------------------ one step
     def _context(self) -> StepContext:
@@ -87,10 +99,18 @@ class DecodeSession:
     def _run(self) -> None:
         logits = self.engine.model.forward(self._context())
         self.sampler(logits, self.keys, self.steps, self.sampled, self.prev, self.n_prev)
-        ops.advance(self.token_ids, self.sampled, self.positions, self.steps)
+        ops.advance(self.token_ids, self.sampled, self.positions, self.steps, self.prev, self.n_prev, self.cursor)
 
     def step(self) -> List[int]:
         """Runs one token of every bound sequence and returns the next sampled tokens."""
+        return self.collect(self.launch())
+
+    def launch(self) -> int:
+        """Starts one step (the sampled token of the step before is fed back on the device) and
+        returns its handle without waiting for it.  At most two steps may be outstanding, so
+        the host can start step n + 1 before it has looked at the tokens of step n."""
+        if self._launched - self._collected >= 2:
+            raise RuntimeError("two decode steps are already in flight")
         cache = self.engine.cache
         new_len = {s: cache.length(s) + 1 for s in self.slots}
         if max(new_len.values()) > self.max_len:
@@ -122,6 +142,26 @@ class DecodeSession:
                 self._run()
             self.graph = graph
             graph.replay()
-        tokens = self.sampled.cpu().tolist()
+        k = self._launched % 2
+        if self._pinned is not None:
+            self._pinned[k].copy_(self.sampled, non_blocking=True)
+            self._events[k].record()
+        else:
+            self._host_out[k] = self.sampled.cpu().tolist()
         cache.commit(new_len)
+        self._launched += 1
+        return self._launched - 1
+
+    def collect(self, handle: int) -> List[int]:
+        """The sampled tokens of a launched step, in the order of the bound sequences; steps are
+        collected in the order they were launched."""
+        if handle != self._collected or handle >= self._launched:
+            raise RuntimeError(f"decode step {handle} is not the next one to collect")
+        k = handle % 2
+        if self._pinned is not None:
+            self._events[k].synchronize()
+            tokens = self._pinned[k].tolist()
+        else:
+            tokens = self._host_out[k]
+        self._collected += 1
         return tokens

@@ -91,15 +91,18 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: Optional[Sampling
     result.batches = plan_batches([len(p) for p in prompts], max_new, capacity, max_batch, limit)
     dev = engine.device
 
-    def decide(req: int, tok: int, slot: int, live: Dict[int, int]) -> None:
-        """After sampling `tok` for request `req`: stop, emit, or emit and end."""
+    def decide(req: int, tok: int, slot: int, live: Dict[int, int], length: Optional[int] = None) -> None:
+        """After sampling `tok` for request `req`: stop, emit, or emit and end.  `length` is what
+        the sequence held after the step that gave `tok` (default: what it holds now)."""
+        if length is None:
+            length = engine.length(slot)
         if tok in stops:
             result.finish_reasons[req] = "stop"
         else:
             result.tokens[req].append(tok)
             if on_token:
                 on_token(req, tok)
-            if len(result.tokens[req]) < max_new and engine.length(slot) + 1 <= limit:
+            if len(result.tokens[req]) < max_new and length + 1 <= limit:
                 live[req] = slot
                 return
             result.finish_reasons[req] = "length"
@@ -122,32 +125,70 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: Optional[Sampling
         next_tok = {r: result.tokens[r][-1] for r in live}
 
         t0 = time.perf_counter()
-        session, bound = None, None
         while live:
             order = sorted(live)
             if use_graph and hasattr(engine, "decode_session"):
-                if bound != order:
-                    cap = max(min(len(prompts[r]) + max_new, limit) for r in order)
-                    session = engine.decode_session(len(order), cap, sampler)
-                    session.bind([live[r] for r in order], [next_tok[r] for r in order], order,
-                                 [len(result.tokens[r]) for r in order])
-                    bound = order
-                if params.has_penalties:
-                    session.set_windows([windows[r] for r in order])
-                toks = session.step()
+                live = _decode_bound(engine, sampler, params, order, live, next_tok, windows, prompts, result,
+                                     max_new, limit, decide)
             else:
                 logits = engine.step([live[r] for r in order], [[next_tok[r]] for r in order], "last")
                 toks = _sample(sampler, logits, order, [len(result.tokens[r]) for r in order],
                                [windows[r] for r in order], dev)
-            result.decode_tokens += len(order)
-            was, live = live, {}
-            for r, tok in zip(order, toks):
-                windows[r] = (windows[r] + [tok])[-REPEAT_LAST_N:]
-                decide(r, tok, was[r], live)
+                result.decode_tokens += len(order)
+                was, live = live, {}
+                for r, tok in zip(order, toks):
+                    windows[r] = (windows[r] + [tok])[-REPEAT_LAST_N:]
+                    decide(r, tok, was[r], live)
             next_tok = {r: result.tokens[r][-1] for r in live}
         _sync(engine)
         result.decode_seconds += time.perf_counter() - t0
     return result
+
+
+def _decode_bound(engine, sampler, params, order, live, next_tok, windows, prompts, result, max_new, limit,
+                  decide) -> Dict[int, int]:
+    """Decodes the requests in `order` as one bound set until one of them ends, and returns the
+    requests still alive.  The step after the one whose tokens the host is about to read is
+    started first whenever no request can end by length in between: the device never waits
+    for the host.  A request that ends on a stop token then has one more step in flight; its
+    result is dropped, and what that step wrote into the cache goes with the sequence."""
+    cap = max(min(len(prompts[r]) + max_new, limit) for r in order)
+    session = engine.decode_session(len(order), cap, sampler)
+    session.bind([live[r] for r in order], [next_tok[r] for r in order], order,
+                 [len(result.tokens[r]) for r in order])
+    if params.has_penalties:
+        session.set_windows([windows[r] for r in order])
+    slots = dict(live)
+    alive = set(order)
+    held = {r: engine.length(slots[r]) for r in order}      # tokens in the cache after the step taken last
+
+    def take(tokens) -> None:
+        """The tokens of one step, for the requests that had not ended before it."""
+        now: Dict[int, int] = {}
+        for r, tok in zip(order, tokens):
+            if r not in alive:
+                continue
+            held[r] += 1
+            result.decode_tokens += 1
+            windows[r] = (windows[r] + [tok])[-REPEAT_LAST_N:]
+            decide(r, tok, slots[r], now, held[r])
+        alive.intersection_update(now)
+
+    pending = session.launch()
+    while True:
+        ahead = None
+        # `pending` has been launched and not taken: it will bring every request to
+        # len + 1 tokens and held + 1 positions; one more step must be allowed after that
+        if all(len(result.tokens[r]) + 1 < max_new and held[r] + 2 <= limit for r in order):
+            ahead = session.launch()
+        take(session.collect(pending))
+        if ahead is None:
+            break
+        if len(alive) < len(order):       # somebody ended: finish the step in flight, then rebind
+            take(session.collect(ahead))
+            break
+        pending = ahead
+    return {r: slots[r] for r in order if r in alive}
 
 
 def _sample(sampler: Sampler, logits: torch.Tensor, keys: Sequence[int], steps: Sequence[int],

@@ -69,7 +69,7 @@ _PROTOTYPES = {
         "mf_penalties": [_P, c_int, c_int, c_int, _P, c_int, _P, c_float, c_float, c_float, _P],
         "mf_top_k": [_P, c_int, c_int, c_int, c_int, _P],
         "mf_top_p": [_P, c_int, c_int, c_int, c_float, _P],
-        "mf_advance": [_P, _P, _P, _P, c_int, _P],
+        "mf_advance": [_P, _P, _P, _P, c_int, _P, c_int, _P, _P, _P],
     },
 }
 _functions: Dict[str, object] = {}
@@ -548,10 +548,23 @@ def top_p(logits: torch.Tensor, p: float) -> None:
     _check(_fn("sampling", "mf_top_p")(_ptr(logits), vocab, rows, vocab, float(p), _stream()), "top_p")
 
 
-def advance(next_ids: torch.Tensor, sampled: torch.Tensor, positions: torch.Tensor,
-            steps: torch.Tensor) -> None:
+def advance(next_ids: torch.Tensor, sampled: torch.Tensor, positions: torch.Tensor, steps: torch.Tensor,
+            prev: Optional[torch.Tensor] = None, n_prev: Optional[torch.Tensor] = None,
+            cursor: Optional[torch.Tensor] = None) -> None:
+    """After a decode step: next_ids = sampled, positions and steps move on by one; with `prev`
+    `[n][window]` the sampled token also enters the window of recent tokens (n_prev entries in
+    use, cursor = where the next one goes)."""
     n = next_ids.numel()
     for name, t in (("next_ids", next_ids), ("sampled", sampled), ("positions", positions), ("steps", steps)):
         _need(t, "advance." + name, torch.int32, (n,))
+    max_prev = 0
+    if prev is not None:
+        _need(prev, "advance.prev", torch.int32)
+        if prev.dim() != 2 or prev.shape[0] != n:
+            raise KernelError(f"advance.prev: shape {tuple(prev.shape)}, expected [{n}, window]")
+        max_prev = prev.shape[1]
+        _need(n_prev, "advance.n_prev", torch.int32, (n,))
+        _need(cursor, "advance.cursor", torch.int32, (n,))
     _check(_fn("sampling", "mf_advance")(_ptr(next_ids), _ptr(sampled), _ptr(positions), _ptr(steps), n,
-                                          _stream()), "advance")
+                                          _ptr(prev), max_prev, _ptr(n_prev if prev is not None else None),
+                                          _ptr(cursor if prev is not None else None), _stream()), "advance")

@@ -220,10 +220,16 @@ def top_p(logits, p):
         logits[i] = torch.from_numpy(pq.apply_top_p(logits[i].numpy(), p))
 
 
-def advance(next_ids, sampled, positions, steps):
+def advance(next_ids, sampled, positions, steps, prev=None, n_prev=None, cursor=None):
     next_ids.copy_(sampled)
     positions += 1
     steps += 1
+    if prev is not None:
+        for i in range(next_ids.numel()):
+            c = int(cursor[i])
+            prev[i, c] = sampled[i]
+            cursor[i] = (c + 1) % prev.shape[1]
+            n_prev[i] = min(int(n_prev[i]) + 1, prev.shape[1])
 
 
 NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", "rope_table",

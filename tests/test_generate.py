@@ -161,6 +161,40 @@ def test_real_engine_on_cpu_matches_plain_generation(tmp_path, name, use_graph):
     assert not llm.engine.cache.live_slots()
 
 
+def test_running_ahead_drops_what_follows_a_stop_and_respects_lengths(tmp_path):
+    """The decode loop starts step n + 1 before it reads the tokens of step n.  A request that
+    stops at step n then has a step in flight: nothing of it may show, the others must not
+    notice, and no request may run past max_new or the context bound because of it."""
+    from minfer_amd import LLM
+    folder = write_tiny(tmp_path, "A", seed=4)
+    vocab = TINIES["A"]["vocab_size"]
+    llm = LLM(folder, dtype="float32", device="cpu", n_ctx=128, n_slots=4)
+    prompts = [random_tokens(vocab, n, 10 + i) for i, n in enumerate((4, 7, 2, 9))]
+    free = llm.generate(prompts, max_new=9, temp=0.0, stop_tokens=[]).tokens
+    assert all(len(t) == 9 for t in free)
+    # a token that request 1 produces in the middle and that the others do not produce earlier
+    for k in range(2, 8):
+        stop = free[1][k]
+        first_hit = [t.index(stop) if stop in t else 99 for t in free]
+        if first_hit[1] == k:
+            break
+    res = llm.generate(prompts, max_new=9, temp=0.0, stop_tokens=[stop])
+    for i, got in enumerate(res.tokens):
+        cut = first_hit[i]
+        assert got == free[i][:cut], i
+        assert res.finish_reasons[i] == ("stop" if cut < 9 else "length")
+    llm.engine.cache.check_invariants()
+    assert not llm.engine.cache.live_slots()
+    # the context bound: prompt + generated never exceeds n_ctx, and every request gets all it may
+    small = LLM(folder, dtype="float32", device="cpu", n_ctx=12, n_slots=4)
+    res = small.generate(prompts, max_new=50, temp=0.0, stop_tokens=[])
+    for p, got in zip(prompts, res.tokens):
+        assert len(got) == 12 - len(p) + 1          # one from the prompt's step, one per free position
+        assert got == llm.generate([p], max_new=len(got), temp=0.0, stop_tokens=[], use_graph=False).tokens[0]
+    assert res.finish_reasons == ["length"] * 4
+    assert not small.engine.cache.live_slots()
+
+
 def test_step_errors_leave_the_cache_alone(tmp_path):
     from minfer_amd import LLM, StepError
     from minfer_amd.cache import CacheFull

@@ -148,3 +148,36 @@ def test_pipeline_order_and_greedy_with_penalty():
                     torch.full((rows,), 20, dtype=torch.int32, device=DEV))
     want = [pq.sample(base[i].numpy(), 0.7, uniform(9, i, 3), 40, 0.9, 1.3, 0.2, 0.1, windows[i]) for i in range(rows)]
     assert out.cpu().tolist() == want
+
+
+def test_advance_feeds_back_and_keeps_the_recent_window(ops):
+    """After a step the sampled token is the next input, positions and steps move on, and the
+    token enters the window of recent tokens: appended while there is room, over the oldest
+    afterwards; the penalties then see exactly the last `window` tokens."""
+    import plain_ops
+    n, window = 3, 4
+    next_ids = torch.zeros(n, dtype=torch.int32)
+    positions = torch.tensor([5, 0, 70], dtype=torch.int32)
+    steps = torch.tensor([1, 0, 9], dtype=torch.int32)
+    prev = torch.zeros(n, window, dtype=torch.int32)
+    prev[0, :2] = torch.tensor([7, 8], dtype=torch.int32)
+    prev[2] = torch.tensor([1, 2, 3, 4], dtype=torch.int32)
+    n_prev = torch.tensor([2, 0, 4], dtype=torch.int32)
+    cursor = torch.tensor([2, 0, 0], dtype=torch.int32)
+    dev = [t.to(DEV) for t in (next_ids, positions, steps, prev, n_prev, cursor)]
+    cpu = [t.clone() for t in (next_ids, positions, steps, prev, n_prev, cursor)]
+    history = [[7, 8], [], [1, 2, 3, 4]]
+    for step in range(6):
+        sampled = torch.tensor([10 + step, 20 + step, 30 + step], dtype=torch.int32)
+        ops.advance(dev[0], sampled.to(DEV), dev[1], dev[2], dev[3], dev[4], dev[5])
+        plain_ops.advance(cpu[0], sampled, cpu[1], cpu[2], cpu[3], cpu[4], cpu[5])
+        for a, b in zip(dev, cpu):
+            assert torch.equal(a.cpu(), b)
+        for i in range(n):
+            history[i].append(int(sampled[i]))
+            got = sorted(dev[3][i, :int(dev[4][i])].cpu().tolist())
+            assert got == sorted(history[i][-window:])
+    assert dev[0].cpu().tolist() == [15, 25, 35] and dev[1].cpu().tolist() == [11, 6, 76]
+    # without a window nothing but ids, positions and steps is touched
+    ops.advance(dev[0], dev[0].clone(), dev[1], dev[2])
+    assert dev[1].cpu().tolist() == [12, 7, 77]
