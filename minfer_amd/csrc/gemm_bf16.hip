@@ -152,20 +152,28 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const 
     if (more) load_tile(kt + 1);
     const bf16* as = As + cur * BM * LDS_LD;
     const bf16* ws = Ws + cur * BN * LDS_LD;
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      bf16x8 fa[TM], fw[TN];
+    // The fragments of k-step ks + 1 are asked for before the products of k-step ks are issued,
+    // into the other half of fa / fw, so the matrix cores do not wait for LDS inside a tile.
+    bf16x8 fa[2][TM], fw[2][TN];
+    auto read_frags = [&](int ks, int h) {
 #pragma unroll
       for (int i = 0; i < TM; ++i)
-        fa[i] = *reinterpret_cast<const bf16x8*>(&as[(wm + i * 32 + fr) * LDS_LD + ks * 16 + fk]);
+        fa[h][i] = *reinterpret_cast<const bf16x8*>(&as[(wm + i * 32 + fr) * LDS_LD + ks * 16 + fk]);
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        fw[j] = *reinterpret_cast<const bf16x8*>(&ws[(wn + j * 32 + fr) * LDS_LD + ks * 16 + fk]);
+        fw[h][j] = *reinterpret_cast<const bf16x8*>(&ws[(wn + j * 32 + fr) * LDS_LD + ks * 16 + fk]);
+    };
+    read_frags(0, 0);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      if (ks + 1 < BK / 16) read_frags(ks + 1, (ks + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][i], fw[ks & 1][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (more) {
       bf16* an = As + (cur ^ 1) * BM * LDS_LD;
