@@ -58,6 +58,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       qf[ks] = *reinterpret_cast<const bf16x8*>(q + ((size_t)(tok0 + qi) * nh + h) * HD + ks * 16 + hf * 8);
   }
   // positions this wave and this block need
+  const float sl2 = scale * 1.44269504088896340736f;    // scores -> exponents of 2
+  const bool wave_q_last_ok = q0 + wid * 32 + 31 < n_new;   // all 32 queries of the wave exist
   const int wave_q_last = min(q0 + wid * 32 + 31, n_new - 1);
   const int wave_p_hi = start + wave_q_last;
   const int wave_p_lo = start + q0 + wid * 32;
@@ -145,19 +147,29 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s[kt], 0, 0, 0);
       }
     }
-    // mask, running maximum: reg r of tile kt is key key0 + 32 kt + 8 (r / 4) + 4 hf + r % 4
+    // Mask, running maximum: reg r of tile kt is key key0 + 32 kt + 8 (r / 4) + 4 hf + r % 4.
+    // Scores stay unscaled; the maximum is kept in units of scale * log2(e), so that
+    // exp((s - m) scale) is one fused multiply-add and one 2^x per score.  A page that every
+    // query of the wave sees whole needs no mask.
     float m_new = m_run;
+    const bool whole = key0 + KT - 1 <= wave_p_lo && wave_q_last_ok && (window <= 0 || key0 > wave_p_hi - window);
+    if (whole) {
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
+      for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = key0 + kt * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
-        const bool vis = q_ok && key <= pq && (window <= 0 || key > pq - window);
-        s[kt][r] = vis ? s[kt][r] * scale : -INFINITY;
-        m_new = fmaxf(m_new, s[kt][r]);
-      }
+        for (int r = 0; r < 16; ++r) m_new = fmaxf(m_new, s[kt][r] * sl2);
+    } else {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = key0 + kt * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
+          const bool vis = q_ok && key <= pq && (window <= 0 || key > pq - window);
+          s[kt][r] = vis ? s[kt][r] : -INFINITY;
+          m_new = fmaxf(m_new, s[kt][r] * sl2);
+        }
+    }
     m_new = fmaxf(m_new, __shfl_xor(m_new, 32, MF_WAVE));
-    const float corr = (m_new == -INFINITY) ? 1.f : __expf(m_run - m_new);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
     float psum = 0.f;
     bf16x8 pb[4];
@@ -165,16 +177,21 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float pe = __expf(s[kt][r] - m_use);       // exp(-inf) = 0 for masked keys
+        const float pe = __builtin_amdgcn_exp2f(fmaf(s[kt][r], sl2, -m_use));    // 2^(-inf) = 0 for masked keys
         psum += pe;
         pb[kt * 2 + (r >> 3)][r & 7] = (bf16)pe;
       }
-    l_run = l_run * corr + psum;
-    m_run = m_new;
+    // the accumulators are rescaled only when some query's maximum moved
+    if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+      const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
+      l_run *= corr;
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt)
+      for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[dt][r] *= corr;
+        for (int r = 0; r < 16; ++r) oacc[dt][r] *= corr;
+      m_run = m_new;
+    }
+    l_run += psum;
     // O^T += V^T P^T; operand element e of group kg is key 16 kg + 8 (e / 4) + 4 hf + e % 4
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)

@@ -476,6 +476,8 @@ def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pa
     _need(out, "attn_prefill.out", torch.bfloat16, (n_tok, n_heads * head_dim))
     _need_caches("attn_prefill", kcache, vcache, torch.bfloat16, n_kv_heads, head_dim)
     _need(page_table, "attn_prefill.page_table", torch.int32)
+    if not scale > 0.0:
+        raise KernelError(f"attn_prefill: scale {scale} must be positive")
     _need(ctx.cu_seqlens, "attn_prefill.cu_seqlens", torch.int32, (ctx.n_seqs + 1,))
     _need(ctx.start_pos, "attn_prefill.start_pos", torch.int32, (ctx.n_seqs,))
     if head_dim % 16 or not 16 <= head_dim <= 256:
