@@ -251,3 +251,170 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
     compare(run_steps(eng, whole_steps(requests)), ref, dtype, "toy whole")
     compare(run_steps(eng, tail_steps(requests, tail=8)), ref, dtype, "toy one by one")
     compare(run_steps(eng, batch_steps(requests, [ids[:3], ids[3:]])), ref, dtype, "toy batches")   # slots used again
+
+
+# ------------------------------------------------------------------ more toy parts
+# A feed-forward with routing, a position encoding that is not a rotation, a norm without a
+# weight and a post-norm block, all defined here and put into one model: the registries, the
+# loader, the cache, the step and the replays take them as they come.
+from minfer_amd.parts import (Block, FeedForward, Norm, PositionEncoding, register_block,      # noqa: E402
+                              register_feed_forward, register_norm, register_position)
+
+
+@register_feed_forward("toy_top1_experts")
+class ToyTop1Experts(FeedForward):
+    """Router logits r = R x in 32-bit; the expert with the largest logit (the first on a tie)
+    runs y = W2 relu(W1 x), weighted by the softmax probability of its logit."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        p = spec.params
+        self.hidden, self.inter, self.n_experts = int(p["hidden_size"]), int(p["intermediate_size"]), int(p["experts"])
+
+    def tensor_specs(self):
+        out = {"router.weight": TensorSpec((self.n_experts, self.hidden))}
+        for e in range(self.n_experts):
+            out[f"e{e}.w1"] = TensorSpec((self.inter, self.hidden))
+            out[f"e{e}.w2"] = TensorSpec((self.hidden, self.inter))
+        return out
+
+    def load(self, get):
+        self.router = get("router.weight").float()
+        self.w1 = [get(f"e{e}.w1").float() for e in range(self.n_experts)]
+        self.w2 = [get(f"e{e}.w2").float() for e in range(self.n_experts)]
+
+    def forward(self, x, h, ctx):
+        x = x.float()
+        logits = x @ self.router.t()
+        prob = torch.softmax(logits, dim=-1)
+        pick = torch.argmax(logits, dim=-1)
+        for e in range(self.n_experts):
+            rows = torch.nonzero(pick == e).flatten()
+            if rows.numel():
+                y = torch.relu(x[rows] @ self.w1[e].t()) @ self.w2[e].t()
+                h[rows] += y * prob[rows, e:e + 1]
+
+
+@register_position("toy_position_bias")
+class ToyPositionBias(PositionEncoding):
+    """No rotation: position p adds p * slope to the first element of every q and k head."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.head_dim, self.slope = int(spec.params["head_dim"]), float(spec.params["slope"])
+
+    def rotate_and_store(self, qkv, ctx, q_out, kcache, vcache, page_table, n_heads, n_kv_heads, write_kv):
+        t, hd = qkv.shape[0], self.head_dim
+        x = qkv.view(t, n_heads + 2 * n_kv_heads, hd).clone()
+        bump = ctx.positions.float() * self.slope
+        x[:, :n_heads + n_kv_heads, 0] += bump[:, None]
+        q_out.copy_(x[:, :n_heads].reshape(t, n_heads * hd).to(q_out.dtype))
+        if not write_kv:
+            return
+        pos = ctx.positions.long()
+        page = page_table.long()[ctx.seq_of_tok.long(), pos // 64]
+        k, v = x[:, n_heads:n_heads + n_kv_heads], x[:, n_heads + n_kv_heads:]
+        kcache[page, :, pos % 64, :] = k.to(kcache.dtype)
+        if vcache.shape[-1] == 64 and vcache.dtype == torch.bfloat16:      # a bfloat16 page of V is [hd][64]
+            vcache[page, :, :, pos % 64] = v.to(vcache.dtype)
+        else:
+            vcache[page, :, pos % 64, :] = v.to(vcache.dtype)
+
+
+@register_norm("toy_scale_norm")
+class ToyScaleNorm(Norm):
+    """y = x / (mean |x| + eps): no weight, not an RMS norm, so nothing folds it into a product."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.eps = float(spec.params["eps"])
+
+    def forward(self, h, out=None, row_idx=None):
+        src = h if row_idx is None else h[row_idx.long()]
+        y = (src / (src.abs().mean(dim=-1, keepdim=True) + self.eps)).to(self.rt.dtype)
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+
+
+@register_block("toy_postnorm")
+class ToyPostNormBlock(Block):
+    """h <- norm1(h + mixer(h)); h <- norm2(h + feed_forward(h)): the parts get the residual
+    stream itself as their input."""
+
+    def forward(self, h, ctx, entry, writes_cache, keep_rows=None):
+        self.mixer.forward(h.to(self.rt.dtype), h, ctx, entry, writes_cache)
+        h.copy_(self.mixer_norm.forward(h).float())
+        if keep_rows is not None:
+            h = h[keep_rows.long()].contiguous()
+        self.feed_forward.forward(h.to(self.rt.dtype), h, ctx)
+        h.copy_(self.feed_forward_norm.forward(h).float())
+        return h
+
+
+class ToyRoutedConfig(ToyConfig):
+    def model_spec(self):
+        hid = self.hidden
+        snorm = lambda: PartSpec("toy_scale_norm", dict(eps=1e-3))
+        pos = PartSpec("toy_position_bias", dict(head_dim=16, slope=0.01))
+        attn = PartSpec("gqa_attention", dict(hidden_size=hid, n_heads=4, n_kv_heads=2, head_dim=16, scale=0.25, window=None,
+                                              qkv_bias=True, out_bias=False, position=pos, q="a.q", k="a.k", v="a.v", o="a.o"))
+        moe = PartSpec("toy_top1_experts", dict(hidden_size=hid, intermediate_size=24, experts=3))
+        blocks = (BlockSpec("toy_postnorm", "l0.", attn, moe, snorm(), snorm()),
+                  BlockSpec("toy_postnorm", "l1.", attn, moe, snorm(), snorm()))
+        return ModelSpec(hidden_size=hid, vocab_size=self.vocab, embedding_name="emb", head_name="head",
+                         final_norm=PartSpec("rmsnorm", dict(size=hid, eps=1e-5, weight="nf")), blocks=blocks,
+                         schedule=(RunEntry(0, 0), RunEntry(1, 1)), max_positions=256)
+
+
+class PlainRouted:
+    def __init__(self, folder):
+        from safetensors.torch import load_file
+        self.w = {k: v.double().numpy() for k, v in load_file(folder + "/model.safetensors").items()}
+
+    @staticmethod
+    def snorm(h):
+        return h / (np.abs(h).mean(axis=-1, keepdims=True) + 1e-3)
+
+    def forward(self, tokens):
+        w, pos = self.w, np.arange(len(tokens))
+        h = w["emb"][tokens]
+        for p in ("l0.", "l1."):
+            q = pq.linear(h, w[p + "a.q.weight"], w[p + "a.q.bias"]).reshape(len(tokens), 4, 16)
+            k = pq.linear(h, w[p + "a.k.weight"], w[p + "a.k.bias"]).reshape(len(tokens), 2, 16)
+            v = pq.linear(h, w[p + "a.v.weight"], w[p + "a.v.bias"])
+            q[:, :, 0] += pos[:, None] * 0.01
+            k[:, :, 0] += pos[:, None] * 0.01
+            a = pq.gqa_attention(q.reshape(len(tokens), -1), k.reshape(len(tokens), -1), v, pos, pos, 4, 2, 16, 0.25)
+            h = self.snorm(h + pq.linear(a, w[p + "a.o.weight"]))
+            logits = h @ w[p + "router.weight"].T
+            prob = np.exp(logits - logits.max(axis=-1, keepdims=True))
+            prob /= prob.sum(axis=-1, keepdims=True)
+            out = np.zeros_like(h)
+            for t in range(len(tokens)):
+                e = int(np.argmax(logits[t]))
+                out[t] = (w[p + f"e{e}.w2"] @ np.maximum(w[p + f"e{e}.w1"] @ h[t], 0.0)) * prob[t, e]
+            h = self.snorm(h + out)
+        return pq.rms_norm(h, w["nf"], 1e-5) @ w["head"].T
+
+
+def test_toy_routing_position_norm_and_block_parts(tmp_path):
+    """32-bit only: a routing decision is a jump, and bfloat16 rounding would move tokens that
+    sit on one across it; the architecture's own bfloat16 runs are covered elsewhere."""
+    from minfer_amd import Engine, load_model, register_architecture, write_random_model
+    register_architecture("ToyRoutedLM", ToyRoutedConfig)
+    cfg = ToyRoutedConfig(dict(architectures=["ToyRoutedLM"], hidden_size=40, vocab_size=211))
+    folder = write_random_model(str(tmp_path / "routed"), cfg, seed=5)
+    model = load_model(folder, dtype="float32")
+    assert "l1.e2.w2" in model.expected_tensors() and "l0.router.weight" in model.expected_tensors()
+    eng = Engine(model, max_tokens=64 * 6, max_seqs=3, poison_cache=True)
+    plain = PlainRouted(folder)
+    requests = requests_for(211, (6, 67, 30, 11), seed=6)
+    ref = {r: plain.forward(t) for r, t in requests.items()}
+    picks = [int(np.argmax(plain.w["emb"][t] @ plain.w["l0.router.weight"].T, axis=-1).max()) for t in requests.values()]
+    assert max(picks) >= 1, "the routing is exercised: not every token goes to expert 0"
+    ids = list(requests)
+    compare(run_steps(eng, whole_steps(requests)), ref, "float32", "routed whole")
+    compare(run_steps(eng, tail_steps(requests, tail=8)), ref, "float32", "routed one by one")
+    compare(run_steps(eng, batch_steps(requests, [ids[:3], ids[3:]])), ref, "float32", "routed batches")
