@@ -122,12 +122,18 @@ _FLOATS = (torch.float32, torch.bfloat16)
 _workspaces: Dict[Tuple[str, int], torch.Tensor] = {}
 
 
+_retired: list = []
+
+
 def workspace(tag: str, n_floats: int, device) -> torch.Tensor:
     """A float32 scratch tensor of at least n_floats, kept per (tag, device) and grown when
-    needed.  Kernels that use one run in stream order, so sharing it is safe."""
+    needed.  Kernels that use one run in stream order, so sharing it is safe.  A tensor that
+    was outgrown is kept alive: a captured graph may still hold its address."""
     key = (tag, torch.device(device).index or 0)
     w = _workspaces.get(key)
     if w is None or w.numel() < n_floats:
+        if w is not None:
+            _retired.append(w)
         w = torch.empty(max(n_floats, 1 << 16), dtype=torch.float32, device=device)
         _workspaces[key] = w
     return w

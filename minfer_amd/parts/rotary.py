@@ -25,6 +25,7 @@ class RotaryNeoX(PositionEncoding):
         if self.head_dim % 2:
             raise ValueError(f"rope_neox: head_dim {self.head_dim} is odd")
         self.cos = self.sin = None
+        self._outgrown = []            # earlier tables: a captured graph may still hold their addresses
 
     def prepare(self, max_len: int) -> None:
         if max_len > self.max_positions:
@@ -32,6 +33,8 @@ class RotaryNeoX(PositionEncoding):
         have = 0 if self.cos is None else self.cos.shape[0]
         if max_len > have:
             n = min(self.max_positions, max(256, 1 << (max_len - 1).bit_length()))
+            if self.cos is not None:
+                self._outgrown.append((self.cos, self.sin))
             self.cos, self.sin = ops.rope_table(n, self.head_dim // 2, self.theta, self.freq_scale,
                                                 self.rt.device)
 

@@ -111,6 +111,29 @@ def test_first_tokens_of_a_sequence(folders, dtype):
     compare(run_steps(eng, steps), ref, dtype, "first tokens")
 
 
+def test_captured_steps_survive_growth_of_shared_scratch(folders):
+    """A captured decode step holds the addresses of the shared scratch buffers and of the
+    rotation table.  When a later, larger job makes them grow, the earlier graphs must go on
+    working: what was outgrown stays allocated."""
+    import torch
+    from minfer_amd import LLM
+    from minfer_amd.kernels import ops
+    vocab = TINIES["C"]["vocab_size"]
+    llm = LLM(folders["C"], dtype="bfloat16", n_ctx=1024, n_slots=4)
+    prompts = [random_tokens(vocab, n, 40 + i) for i, n in enumerate((30, 70))]
+    first = llm.generate(prompts, max_new=12, temp=0.0, stop_tokens=[]).tokens       # captures graphs for 2 sequences
+    held = {k: v for k, v in ops._workspaces.items()}
+    for (tag, dev), w in held.items():                    # somebody needs more of every scratch buffer
+        ops.workspace(tag, w.numel() * 2 + 1, w.device)
+    junk = [torch.full((w.numel(),), float("nan"), device=w.device) for w in held.values()]   # would land in freed blocks
+    long_prompt = [random_tokens(vocab, 700, 50)]
+    llm.generate(long_prompt, max_new=4, temp=0.0, stop_tokens=[])        # a longer sequence: the rotation table grows
+    again = llm.generate(prompts, max_new=12, temp=0.0, stop_tokens=[]).tokens       # the old graphs replay
+    eager = llm.generate(prompts, max_new=12, temp=0.0, stop_tokens=[], use_graph=False).tokens
+    assert again == first == eager
+    del junk
+
+
 def test_command_line(folders, tmp_path):
     env = dict(os.environ, PYTHONPATH=ROOT)
     exe = [sys.executable, os.path.join(ROOT, "bin", "minfer")]
