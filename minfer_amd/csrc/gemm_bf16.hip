@@ -72,6 +72,47 @@ __device__ __forceinline__ bf16x8 load8_inside(const bf16* __restrict__ base, in
   return *reinterpret_cast<const bf16x8*>(base + (size_t)row * ld + k);
 }
 
+// The epilogue of a wave's TM x TN tiles of 32 x 32 (D[m][n]: lane holds n = lane % 32,
+// m = 8 (r / 4) + 4 (lane / 32) + r % 4): bias, then store / accumulate / round / SwiGLU.
+template <int TM, int TN>
+__device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[TM][TN], const float* __restrict__ bias,
+                                              void* __restrict__ C, int ldc, int M, int N, int epi, int m0,
+                                              int wm, int n0, int wn, int lane) {
+  const int fr = lane & 31;
+  // D[m][n]: lane holds n = lane % 32, m = 8 (r / 4) + 4 (lane / 32) + r % 4
+  if (epi == EPI_SWIGLU) {
+    if constexpr (TN % 2 == 0) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; j += 2) {
+          const int ng = n0 + wn + j * 32 + fr;            // gate column; its up column is ng + 32
+          const int col = (ng >> 6) * 32 + (ng & 63);
+          if (col >= ldc) continue;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int m = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            if (m < M) ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(acc[i][j][r], acc[i][j + 1][r]);
+          }
+        }
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn + j * 32 + fr;
+      if (n >= N) continue;
+      const float b = bias ? bias[n] : 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        if (m < M) store_out(C, ldc, m, n, acc[i][j][r] + b, epi);
+      }
+    }
+}
+
 // ------------------------------------------------------------------ tiled kernel
 // LDS row stride is BK + 8 elements (144 bytes for BK 64, 80 for BK 32): conflict-free b128 reads
 template <int BM, int BN, int WM, int WN, int BK, bool VEC>
@@ -188,38 +229,177 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const 
     __syncthreads();
   }
 
-  // D[m][n]: lane holds n = lane % 32, m = 8 (r / 4) + 4 (lane / 32) + r % 4
-  if (epi == EPI_SWIGLU) {
-    if constexpr (TN % 2 == 0) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; j += 2) {
-          const int ng = n0 + wn + j * 32 + fr;            // gate column; its up column is ng + 32
-          const int col = (ng >> 6) * 32 + (ng & 63);
-          if (col >= ldc) continue;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int m = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-            if (m < M) ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(acc[i][j][r], acc[i][j + 1][r]);
-          }
-        }
-    }
-    return;
+  tile_epilogue<TM, TN>(acc, bias, C, ldc, M, N, epi, m0, wm, n0, wn, lane);
+}
+
+// ------------------------------------------------------------------ tiled kernel, loads straight into LDS
+// The same 256 x 256 tile on 8 waves (each 128 x 64), but k tiles of 32 travel global -> LDS
+// without passing registers (global_load_lds_dwordx4: lane i's 16 bytes land at the wave's LDS
+// base + 16 i), four stages deep, so that a tile's loads have three to four tiles of products to arrive
+// in instead of one, and the 32 staging registers are gone.  There is no room for
+// padding in such a copy, so a row's four 16-byte chunks are stored permuted: chunk c of row
+// r sits at position c ^ ((r >> 2) & 3), which spreads the 16 rows that one pass of a
+// 16-byte fragment read covers over all 64 banks (measured: no bank conflicts; with
+// (r >> 1) & 3, right for 32 banks, every read took twice as long).  Which chunk a lane fetches is free (its
+// global address), so the permutation costs nothing on the way in.
+//
+// The compiler does not know that these loads write LDS and so does not wait for them; the
+// kernel does, with vmcnt counts it keeps itself (4 loads per wave and tile, in order) and
+// one barrier per tile: after it, tile kt has landed for every wave, and the stage of tile
+// kt - 1, whose products all waves have issued, is free to take tile kt + stages - 1.
+// Needs 16-byte aligned rows and K a multiple of 32.
+constexpr int DMA_BM = 256, DMA_BN = 256, DMA_BK = 32, DMA_STAGES = 4;
+constexpr int DMA_STAGE_BYTES = (DMA_BM + DMA_BN) * DMA_BK * 2;
+
+__device__ __forceinline__ void dma16(const bf16* g, unsigned lds_byte) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte)
+               : "memory", "m0");
+}
+
+__global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ A, int lda,
+                                                       const bf16* __restrict__ W, int ldw,
+                                                       const float* __restrict__ bias, void* __restrict__ C,
+                                                       int ldc, int M, int N, int K, int epi, int tiles_m,
+                                                       int xcd_remap) {
+  constexpr int TM = 4, TN = 2;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  int tile = blockIdx.x;
+  if (xcd_remap) {
+    const int n_tiles = gridDim.x, per = n_tiles / 8, rem = n_tiles % 8;
+    const int x = blockIdx.x % 8, qq = blockIdx.x / 8;
+    tile = x * per + min(x, rem) + qq;
   }
+  const int bm = tile % tiles_m, bn = tile / tiles_m;
+  const int m0 = bm * DMA_BM, n0 = bn * DMA_BN;
+  const int lane = threadIdx.x & 63;
+  const int wid = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = (wid & 1) * 128, wn = (wid >> 1) * 64;
+  const int fr = lane & 31, fk = lane >> 5;
+
+  floatx16 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = n0 + wn + j * 32 + fr;
-      if (n >= N) continue;
-      const float b = bias ? bias[n] : 0.f;
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        if (m < M) store_out(C, ldc, m, n, acc[i][j][r] + b, epi);
-      }
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // this lane's share of a tile's copy: wave `wid` moves 1 KB blocks wid and 8 + wid (16 rows
+  // each) of the A tile and of the W tile; the lane fetches row 16 b + lane / 4, the chunk that
+  // belongs at position lane % 4
+  const unsigned lds0 = (unsigned)(uintptr_t)smem;
+  const bf16* ga[2];
+  const bf16* gw[2];
+  unsigned la[2], lw[2];
+#pragma unroll
+  for (int jj = 0; jj < 2; ++jj) {
+    const int b = jj * 8 + wid;
+    const int r = 16 * b + (lane >> 2);
+    const int chunk = (lane & 3) ^ ((r >> 2) & 3);
+    ga[jj] = A + (size_t)min(m0 + r, M - 1) * lda + chunk * 8;
+    gw[jj] = W + (size_t)min(n0 + r, N - 1) * ldw + chunk * 8;
+    la[jj] = lds0 + b * 1024;
+    lw[jj] = lds0 + DMA_BM * DMA_BK * 2 + b * 1024;
+  }
+  auto issue = [&](int kt) {
+    const unsigned st = (unsigned)(kt % DMA_STAGES) * DMA_STAGE_BYTES;
+    const int k = kt * DMA_BK;
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) dma16(ga[jj] + k, __builtin_amdgcn_readfirstlane(la[jj] + st));
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) dma16(gw[jj] + k, __builtin_amdgcn_readfirstlane(lw[jj] + st));
+  };
+  // fragment reads: row R of a tile, chunk ks * 2 + fk of its 4, at position chunk ^ ((R >> 2) & 3)
+  const int sw = (fr >> 2) & 3;
+  int offa[TM], offw[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) offa[i] = (wm + i * 32 + fr) * (DMA_BK * 2);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) offw[j] = DMA_BM * DMA_BK * 2 + (wn + j * 32 + fr) * (DMA_BK * 2);
+  const int pos0 = ((0 + fk) ^ sw) * 16, pos1 = ((2 + fk) ^ sw) * 16;
+
+  const int nkt = K / DMA_BK;
+  // Fragments of tile kt + 1 are read from LDS while the second half of tile kt's products runs,
+  // into the other register set: behind the barrier there is always work for the matrix cores.
+  bf16x8 fa[2][2][TM], fw[2][2][TN];          // [set][k-step][tile]
+  auto read_frags = [&](int stage, auto SET) {
+    constexpr int set = decltype(SET)::value;
+    const unsigned char* st = smem + stage * DMA_STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[set][0][i] = *reinterpret_cast<const bf16x8*>(st + offa[i] + pos0);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fw[set][0][j] = *reinterpret_cast<const bf16x8*>(st + offw[j] + pos0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[set][1][i] = *reinterpret_cast<const bf16x8*>(st + offa[i] + pos1);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fw[set][1][j] = *reinterpret_cast<const bf16x8*>(st + offw[j] + pos1);
+  };
+  auto multiply = [&](int ks, auto SET) {
+    constexpr int set = decltype(SET)::value;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][ks][i], fw[set][ks][j], acc[i][j], 0, 0, 0);
+  };
+  // wait until the loads of tile t (of this wave) have landed: at most those of the tiles
+  // issued after it may still be in flight, `issued` being the last tile asked for so far
+  auto wait_tile = [&](int t, int issued) {
+    const int later = issued - t;
+    if (later >= 3) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    else if (later == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if (later == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  };
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  int issued = -1;
+#pragma unroll
+  for (int t = 0; t < DMA_STAGES; ++t)
+    if (t < nkt) { issue(t); issued = t; }
+  wait_tile(0, issued);
+  __syncthreads();
+  read_frags(0, S0{});
+  int stage = 0;                               // of tile kt
+  // one round: tile kt from register set SET; in its middle the barrier that makes tile kt + 1
+  // readable and tile kt's stage free (every wave holds tile kt in registers by then)
+  auto round = [&](int kt, auto SET, auto OTHER) {
+    multiply(0, SET);
+    __builtin_amdgcn_sched_barrier(0);
+    if (kt + 1 < nkt) {
+      wait_tile(kt + 1, issued);
+      __syncthreads();
+      if (issued + 1 < nkt) { issue(issued + 1); ++issued; }      // into the stage of tile kt
+      const int next_stage = stage + 1 == DMA_STAGES ? 0 : stage + 1;
+      read_frags(next_stage, OTHER);
+      stage = next_stage;
     }
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(1, SET);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  for (int kt = 0; kt < nkt; kt += 2) {
+    round(kt, S0{}, S1{});
+    if (kt + 1 < nkt) round(kt + 1, S1{}, S0{});
+  }
+  tile_epilogue<TM, TN>(acc, bias, C, ldc, M, N, epi, m0, wm, n0, wn, lane);
+}
+
+int launch_tile_dma(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc, int M,
+                    int N, int K, int epi, hipStream_t stream) {
+  constexpr int smem = DMA_STAGES * DMA_STAGE_BYTES;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(tile_dma_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    configured = true;
+  }
+  const int tiles_m = (M + DMA_BM - 1) / DMA_BM, tiles_n = (N + DMA_BN - 1) / DMA_BN;
+  static const int remap = getenv("MF_NO_XCD_REMAP") ? 0 : 1;
+  tile_dma_kernel<<<tiles_m * tiles_n, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, tiles_m,
+                                                            remap && tiles_m * tiles_n >= 16);
+  return mf_launch_status();
 }
 
 template <int BM, int BN, int WM, int WN, int BK, bool VEC>
@@ -897,7 +1077,8 @@ int launch_skinny(const bf16* A, int lda, const bf16* W, int ldw, const float* b
 }  // namespace
 
 // `variant`: 0 picks by shape; 1: 256x256 tile with 4 waves, 2: 128x128, 3: 64x64, 6: 256x128
-// with 8 waves, 9: 256x256 with 8 waves (tests name them).
+// with 8 waves, 9: 256x256 with 8 waves, 12: 256x256 through the direct-to-LDS pipeline (tests
+// name them).
 MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
                         int ldc, int M, int N, int K, int epi, int variant, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -908,12 +1089,19 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
                      ((uintptr_t)W % 16 == 0) && (K % 8 == 0);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
+  const bool dma_ok = vec_ok && K % DMA_BK == 0;
   if (variant == 0) {
-    // measured at 2048 rows: 256x256 tiles (8 waves) win once there are several tiles per CU,
-    // 128x128 otherwise; tiny problems take 64x64
+    // 256x256 tiles run one block per CU at about 0.95 PFLOP/s through the direct-to-LDS pipeline
+    // (0.88 through registers), 128x128 tiles two blocks per CU at about 0.80: the number of
+    // rounds decides (measured at 512, 2048 and 8192 rows); tiny problems take 64x64
     const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
     const long t128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-    variant = (t256 >= 768) ? 9 : (t128 >= 64 || M > 64) ? 2 : 3;
+    const long slots = cu_count();
+    const double cost256 = (double)((t256 + slots - 1) / slots) * (256. * 256.) / (dma_ok ? 0.95 : 0.88);
+    const double cost128 = (t128 <= slots ? 1. : 2. * (double)((t128 + 2 * slots - 1) / (2 * slots))) *
+                           (128. * 128.) / 0.80;
+    if (cost256 < cost128) variant = dma_ok ? 12 : 9;
+    else variant = (t128 >= 64 || M > 64) ? 2 : 3;
   }
   if (epi == EPI_SWIGLU && variant == 3) variant = 2;      // needs two 32-column tiles per wave
   switch (variant) {
@@ -922,6 +1110,9 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
     case 3: return launch_tile<64, 64, 32, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case 6: return launch_tile<256, 128, 64, 64, 32>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case 9: return launch_tile<256, 256, 128, 64, 64>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case 12:
+      if (!dma_ok) return (int)hipErrorInvalidValue;
+      return launch_tile_dma(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
   }
   return (int)hipErrorInvalidValue;
 }
