@@ -527,6 +527,84 @@ __global__ __launch_bounds__(512) void skinny_kernel(const bf16* __restrict__ A,
     }
 }
 
+// The same product where every chunk is whole (K and the splits in multiples of 256, aligned rows),
+// as a ring: each wave keeps its 8 weight fragments of a chunk in registers and refills one right
+// behind the MFMA that used it, with the next chunk's, so the loads in flight never run dry at a
+// chunk's end as they do above; the sums leave through an LDS tile, in rows of 512 bytes.
+constexpr int SR_LD = 128 + 4;      // row stride of that tile (floats)
+
+template <int MT>
+__global__ __launch_bounds__(512) void skinny_ring_kernel(const bf16* __restrict__ A, int lda,
+                                                          const bf16* __restrict__ W, int ldw,
+                                                          const float* __restrict__ bias,
+                                                          void* __restrict__ C, int ldc,
+                                                          float* __restrict__ part, int M, int N, int K,
+                                                          int k_per_split, int epi) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int ROWS = MT * 16;
+  bf16* As = reinterpret_cast<bf16*>(smem);                                            // [2][ROWS][SK_LD]
+  float* ot = reinterpret_cast<float*>(smem + 2 * ROWS * SK_LD * sizeof(bf16));        // [ROWS][SR_LD]
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  const int r16 = lane & 15, kq = (lane >> 4) * 8;
+  const int n0 = blockIdx.x * 128;
+  const bf16* wrow = W + (size_t)min(n0 + wid * 16 + r16, N - 1) * ldw + kq;
+  const int k_begin = blockIdx.y * k_per_split;
+  const int k_end = min(K, k_begin + k_per_split);
+  const int sk = (tid & 31) * 8;
+  const bf16* src[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) src[i] = A + (size_t)min(i * 16 + (tid >> 5), M - 1) * lda + sk;
+  bf16x8 stage[MT], wr[KC / 32];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) stage[i] = *reinterpret_cast<const bf16x8*>(src[i] + k_begin);
+#pragma unroll
+  for (int s = 0; s < KC / 32; ++s) wr[s] = *reinterpret_cast<const bf16x8*>(wrow + k_begin + s * 32);
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+    *reinterpret_cast<bf16x8*>(&As[(i * 16 + (tid >> 5)) * SK_LD + sk]) = stage[i];
+  __syncthreads();
+  floatx4 acc[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  int buf = 0;
+  for (int k0 = k_begin; k0 < k_end; k0 += KC) {
+    const int kn = k0 + KC < k_end ? k0 + KC : k_begin;     // behind the last chunk: the first again, dropped
+#pragma unroll
+    for (int i = 0; i < MT; ++i) stage[i] = *reinterpret_cast<const bf16x8*>(src[i] + kn);
+    __builtin_amdgcn_sched_barrier(0);
+    const bf16* as = As + buf * ROWS * SK_LD;
+#pragma unroll
+    for (int s = 0; s < KC / 32; ++s) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&as[(i * 16 + r16) * SK_LD + s * 32 + kq]);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, wr[s], acc[i], 0, 0, 0);
+      }
+      wr[s] = *reinterpret_cast<const bf16x8*>(wrow + kn + s * 32);
+      __builtin_amdgcn_sched_barrier(0);      // use a register, then refill it, in this order
+    }
+    buf ^= 1;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+      *reinterpret_cast<bf16x8*>(&As[(buf * ROWS + i * 16 + (tid >> 5)) * SK_LD + sk]) = stage[i];
+    __syncthreads();
+  }
+  // D[m][n]: n = lane % 16, m = 4 (lane / 16) + r
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) ot[(i * 16 + (lane >> 4) * 4 + r) * SR_LD + wid * 16 + r16] = acc[i][r];
+  __syncthreads();
+  const int c = tid & 127, n = n0 + c;
+  if (n >= N) return;
+  if (part) {
+    for (int m = tid >> 7; m < M; m += 4) part[((size_t)blockIdx.y * M + m) * N + n] = ot[m * SR_LD + c];
+  } else {
+    const float b = bias ? bias[n] : 0.f;
+    for (int m = tid >> 7; m < M; m += 4) store_out(C, ldc, m, n, ot[m * SR_LD + c] + b, epi);
+  }
+}
+
 // At most 16 rows: no LDS staging at all.  A block owns 16 NT weight rows; its NW waves split
 // K between them, each streaming its slice of the weights from HBM and the matching slice of
 // the few activation rows from L2 straight into MFMA operands, S steps (32 S k) of loads in
@@ -1016,6 +1094,161 @@ int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const fl
   return mf_launch_status();
 }
 
+// 17 to 64 rows against a wide matrix (at least 8 tiles of 16 weight rows for every CU): one block
+// per CU with an equal share of the matrix, the whole of K, no partial sums between blocks and no
+// second kernel.  The share is cut into passes of at most 16 tiles; wave w multiplies tiles w and
+// w + 8 of the pass.  A slot with no tile multiplies the matrix's first bytes, read by all lanes
+// alike, and its sums are dropped: every wave runs the same instructions, so the loads in flight
+// can be counted, and such a load is one look-up in the CU's cache where a tile's (64 lanes in
+// 16 rows) is 64 -- repeating a real tile there made the cache's tag rate the limit.  Weights go
+// from HBM straight into MFMA operands through a ring of 16 fragments a wave: the load of the
+// next chunk's fragment is issued right behind the MFMA that frees the register, and runs on
+// into the next pass (a ring of two chunks measured the same).  The activations of a chunk
+// (256 k) are staged in LDS once per block, double-buffered, as in skinny_kernel; a pass re-reads
+// them from L2.  At the end of a pass the sums go through an LDS tile so that rows are stored in
+// whole lines, and SwiGLU pairs a gate tile with its up tile there.  (Folding the RMS norm into
+// the staging, as the 16-row kernel does, measured slower here: every block would re-read the
+// activations in 32 bits.)
+constexpr int PANEL_TILES = 16;                 // tiles of a pass
+constexpr int OT_LD = PANEL_TILES * 16 + 4;     // row stride of the output tile in LDS (floats)
+
+template <int MT>
+__global__ __launch_bounds__(512) void panel_kernel(const bf16* __restrict__ A, int lda,
+                                                    const bf16* __restrict__ W, int ldw,
+                                                    const float* __restrict__ bias, void* __restrict__ C,
+                                                    int ldc, int M, int N, int K, int units_total, int epi) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int ROWS = MT * 16;
+  bf16* As = reinterpret_cast<bf16*>(smem);                                            // [2][ROWS][SK_LD]
+  float* ot = reinterpret_cast<float*>(smem + 2 * ROWS * SK_LD * sizeof(bf16));        // [ROWS][OT_LD]
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  const int r16 = lane & 15, kq = (lane >> 4) * 8;
+  const bool pair = epi == EPI_SWIGLU;
+  // a unit is 32 weight rows: 32 outputs, or (pair) 16 gate rows and the 16 up rows of the same outputs
+  const int u_begin = (int)((long)blockIdx.x * units_total / gridDim.x);
+  const int u_end = (int)((long)(blockIdx.x + 1) * units_total / gridDim.x);
+  const int n_u = u_end - u_begin;
+  if (n_u <= 0) return;
+  const int n_pass = (2 * n_u + PANEL_TILES - 1) / PANEL_TILES;
+  const int per_u = (n_u + n_pass - 1) / n_pass;          // units of a pass (the last may have fewer)
+  const int nch = K / KC;
+  // what this lane reads for slot j of pass p, as a pointer at chunk 0
+  auto slot_ptr = [&](int p, int j) -> const bf16* {
+    if (p >= n_pass) return W;                             // behind the last pass: dropped
+    const int cnt = 2 * min(per_u, n_u - p * per_u);       // tiles of the pass
+    const int t = wid + 8 * j;
+    if (t >= cnt) return W;                                // no tile
+    const int u = u_begin + p * per_u + (t >> 1), which = t & 1;
+    const int row0 = pair ? (u >> 1) * 64 + (u & 1) * 16 + 32 * which : u * 32 + 16 * which;
+    return W + (size_t)min(row0 + r16, N - 1) * ldw + kq;
+  };
+  // staging: this thread handles rows i * 16 + tid / 32, k (tid % 32) * 8 of a chunk
+  const int sk = (tid & 31) * 8;
+  const bf16* src[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) src[i] = A + (size_t)min(i * 16 + (tid >> 5), M - 1) * lda + sk;
+  bf16x8 stage[MT];
+  auto load_stage = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i) stage[i] = *reinterpret_cast<const bf16x8*>(src[i] + k0);
+  };
+  auto store_stage = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+      *reinterpret_cast<bf16x8*>(&As[(buf * ROWS + i * 16 + (tid >> 5)) * SK_LD + sk]) = stage[i];
+  };
+
+  const bf16* wp[2] = {slot_ptr(0, 0), slot_ptr(0, 1)};
+  bf16x8 wr[2][KC / 32];
+  load_stage(0);
+#pragma unroll
+  for (int s = 0; s < KC / 32; ++s) {
+    wr[0][s] = *reinterpret_cast<const bf16x8*>(wp[0] + s * 32);
+    wr[1][s] = *reinterpret_cast<const bf16x8*>(wp[1] + s * 32);
+  }
+  store_stage(0);
+  __syncthreads();
+  floatx4 acc[2][MT];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[j][i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  int buf = 0, pass = 0, kc = 0;
+  const int total = n_pass * nch;
+  for (int t = 0; t < total; ++t) {
+    // the next step: the pass's next chunk, or chunk 0 of the next pass
+    const bool last_chunk = kc + 1 == nch;
+    const int kn = last_chunk ? 0 : (kc + 1) * KC;
+    const bf16* wnext[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) wnext[j] = last_chunk ? slot_ptr(pass + 1, j) : wp[j];
+    load_stage(kn);
+    __builtin_amdgcn_sched_barrier(0);
+    const bf16* as = As + buf * ROWS * SK_LD;
+#pragma unroll
+    for (int s = 0; s < KC / 32; ++s) {
+      bf16x8 a[MT];
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+        a[i] = *reinterpret_cast<const bf16x8*>(&as[(i * 16 + r16) * SK_LD + s * 32 + kq]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+          acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], wr[j][s], acc[j][i], 0, 0, 0);
+        wr[j][s] = *reinterpret_cast<const bf16x8*>(wnext[j] + kn + s * 32);
+        __builtin_amdgcn_sched_barrier(0);      // use a register, then refill it, in this order
+      }
+    }
+    store_stage(buf ^ 1);
+    buf ^= 1;
+    __syncthreads();        // the next chunk is staged
+    if (!last_chunk) {
+      ++kc;
+      continue;
+    }
+    // ---- end of a pass
+    const int cnt = 2 * min(per_u, n_u - pass * per_u);
+    // D[m][n]: n = lane % 16, m = 4 (lane / 16) + r
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int tl = wid + 8 * j;
+      if (tl < cnt) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            ot[(i * 16 + (lane >> 4) * 4 + r) * OT_LD + tl * 16 + r16] = acc[j][i][r];
+      }
+#pragma unroll
+      for (int i = 0; i < MT; ++i) acc[j][i] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    __syncthreads();        // the tile is whole; the next pass writes it behind its own barriers
+    {
+      const int c = tid & 255;
+      const int u0 = u_begin + pass * per_u;
+      if (pair) {
+        const int col = u0 * 16 + c;                       // unit c / 16 holds gate at 32 (c / 16), up 16 further
+        if (c < cnt * 8 && col < ldc) {
+          const int o = (c >> 4) * 32 + (c & 15);
+          for (int m = tid >> 8; m < M; m += 2)
+            ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(ot[m * OT_LD + o], ot[m * OT_LD + o + 16]);
+        }
+      } else {
+        const int col = u0 * 32 + c;
+        if (c < cnt * 16 && col < N) {
+          const float b = bias ? bias[col] : 0.f;
+          for (int m = tid >> 8; m < M; m += 2) store_out(C, ldc, m, col, ot[m * OT_LD + c] + b, epi);
+        }
+      }
+    }
+    wp[0] = wnext[0];
+    wp[1] = wnext[1];
+    ++pass;
+    kc = 0;
+  }
+}
+
 __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restrict__ part,
                                                             const float* __restrict__ bias,
                                                             void* __restrict__ C, int ldc, int M, int N,
@@ -1053,8 +1286,22 @@ int launch_skinny_v(const bf16* A, int lda, const bf16* W, int ldw, const float*
   }
   dim3 grid((N + 127) / 128, splits);
   const bool two_pass = splits > 1 || epi == EPI_SWIGLU;   // gate and up columns sit in different waves
-  kern<<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, two_pass ? part : nullptr, M, N, K,
-                                    k_per_split, epi);
+  static const int no_ring = getenv("MF_NO_SKINNY_RING") ? 1 : 0;
+  if (VEC && !no_ring && K % KC == 0 && (long)(splits - 1) * k_per_split < K) {      // whole chunks only
+    constexpr int smem_ring = smem + MT * 16 * SR_LD * (int)sizeof(float);
+    static bool ring_configured = false;
+    if (!ring_configured) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_ring_kernel<MT>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, smem_ring);
+      if (e != hipSuccess) return (int)e;
+      ring_configured = true;
+    }
+    skinny_ring_kernel<MT><<<grid, 512, smem_ring, stream>>>(A, lda, W, ldw, bias, C, ldc,
+                                                             two_pass ? part : nullptr, M, N, K, k_per_split, epi);
+  } else {
+    kern<<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, two_pass ? part : nullptr, M, N, K,
+                                      k_per_split, epi);
+  }
   int rc = mf_launch_status();
   if (rc == 0 && two_pass) {
     dim3 g2(((epi == EPI_SWIGLU ? ldc : N) + 255) / 256, M);
@@ -1072,6 +1319,43 @@ int launch_skinny(const bf16* A, int lda, const bf16* W, int ldw, const float* b
                                             epi, stream)
                 : launch_skinny_v<MT, false>(A, lda, W, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split,
                                              epi, stream);
+}
+
+// The whole-K kernel for 17 to 64 rows, where the matrix is wide enough to give every CU at least
+// 8 tiles; MF_NOT_BUILT (nothing launched) for any other shape.
+constexpr int MF_NOT_BUILT = -2;
+template <int MT>
+int launch_panel_mt(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc, int M,
+                    int N, int K, int epi, int grid, int units, hipStream_t stream) {
+  constexpr int smem = 2 * MT * 16 * SK_LD * (int)sizeof(bf16) + MT * 16 * OT_LD * (int)sizeof(float);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(panel_kernel<MT>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    configured = true;
+  }
+  panel_kernel<MT><<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, units, epi);
+  return mf_launch_status();
+}
+
+int launch_panel(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc, int M, int N,
+                 int K, int epi, hipStream_t stream) {
+  static const int off = getenv("MF_NO_PANEL") ? 1 : 0;
+  if (off || M <= 16 || M > 64 || K % KC != 0 || ldw % 8 != 0 || (uintptr_t)W % 16 != 0 || lda % 8 != 0 ||
+      (uintptr_t)A % 16 != 0)
+    return MF_NOT_BUILT;
+  if (epi == EPI_SWIGLU && N % 64 != 0) return MF_NOT_BUILT;
+  const int n_cu = cu_count();
+  if (n_cu <= 0) return (int)hipErrorUnknown;
+  const int units = (N + 31) / 32;
+  if (units < 4 * n_cu) return MF_NOT_BUILT;
+  switch ((M + 15) / 16) {
+    case 2: return launch_panel_mt<2>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
+    case 3: return launch_panel_mt<3>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
+    case 4: return launch_panel_mt<4>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
+  }
+  return MF_NOT_BUILT;
 }
 
 }  // namespace
@@ -1119,7 +1403,6 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
 
 // The register-resident kernel for the shapes it is built for (K = 256 NS with enough tiles to
 // go round); MF_NOT_BUILT for any other, and nothing is launched.
-constexpr int MF_NOT_BUILT = -2;
 static int stationary16(const void* a, int lda, const bf16* w, int ldw, const float* bias, void* C, int ldc, int M,
                  int N, int K, int epi, const NormArgs* norm, hipStream_t stream) {
   static const int off = getenv("MF_NO_STATIONARY") ? 1 : 0;
@@ -1187,6 +1470,10 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
     if (v == 2) return launch_skinny16<4, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     if (v == 3) return launch_skinny16<8, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     return launch_skinny16<4, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+  }
+  if (M > 16) {
+    const int rc = launch_panel(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+    if (rc != MF_NOT_BUILT) return rc;
   }
   switch ((M + 15) / 16) {
     case 1: return launch_skinny<1>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);

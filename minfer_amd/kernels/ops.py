@@ -236,10 +236,25 @@ def rope_kvwrite(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positi
 
 
 # ------------------------------------------------------------------ matrix products
-def skinny_plan(m: int, n: int, k: int, target_blocks: int = 1024) -> Tuple[int, int]:
-    """(splits, k_per_split) of the decode product: enough blocks to fill the chip."""
+_CU_COUNT: Optional[int] = None
+
+
+def cu_count() -> int:
+    """Compute units of the current device (256 on MI355X)."""
+    global _CU_COUNT
+    if _CU_COUNT is None:
+        _CU_COUNT = int(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count)
+    return _CU_COUNT
+
+
+def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None) -> Tuple[int, int]:
+    """(splits, k_per_split) of the decode product.  17 to 64 rows: blocks of 128 weight rows,
+    and K split so that there is about one block per CU (measured: with four times as many,
+    the partial sums and the start of each block cost a fifth more)."""
     if m <= 16:
         return 1, (k + 255) // 256 * 256      # one kernel: K is split between the waves of a block
+    if target_blocks is None:
+        target_blocks = int(os.environ.get("MF_SKINNY_TARGET", 0)) or cu_count()
     n_blocks = (n + 127) // 128
     chunks = (k + 255) // 256
     splits = max(1, min(chunks, target_blocks // max(1, n_blocks)))

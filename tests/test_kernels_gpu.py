@@ -196,7 +196,9 @@ def test_gemm_f32(ops, m, n, k):
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 6, 9, 12])
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(2048, 512, 256), (1, 152064, 64), (64, 3584, 3584),
                                                  # at most 16 rows with K of 1536..4096: activations in registers
-                                                 (1, 2100, 1536), (5, 2050, 2048), (8, 4001, 3584), (16, 2048, 4096)])
+                                                 (1, 2100, 1536), (5, 2050, 2048), (8, 4001, 3584), (16, 2048, 4096),
+                                                 # 17..64 rows, whole chunks of K: the ring kernel, with K split
+                                                 (20, 200, 768), (50, 1000, 4096)])
 def test_gemm_bf16(ops, variant, m, n, k):
     if variant and (m * n * k > 3e9):
         pytest.skip("large shape is covered by the default variant")
@@ -461,10 +463,35 @@ def test_attn_prefill_far_key_and_window_edge(ops):
     assert not torch.allclose(out[2, :hd].float().cpu(), vrow, atol=3e-2)
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 33000, 512), (17, 32768, 256), (40, 40001, 768), (33, 152064, 256)])
+def test_gemm_bf16_wide_few_rows(ops, m, n, k):
+    """17..64 rows against a matrix wide enough for the whole-K kernel (a share of at least 8
+    tiles for every CU; the widest takes several passes; 40001 ends inside a tile)."""
+    x, w, b = rnd((m, k), torch.bfloat16, 70), rnd((n, k), torch.bfloat16, 71, 0.05), rnd((n,), seed=72)
+    ref = x.double() @ w.double().t() + b.double()
+    xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+    tol = 2e-5 * math.sqrt(k)
+    out = torch.full((m, n), 7.0, device=DEV)
+    ops.linear(xd, wd, bd, out)
+    close(out, ref, tol, 1e-5)
+    again = torch.empty(m, n, device=DEV)
+    ops.linear(xd, wd, bd, again)
+    assert torch.equal(out, again)
+    base = rnd((m, n), seed=73)
+    acc = base.to(DEV).clone()
+    ops.linear(xd, wd, None, acc, accumulate=True)
+    close(acc, ref - b.double() + base.double(), tol, 1e-5)
+    ob = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    ops.linear(xd, wd, bd, ob)
+    close(ob, ref, tol + 1e-3, 1e-2)
+
+
 @pytest.mark.parametrize("variant", [0, 1, 2, 9, 12])
 @pytest.mark.parametrize("m,nf,k", [(1, 176, 64), (8, 344, 128), (16, 32, 200), (17, 176, 64), (64, 1000, 344),
                                     (65, 232, 200), (300, 18944, 256), (130, 31, 72),
-                                    (8, 1100, 1536), (3, 2100, 3584), (16, 1030, 4096), (1, 1024, 2048)])
+                                    (8, 1100, 1536), (3, 2100, 3584), (16, 1030, 4096), (1, 1024, 2048),
+                                    # 17..64 rows against a wide matrix: one block per CU over the whole of K
+                                    (64, 18944, 512), (33, 16400, 256), (40, 300, 512)])
 def test_gemm_bf16_swiglu(ops, variant, m, nf, k):
     if variant == 12 and k % 32:
         pytest.skip("the direct-to-LDS pipeline takes k in steps of 32")
