@@ -233,22 +233,30 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const 
 }
 
 // ------------------------------------------------------------------ tiled kernel, loads straight into LDS
-// The same 256 x 256 tile on 8 waves (each 128 x 64), but k tiles of 32 travel global -> LDS
+// The same 256 x 256 tile on 8 waves (each 128 x 64), but k tiles of 64 travel global -> LDS
 // without passing registers (global_load_lds_dwordx4: lane i's 16 bytes land at the wave's LDS
-// base + 16 i), four stages deep, so that a tile's loads have three to four tiles of products to arrive
-// in instead of one, and the 32 staging registers are gone.  There is no room for
-// padding in such a copy, so a row's four 16-byte chunks are stored permuted: chunk c of row
-// r sits at position c ^ ((r >> 2) & 3), which spreads the 16 rows that one pass of a
-// 16-byte fragment read covers over all 64 banks (measured: no bank conflicts; with
-// (r >> 1) & 3, right for 32 banks, every read took twice as long).  Which chunk a lane fetches is free (its
-// global address), so the permutation costs nothing on the way in.
+// base + 16 i), two stages of 64 KB, and the 32 staging registers are gone.
+//
+// A row of a k tile is one 128-byte line, fetched by 8 adjacent lanes: a CU keeps only about 64
+// requests to L2 in flight (measured: 64-byte requests, which k tiles of 32 make, drew 28 GB/s
+// a CU at L2's 300 cycles and left the waves waiting for their tiles 40% of the time), so every
+// request has to be a whole line.
+//
+// There is no room for padding in such a copy, so a row's eight 16-byte chunks are stored
+// permuted: chunk c of row r sits at position c ^ ((r >> 1) & 7), which spreads the 16 rows
+// that one pass of a 16-byte fragment read covers over all 64 banks.  Which chunk a lane fetches
+// is free (its global address), so the permutation costs nothing on the way in.
 //
 // The compiler does not know that these loads write LDS and so does not wait for them; the
-// kernel does, with vmcnt counts it keeps itself (4 loads per wave and tile, in order) and
-// one barrier per tile: after it, tile kt has landed for every wave, and the stage of tile
-// kt - 1, whose products all waves have issued, is free to take tile kt + stages - 1.
-// Needs 16-byte aligned rows and K a multiple of 32.
-constexpr int DMA_BM = 256, DMA_BN = 256, DMA_BK = 32, DMA_STAGES = 4;
+// kernel does, with vmcnt counts it keeps itself (8 loads per wave and tile, in order) and
+// one barrier per tile: behind it, tile kt + 1 has landed for every wave, and the stage of tile
+// kt, which every wave holds in registers by then, is free to take tile kt + 2.
+// Needs 16-byte aligned rows and K a multiple of 64.
+// Measured on the 2048 x 37888 x 3584 product (0.95 PFLOP/s): without the copies 1.1, without
+// copies and fragment reads 1.3 (the matrix cores alone, with the epilogue's 310 MB of output),
+// at a clock of 2.0 GHz under this load; asking for a tile in four parts spread over a tile's
+// products, or leaving the barrier out, changed nothing.
+constexpr int DMA_BM = 256, DMA_BN = 256, DMA_BK = 64, DMA_STAGES = 2;
 constexpr int DMA_STAGE_BYTES = (DMA_BM + DMA_BN) * DMA_BK * 2;
 
 __device__ __forceinline__ void dma16(const bf16* g, unsigned lds_byte) {
@@ -262,6 +270,7 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
                                                        int ldc, int M, int N, int K, int epi, int tiles_m,
                                                        int xcd_remap) {
   constexpr int TM = 4, TN = 2;
+  constexpr int ROW = DMA_BK * 2;              // bytes of a row in LDS
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   int tile = blockIdx.x;
   if (xcd_remap) {
@@ -284,55 +293,53 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // this lane's share of a tile's copy: wave `wid` moves 1 KB blocks wid and 8 + wid (16 rows
-  // each) of the A tile and of the W tile; the lane fetches row 16 b + lane / 4, the chunk that
-  // belongs at position lane % 4
+  // this lane's share of a tile's copy: wave `wid` moves the 1 KB blocks wid, 8 + wid, 16 + wid
+  // and 24 + wid (8 rows each) of the A tile and of the W tile; the lane fetches row
+  // 8 b + lane / 8, the chunk that belongs at position lane % 8
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
-  const bf16* ga[2];
-  const bf16* gw[2];
-  unsigned la[2], lw[2];
+  const bf16* ga[4];
+  const bf16* gw[4];
 #pragma unroll
-  for (int jj = 0; jj < 2; ++jj) {
-    const int b = jj * 8 + wid;
-    const int r = 16 * b + (lane >> 2);
-    const int chunk = (lane & 3) ^ ((r >> 2) & 3);
+  for (int jj = 0; jj < 4; ++jj) {
+    const int r = 8 * (jj * 8 + wid) + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((r >> 1) & 7);
     ga[jj] = A + (size_t)min(m0 + r, M - 1) * lda + chunk * 8;
     gw[jj] = W + (size_t)min(n0 + r, N - 1) * ldw + chunk * 8;
-    la[jj] = lds0 + b * 1024;
-    lw[jj] = lds0 + DMA_BM * DMA_BK * 2 + b * 1024;
   }
   auto issue = [&](int kt) {
-    const unsigned st = (unsigned)(kt % DMA_STAGES) * DMA_STAGE_BYTES;
+    const unsigned st = lds0 + (unsigned)(kt % DMA_STAGES) * DMA_STAGE_BYTES + wid * 1024;
     const int k = kt * DMA_BK;
 #pragma unroll
-    for (int jj = 0; jj < 2; ++jj) dma16(ga[jj] + k, __builtin_amdgcn_readfirstlane(la[jj] + st));
+    for (int jj = 0; jj < 4; ++jj) dma16(ga[jj] + k, __builtin_amdgcn_readfirstlane(st + jj * 8192));
 #pragma unroll
-    for (int jj = 0; jj < 2; ++jj) dma16(gw[jj] + k, __builtin_amdgcn_readfirstlane(lw[jj] + st));
+    for (int jj = 0; jj < 4; ++jj)
+      dma16(gw[jj] + k, __builtin_amdgcn_readfirstlane(st + DMA_BM * ROW + jj * 8192));
   };
-  // fragment reads: row R of a tile, chunk ks * 2 + fk of its 4, at position chunk ^ ((R >> 2) & 3)
-  const int sw = (fr >> 2) & 3;
+  // fragment reads: row R of a tile, chunk 4 half + 2 ks + fk of its 8, at position chunk ^ ((R >> 1) & 7)
+  const int sw = (fr >> 1) & 7;
   int offa[TM], offw[TN];
 #pragma unroll
-  for (int i = 0; i < TM; ++i) offa[i] = (wm + i * 32 + fr) * (DMA_BK * 2);
+  for (int i = 0; i < TM; ++i) offa[i] = (wm + i * 32 + fr) * ROW;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) offw[j] = DMA_BM * DMA_BK * 2 + (wn + j * 32 + fr) * (DMA_BK * 2);
-  const int pos0 = ((0 + fk) ^ sw) * 16, pos1 = ((2 + fk) ^ sw) * 16;
+  for (int j = 0; j < TN; ++j) offw[j] = DMA_BM * ROW + (wn + j * 32 + fr) * ROW;
 
   const int nkt = K / DMA_BK;
-  // Fragments of tile kt + 1 are read from LDS while the second half of tile kt's products runs,
-  // into the other register set: behind the barrier there is always work for the matrix cores.
+  // A tile is multiplied in two halves of two k-steps, from two register sets: the fragments of
+  // the next half are read from LDS while the second k-step of this one runs, so that behind the
+  // barrier there is always work for the matrix cores.
   bf16x8 fa[2][2][TM], fw[2][2][TN];          // [set][k-step][tile]
-  auto read_frags = [&](int stage, auto SET) {
-    constexpr int set = decltype(SET)::value;
+  auto read_frags = [&](int stage, auto HALF) {
+    constexpr int half = decltype(HALF)::value;          // which is also the register set
     const unsigned char* st = smem + stage * DMA_STAGE_BYTES;
+    const int pos0 = ((half * 4 + fk) ^ sw) * 16, pos1 = ((half * 4 + 2 + fk) ^ sw) * 16;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) fa[set][0][i] = *reinterpret_cast<const bf16x8*>(st + offa[i] + pos0);
+    for (int i = 0; i < TM; ++i) fa[half][0][i] = *reinterpret_cast<const bf16x8*>(st + offa[i] + pos0);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fw[set][0][j] = *reinterpret_cast<const bf16x8*>(st + offw[j] + pos0);
+    for (int j = 0; j < TN; ++j) fw[half][0][j] = *reinterpret_cast<const bf16x8*>(st + offw[j] + pos0);
 #pragma unroll
-    for (int i = 0; i < TM; ++i) fa[set][1][i] = *reinterpret_cast<const bf16x8*>(st + offa[i] + pos1);
+    for (int i = 0; i < TM; ++i) fa[half][1][i] = *reinterpret_cast<const bf16x8*>(st + offa[i] + pos1);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fw[set][1][j] = *reinterpret_cast<const bf16x8*>(st + offw[j] + pos1);
+    for (int j = 0; j < TN; ++j) fw[half][1][j] = *reinterpret_cast<const bf16x8*>(st + offw[j] + pos1);
   };
   auto multiply = [&](int ks, auto SET) {
     constexpr int set = decltype(SET)::value;
@@ -342,45 +349,40 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
       for (int j = 0; j < TN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][ks][i], fw[set][ks][j], acc[i][j], 0, 0, 0);
   };
-  // wait until the loads of tile t (of this wave) have landed: at most those of the tiles
-  // issued after it may still be in flight, `issued` being the last tile asked for so far
-  auto wait_tile = [&](int t, int issued) {
-    const int later = issued - t;
-    if (later >= 3) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-    else if (later == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else if (later == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  };
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
-  int issued = -1;
-#pragma unroll
-  for (int t = 0; t < DMA_STAGES; ++t)
-    if (t < nkt) { issue(t); issued = t; }
-  wait_tile(0, issued);
+  issue(0);
+  int issued = 0;
+  if (nkt > 1) { issue(1); issued = 1; }
+  // the loads of tile 0 (of this wave) have landed when at most tile 1's eight are in flight
+  if (issued == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   read_frags(0, S0{});
   int stage = 0;                               // of tile kt
-  // one round: tile kt from register set SET; in its middle the barrier that makes tile kt + 1
-  // readable and tile kt's stage free (every wave holds tile kt in registers by then)
-  auto round = [&](int kt, auto SET, auto OTHER) {
-    multiply(0, SET);
+  for (int kt = 0; kt < nkt; ++kt) {
+    // first half, from set 0; the second half of the same stage goes into set 1
+    multiply(0, S0{});
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(stage, S1{});
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(1, S0{});
+    __builtin_amdgcn_sched_barrier(0);
+    // second half, from set 1; in its middle the barrier that makes tile kt + 1 readable and
+    // this tile's stage free
+    multiply(0, S1{});
     __builtin_amdgcn_sched_barrier(0);
     if (kt + 1 < nkt) {
-      wait_tile(kt + 1, issued);
+      if (issued > kt + 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (issued + 1 < nkt) { issue(issued + 1); ++issued; }      // into the stage of tile kt
-      const int next_stage = stage + 1 == DMA_STAGES ? 0 : stage + 1;
-      read_frags(next_stage, OTHER);
-      stage = next_stage;
+      stage ^= 1;
+      read_frags(stage, S0{});
     }
     __builtin_amdgcn_sched_barrier(0);
-    multiply(1, SET);
+    multiply(1, S1{});
     __builtin_amdgcn_sched_barrier(0);
-  };
-  for (int kt = 0; kt < nkt; kt += 2) {
-    round(kt, S0{}, S1{});
-    if (kt + 1 < nkt) round(kt + 1, S1{}, S0{});
   }
   tile_epilogue<TM, TN>(acc, bias, C, ldc, M, N, epi, m0, wm, n0, wn, lane);
 }
@@ -1361,7 +1363,7 @@ int launch_panel(const bf16* A, int lda, const bf16* W, int ldw, const float* bi
 }  // namespace
 
 // `variant`: 0 picks by shape; 1: 256x256 tile with 4 waves, 2: 128x128, 3: 64x64, 6: 256x128
-// with 8 waves, 9: 256x256 with 8 waves, 12: 256x256 through the direct-to-LDS pipeline (tests
+// with 8 waves, 9: 256x256 with 8 waves, 12: 256x256 through the direct-to-LDS pipeline, K in 64s (tests
 // name them).
 MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
                         int ldc, int M, int N, int K, int epi, int variant, hipStream_t stream) {

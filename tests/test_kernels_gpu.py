@@ -202,8 +202,8 @@ def test_gemm_f32(ops, m, n, k):
 def test_gemm_bf16(ops, variant, m, n, k):
     if variant and (m * n * k > 3e9):
         pytest.skip("large shape is covered by the default variant")
-    if variant == 12 and k % 32:
-        pytest.skip("the direct-to-LDS kernel takes K in multiples of 32")
+    if variant == 12 and k % 64:
+        pytest.skip("the direct-to-LDS kernel takes K in multiples of 64")
     x, w, b = rnd((m, k), torch.bfloat16, 8), rnd((n, k), torch.bfloat16, 9, 0.05), rnd((n,), seed=10)
     ref = x.double() @ w.double().t() + b.double()
     xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
@@ -493,8 +493,8 @@ def test_gemm_bf16_wide_few_rows(ops, m, n, k):
                                     # 17..64 rows against a wide matrix: one block per CU over the whole of K
                                     (64, 18944, 512), (33, 16400, 256), (40, 300, 512)])
 def test_gemm_bf16_swiglu(ops, variant, m, nf, k):
-    if variant == 12 and k % 32:
-        pytest.skip("the direct-to-LDS pipeline takes k in steps of 32")
+    if variant == 12 and k % 64:
+        pytest.skip("the direct-to-LDS pipeline takes k in steps of 64")
     x = rnd((m, k), torch.bfloat16, 30)
     wg, wu = rnd((nf, k), torch.bfloat16, 31, 0.3), rnd((nf, k), torch.bfloat16, 32, 0.3)
     g, u = x.double() @ wg.double().t(), x.double() @ wu.double().t()
