@@ -3,21 +3,21 @@
 // (out[t][o] = dot(W[o][:], x[t][:]) + b[o], src/graph/cpu_backend.rs:214-248 of
 // yusiwen/minfer; the reference's own matrix kernels are quantised and are not followed.)
 //
-// Four kernels:
+// The kernels:
 //  * `tile_kernel`: many rows (prompts).  A BM x BN block tile per 4 or 8 waves, K walked in
 //    steps of BK through double-buffered LDS, 32x32x16 MFMA, each wave a WM x WN tile.
-//    Measured on MI355X at 2048 rows: what bounds it is operand delivery into the CU (the
-//    same loop without its global loads runs a third faster, without its LDS reads a tenth),
-//    so the largest tile that still leaves two waves per SIMD wins where there are enough
-//    tiles; prefetching two tiles ahead in registers changed nothing and was dropped.
+//  * `tile_dma_kernel`: the 256 x 256 tile with its k tiles copied straight into LDS; the
+//    choice for large aligned products.
 //  * `stationary16_kernel`: at most 16 rows and K of 1536, 2048, 3584 or 4096 (decode): one
 //    block per CU keeps the activations in registers and walks over weight tiles.
-//  * `skinny16_kernel`: at most 16 rows, any K (decode).  The time is the weight stream: the waves
-//    of a block split K, each reads weights and activations straight into MFMA operands
-//    (16x16x32) and the partial sums meet in LDS.
-//  * `skinny_kernel`: 17 to 64 rows.  Each wave owns 16 weight rows and reads them from HBM
-//    straight into MFMA operands, the activation rows are staged in LDS and shared by the
-//    block, K may be split over blocks with a fixed-order reduction afterwards.
+//  * `rolling16_kernel`, `skinny16_kernel`: at most 16 rows, any K (decode).  The time is the
+//    weight stream: the waves of a block split K, each reads weights and activations straight
+//    into MFMA operands (16x16x32) and the partial sums meet in LDS.
+//  * `panel_kernel`: 17 to 64 rows against a wide matrix: one block per CU over the whole of K.
+//  * `skinny_ring_kernel`, `skinny_kernel` (any alignment): 17 to 64 rows.  Each wave owns 16
+//    weight rows and reads them from HBM straight into MFMA operands, the activation rows are
+//    staged in LDS and shared by the block, K may be split over blocks with a fixed-order
+//    reduction afterwards.
 // Both operands have K contiguous, which is exactly the MFMA operand layout (8 consecutive
 // k per lane), so nothing is transposed.
 //
