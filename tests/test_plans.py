@@ -1,0 +1,35 @@
+"""The launch plans are plain functions of shapes: what the kernels' host checks rely on holds
+for every shape (no empty split, whole chunks and pages, bounds on the number of splits)."""
+import itertools
+
+from minfer_amd.kernels import ops
+
+
+def test_skinny_plan_covers_k_without_empty_splits():
+    for m, n, k, target in itertools.product((1, 16, 17, 40, 64), (96, 3584, 4608, 37888, 152064),
+                                             (64, 200, 256, 3584, 18944), (64, 256, 1024)):
+        splits, per = ops.skinny_plan(m, n, k, target_blocks=target)
+        assert splits >= 1 and per % 256 == 0
+        assert splits * per >= k, (m, n, k, splits, per)
+        assert (splits - 1) * per < k, (m, n, k, splits, per)        # the last split has work
+        if m <= 16:
+            assert splits == 1
+        else:
+            assert splits * ((n + 127) // 128) <= max(target, (n + 127) // 128), (m, n, k, splits)
+
+
+def test_split_plan_of_the_32_bit_attention():
+    for n_tok, nk, group, hd, max_len in itertools.product((1, 8, 64, 300), (1, 2, 4), (1, 5, 7), (16, 128, 256),
+                                                           (1, 64, 100, 4096, 32768)):
+        n_splits, split_len = ops.split_plan(n_tok, nk, group, hd, max_len)
+        assert 1 <= n_splits <= 64
+        assert split_len % ops.PAGE == 0 and split_len > 0
+        assert n_splits * split_len >= max_len
+        assert (n_splits - 1) * split_len < max_len                   # the last split has keys
+
+
+def test_decode_split_plan_bounds():
+    for n_tok, nk, group, max_len in itertools.product((1, 8, 64, 300), (1, 2, 4), (1, 5, 7, 17), (1, 64, 4096, 32768)):
+        n = ops.decode_split_plan(n_tok, nk, group, max_len)
+        assert 1 <= n <= 16
+        assert n == 1 or n * 128 <= max_len + 127
