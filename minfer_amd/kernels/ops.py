@@ -248,11 +248,14 @@ def cu_count() -> int:
 
 
 def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None) -> Tuple[int, int]:
-    """(splits, k_per_split) of the decode product.  17 to 64 rows: blocks of 128 weight rows,
+    """(splits, k_per_split) of the decode product.  More than 16 rows: blocks of 128 weight rows,
     and K split so that there is about one block per CU (measured: with four times as many,
     the partial sums and the start of each block cost a fifth more)."""
-    if m <= 16:
+    if m <= 8 or (m <= 16 and k < 8192):
         return 1, (k + 255) // 256 * 256      # one kernel: K is split between the waves of a block
+    # (9..16 rows against a long K, which the register-resident kernel does not take: in the one-kernel
+    # form every block reads its own copy of the activations from L2, 42 us at 16 rows of 18944
+    # against 33 with the staged kernel below and its reduction)
     if target_blocks is None:
         target_blocks = int(os.environ.get("MF_SKINNY_TARGET", 0)) or cu_count()
     n_blocks = (n + 127) // 128
@@ -324,7 +327,7 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, vari
         return
     if m <= 64 and variant == 0:
         splits, per = skinny_plan(m, n, k)
-        part = workspace("skinny", splits * m * n, x.device) if m > 16 else None
+        part = workspace("skinny", splits * m * n, x.device) if m > 16 or splits > 1 else None
         _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
                                                         _ptr(part), m, n, k, splits, per, EPI_SWIGLU, _stream()),
                "gemm_bf16_skinny(swiglu)")

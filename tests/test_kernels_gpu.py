@@ -198,7 +198,9 @@ def test_gemm_f32(ops, m, n, k):
                                                  # at most 16 rows with K of 1536..4096: activations in registers
                                                  (1, 2100, 1536), (5, 2050, 2048), (8, 4001, 3584), (16, 2048, 4096),
                                                  # 17..64 rows, whole chunks of K: the ring kernel, with K split
-                                                 (20, 200, 768), (50, 1000, 4096)])
+                                                 (20, 200, 768), (50, 1000, 4096),
+                                                 # 9..16 rows against a long K: the same kernel
+                                                 (12, 300, 8192), (16, 3584, 18944)])
 def test_gemm_bf16(ops, variant, m, n, k):
     if variant and (m * n * k > 3e9):
         pytest.skip("large shape is covered by the default variant")
@@ -491,7 +493,7 @@ def test_gemm_bf16_wide_few_rows(ops, m, n, k):
                                     (65, 232, 200), (300, 18944, 256), (130, 31, 72),
                                     (8, 1100, 1536), (3, 2100, 3584), (16, 1030, 4096), (1, 1024, 2048),
                                     # 17..64 rows against a wide matrix: one block per CU over the whole of K
-                                    (64, 18944, 512), (33, 16400, 256), (40, 300, 512)])
+                                    (64, 18944, 512), (33, 16400, 256), (40, 300, 512), (10, 96, 8192)])
 def test_gemm_bf16_swiglu(ops, variant, m, nf, k):
     if variant == 12 and k % 64:
         pytest.skip("the direct-to-LDS pipeline takes k in steps of 64")
