@@ -40,3 +40,18 @@ def test_one_layer_at_7b_widths(folder, reference, dtype):
                 compare(run_steps(eng, tail_steps(reqs, tail=8)), ref, dtype, "7B widths one by one"),
                 compare(run_steps(eng, batch_steps(reqs, [ids[:3], ids[3:]])), ref, dtype, "7B widths batches"))
     print(f"{dtype}: worst abs err {worst:.3e}")
+
+
+def test_batch_of_twenty_at_7b_widths(folder):
+    """Twenty short requests in one batch: the prompts' step has some 60 rows and the decode steps
+    20 down to 1, so the products run in the kernels for 17 to 64 rows (one block per CU over the
+    whole of K for gate|up and the head, K split for the others) and then in those for at most 16."""
+    from minfer_amd import Engine, load_model
+    plain = PlainQwen2.from_folder(folder, dtype=np.float64)
+    reqs = requests_for(152064, [3 + (i * 5) % 7 for i in range(20)], seed=8)
+    ref = plain_logits(plain, reqs)
+    eng = Engine(load_model(folder, dtype="bfloat16"), max_tokens=64 * 20, poison_cache=True)
+    steps = batch_steps(reqs, [list(reqs)], prompt_frac=0.5)
+    assert 17 <= sum(len(e["tokens"]) for e in steps[0]["entries"]) <= 64 and len(steps[1]["entries"]) > 16
+    worst = compare(run_steps(eng, steps), ref, "bfloat16", "7B widths, batch of 20")
+    print(f"worst abs err {worst:.3e}")
