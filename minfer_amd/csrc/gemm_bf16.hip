@@ -18,6 +18,8 @@
 //    weight rows and reads them from HBM straight into MFMA operands, the activation rows are
 //    staged in LDS and shared by the block, K may be split over blocks with a fixed-order
 //    reduction afterwards.
+// For measurements the environment can take a kernel out of the choice: MF_NO_STATIONARY,
+// MF_NO_PANEL, MF_NO_SKINNY_RING, and MF_NO_XCD_REMAP (the tile kernels' block order).
 // Both operands have K contiguous, which is exactly the MFMA operand layout (8 consecutive
 // k per lane), so nothing is transposed.
 //
@@ -1442,36 +1444,26 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
                      ((uintptr_t)W % 16 == 0) && (K % 8 == 0);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
-  static const int variant16 = getenv("MF_SKINNY16") ? atoi(getenv("MF_SKINNY16")) : 0;
   if (M <= 16 && splits == 1) {
-    // few weight rows: more waves per block so that enough loads are in flight
-    // Measured at 3584..152064 weight rows: many rows -> 4 waves with two 16-row tiles each
-    // (less activation traffic per weight byte); a row count that would leave a short second
-    // round of 16-row blocks -> 8 waves with two tiles; otherwise 8 waves, one tile.
+    // the register-resident kernel where it is built; other aligned shapes the rolling K-split
+    // kernel; the rest (and SwiGLU outside the first) the guarded kernel
     if (vec_ok) {
       const int rc = stationary16(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, nullptr, stream);
       if (rc != MF_NOT_BUILT) return rc;
     }
-    static const int rolling = getenv("MF_ROLLING16") ? atoi(getenv("MF_ROLLING16")) : 1;
-    if (rolling && vec_ok && K % 32 == 0 && epi != EPI_SWIGLU) {
-      switch (rolling) {
-        case 1: return launch_rolling16<8, 1, 16>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
-        case 2: return launch_rolling16<8, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
-        case 3: return launch_rolling16<16, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
-        case 4: return launch_rolling16<8, 2, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
-        case 5: return launch_rolling16<16, 1, 12>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
-        case 6: return launch_rolling16<8, 1, 24>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
-      }
-    }
+    if (vec_ok && K % 32 == 0 && epi != EPI_SWIGLU)
+      return launch_rolling16<8, 1, 16>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
     if (epi == EPI_SWIGLU)
       return launch_skinny16<4, 2, 4, true>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    // Measured at 3584..152064 weight rows: many rows -> 4 waves with two 16-row tiles each
+    // (less activation traffic per weight byte); a row count that would leave a short second
+    // round of 16-row blocks -> 8 waves with two tiles; otherwise 8 waves, one tile.
     const int blocks16 = (N + 15) / 16;
-    int v = variant16;
-    if (v == 0) v = blocks16 >= 1024 ? 4 : (blocks16 > 256 && blocks16 <= 512 ? 3 : 1);
-    if (v == 1) return launch_skinny16<8, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    if (v == 2) return launch_skinny16<4, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    if (v == 3) return launch_skinny16<8, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    return launch_skinny16<4, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    if (blocks16 >= 1024)
+      return launch_skinny16<4, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    if (blocks16 > 256 && blocks16 <= 512)
+      return launch_skinny16<8, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    return launch_skinny16<8, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
   }
   if (M > 16) {
     const int rc = launch_panel(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
