@@ -24,7 +24,14 @@ QWEN25_7B = dict(
     intermediate_size=18944, vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-6,
     max_position_embeddings=32768, tie_word_embeddings=False, use_sliding_window=False,
     initializer_range=0.02)
-FULL_LAYERS = QWEN25_7B["num_hidden_layers"]
+# the larger shapes of the same architecture (for measurements beyond the default run)
+SHAPES = {
+    "7b": ("Qwen2.5-7B", QWEN25_7B),
+    "32b": ("Qwen2.5-32B", dict(QWEN25_7B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=40,
+                                num_key_value_heads=8, intermediate_size=27648, rms_norm_eps=1e-5)),
+    "72b": ("Qwen2.5-72B", dict(QWEN25_7B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
+                                num_key_value_heads=8, intermediate_size=29568, rms_norm_eps=1e-5)),
+}
 
 
 def parse():
@@ -36,7 +43,8 @@ def parse():
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prompt-max", type=int, default=2048)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has")
+    ap.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes (default: Qwen2.5-7B)")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true")
@@ -151,7 +159,10 @@ def main() -> int:
         return 2
     import torch
     from minfer_amd import LLM
-    cfg = dict(QWEN25_7B, num_hidden_layers=a.layers)
+    shape_name, shape = SHAPES[a.shape]
+    full_layers = shape["num_hidden_layers"]
+    a.layers = a.layers or full_layers
+    cfg = dict(shape, num_hidden_layers=a.layers)
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[a.dtype]
     elem = 2 if a.dtype == "bf16" else 4
     batches = [a.batch] + ([] if (a.no_points or a.only) else [1, 64])
@@ -175,11 +186,11 @@ def main() -> int:
         points[f"decode_b{b}"] = round(r["tok_s"], 1)
     flops = prefill_flops(cfg, a.prefill_tokens)
     out = {
-        "metric": "decode tok/s, Qwen2.5-7B shape, batch 8", "value": round(main_run["tok_s"], 1),
+        "metric": f"decode tok/s, {shape_name} shape, batch {a.batch}", "value": round(main_run["tok_s"], 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(main_run["ms"], 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": a.dtype, "data": "synthetic",
-        "config": {"model": "Qwen2.5-7B shape, random weights", "layers": a.layers, "layers_full": FULL_LAYERS,
+        "config": {"model": f"{shape_name} shape, random weights", "layers": a.layers, "layers_full": full_layers,
                    "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["hidden_size"] // cfg["num_attention_heads"],
                    "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],

@@ -248,16 +248,22 @@ def cu_count() -> int:
 
 
 def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None) -> Tuple[int, int]:
-    """(splits, k_per_split) of the decode product.  More than 16 rows: blocks of 128 weight rows,
-    and K split so that there is about one block per CU (measured: with four times as many,
-    the partial sums and the start of each block cost a fifth more)."""
-    if m <= 8 or (m <= 16 and k < 8192):
-        return 1, (k + 255) // 256 * 256      # one kernel: K is split between the waves of a block
-    # (9..16 rows against a long K, which the register-resident kernel does not take: in the one-kernel
-    # form every block reads its own copy of the activations from L2, 42 us at 16 rows of 18944
-    # against 33 with the staged kernel below and its reduction)
+    """(splits, k_per_split) of the decode product.  One split: one kernel, K divided between the
+    waves of a block.  More: blocks of 128 weight rows with the activations staged in LDS, K split
+    so that there is about one block per CU (measured: with four times as many, the partial sums
+    and the start of each block cost a fifth more), and a second kernel that adds the parts.
+
+    At most 16 rows take the one-kernel form, except against a long K (which the register-resident
+    kernel does not hold) where it does badly: from 9 rows on (every block reads its own copy of
+    the activations from L2: 42 us at 16 rows of 18944 against 33), and where a CU's share of the
+    weight rows fills its 16-row tiles poorly (5120 rows over 256 CUs: 20 each, 87 us against 57)."""
     if target_blocks is None:
         target_blocks = int(os.environ.get("MF_SKINNY_TARGET", 0)) or cu_count()
+    if m <= 16:
+        share = (n + target_blocks - 1) // target_blocks          # weight rows of a block in the one-kernel form
+        fill = share / float((share + 15) // 16 * 16)
+        if k < 8192 or (m <= 8 and fill >= 0.8):
+            return 1, (k + 255) // 256 * 256
     n_blocks = (n + 127) // 128
     chunks = (k + 255) // 256
     splits = max(1, min(chunks, target_blocks // max(1, n_blocks)))

@@ -200,7 +200,7 @@ def test_gemm_f32(ops, m, n, k):
                                                  # 17..64 rows, whole chunks of K: the ring kernel, with K split
                                                  (20, 200, 768), (50, 1000, 4096),
                                                  # 9..16 rows against a long K: the same kernel
-                                                 (12, 300, 8192), (16, 3584, 18944)])
+                                                 (12, 300, 8192), (16, 3584, 18944), (4, 5120, 8192)])
 def test_gemm_bf16(ops, variant, m, n, k):
     if variant and (m * n * k > 3e9):
         pytest.skip("large shape is covered by the default variant")

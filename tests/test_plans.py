@@ -12,10 +12,20 @@ def test_skinny_plan_covers_k_without_empty_splits():
         assert splits >= 1 and per % 256 == 0
         assert splits * per >= k, (m, n, k, splits, per)
         assert (splits - 1) * per < k, (m, n, k, splits, per)        # the last split has work
-        if m <= 8 or (m <= 16 and k < 8192):
+        if m <= 16 and k < 8192:
             assert splits == 1
         else:
             assert splits * ((n + 127) // 128) <= max(target, (n + 127) // 128), (m, n, k, splits)
+
+
+def test_skinny_plan_choices_at_the_model_shapes():
+    """At most 8 rows against a long K: one kernel where a CU's share of the weight rows fills its
+    tiles (3584 and 8192 rows over 256 CUs), the staged K-split kernel where it does not (5120)."""
+    assert ops.skinny_plan(8, 3584, 18944, target_blocks=256)[0] == 1
+    assert ops.skinny_plan(8, 8192, 29568, target_blocks=256)[0] == 1
+    assert ops.skinny_plan(1, 5120, 27648, target_blocks=256)[0] > 1
+    assert ops.skinny_plan(9, 3584, 18944, target_blocks=256)[0] > 1
+    assert ops.skinny_plan(16, 37888, 3584, target_blocks=256)[0] == 1
 
 
 def test_split_plan_of_the_32_bit_attention():
