@@ -69,6 +69,7 @@ _PROTOTYPES = {
         "mf_penalties": [_P, c_int, c_int, c_int, _P, c_int, _P, c_float, c_float, c_float, _P],
         "mf_top_k": [_P, c_int, c_int, c_int, c_int, _P],
         "mf_top_p": [_P, c_int, c_int, c_int, c_float, _P],
+        "mf_sample_filtered": [_P, c_int, c_int, c_int, c_int, c_float, c_float, c_uint64, _P, _P, _P, _P, _P, _P],
         "mf_advance": [_P, _P, _P, _P, c_int, _P, c_int, _P, _P, _P],
     },
 }
@@ -578,6 +579,37 @@ def top_k(logits: torch.Tensor, k: int) -> None:
 def top_p(logits: torch.Tensor, p: float) -> None:
     rows, vocab = _logit_rows(logits, "top_p.logits")
     _check(_fn("sampling", "mf_top_p")(_ptr(logits), vocab, rows, vocab, float(p), _stream()), "top_p")
+
+
+FILTERED_K_MAX = 48            # the largest top-k that `sample_filtered` takes
+FILTERED_VOCAB_MAX = 32 * 256 * 32
+
+
+def sample_filtered_takes(vocab: int, k: int, temp: float) -> bool:
+    """Whether `sample_filtered` covers these settings (else: top_k, top_p, sample one after the other)."""
+    return 1 <= k <= FILTERED_K_MAX and k < vocab <= FILTERED_VOCAB_MAX and temp >= 1e-6
+
+
+def sample_filtered(logits: torch.Tensor, k: int, p: float, temp: float, seed: int, keys: torch.Tensor,
+                    steps: torch.Tensor, out: torch.Tensor, forced_r: Optional[torch.Tensor] = None) -> None:
+    """top-k, then top-p (off unless 0 < p < 1), then the temperature draw, as `top_k`, `top_p` and
+    `sample` one after the other give it, but reading each row once: its k largest entries and their
+    ties are picked out by 32 blocks a row and the rest runs on those few.  The logits stay as they
+    are, except for rows with more equal values than the lists hold, which take the whole-row
+    kernels in place."""
+    rows, vocab = _logit_rows(logits, "sample_filtered.logits")
+    if not sample_filtered_takes(vocab, k, temp):
+        raise KernelError(f"sample_filtered: k {k}, vocabulary {vocab}, temperature {temp} are outside what it takes")
+    _need(keys, "sample_filtered.keys", torch.int64, (rows,))
+    _need(steps, "sample_filtered.steps", torch.int32, (rows,))
+    _need(out, "sample_filtered.out", torch.int32, (rows,))
+    if forced_r is not None:
+        _need(forced_r, "sample_filtered.forced_r", torch.float32, (rows,))
+    work = workspace("sample_filtered", rows * 32 * (2 * 64 + 1), logits.device)
+    _check(_fn("sampling", "mf_sample_filtered")(_ptr(logits), vocab, rows, vocab, int(k), float(p), float(temp),
+                                                  seed & 0xFFFFFFFFFFFFFFFF, _ptr(keys), _ptr(steps),
+                                                  _ptr(forced_r), _ptr(work), _ptr(out), _stream()),
+           "sample_filtered")
 
 
 def advance(next_ids: torch.Tensor, sampled: torch.Tensor, positions: torch.Tensor, steps: torch.Tensor,

@@ -1,6 +1,7 @@
 """The sampling pipeline on the device, in the reference's order: penalties -> greedy if
 temperature < 1e-6 -> top-k -> top-p -> temperature draw (`sample_with_penalties`,
-src/sampler.rs:272-290 of yusiwen/minfer).  Logits are changed in place."""
+src/sampler.rs:272-290 of yusiwen/minfer).  Logits are changed in place (a small top-k takes one
+fused kernel for the last three steps, which leaves them alone)."""
 from __future__ import annotations
 
 from typing import Optional
@@ -28,6 +29,9 @@ class Sampler:
             ops.penalties(logits, prev, n_prev, p.repeat_penalty, p.frequency_penalty, p.presence_penalty)
         if p.is_greedy:
             ops.argmax(logits, out)
+            return out
+        if ops.sample_filtered_takes(logits.shape[-1], p.top_k, p.temp):
+            ops.sample_filtered(logits, p.top_k, p.top_p, p.temp, p.seed, keys, steps, out)
             return out
         if p.top_k > 0:
             ops.top_k(logits, p.top_k)

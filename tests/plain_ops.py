@@ -220,6 +220,18 @@ def top_p(logits, p):
         logits[i] = torch.from_numpy(pq.apply_top_p(logits[i].numpy(), p))
 
 
+def sample_filtered_takes(vocab, k, temp):
+    return 1 <= k <= 48 and k < vocab <= 32 * 256 * 32 and temp >= 1e-6
+
+
+def sample_filtered(logits, k, p, temp, seed, keys, steps, out, forced_r=None):
+    work = logits.clone()
+    top_k(work, k)
+    if 0.0 < p < 1.0:
+        top_p(work, p)
+    sample(work, temp, seed, keys, steps, out, forced_r)
+
+
 def advance(next_ids, sampled, positions, steps, prev=None, n_prev=None, cursor=None):
     next_ids.copy_(sampled)
     positions += 1
@@ -234,7 +246,7 @@ def advance(next_ids, sampled, positions, steps, prev=None, n_prev=None, cursor=
 
 NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", "rope_table",
          "rope_kvwrite", "linear", "attn_tokens", "attn_prefill", "argmax", "sample", "penalties",
-         "top_k", "top_p", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed", "attn_decode_rope"]
+         "top_k", "top_p", "sample_filtered", "sample_filtered_takes", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed", "attn_decode_rope"]
 
 
 def install(monkeypatch):

@@ -111,6 +111,54 @@ def test_temperature_draw_matches_plain(ops, vocab, temp):
         assert out[0].item() == want
 
 
+@pytest.mark.parametrize("rows,vocab,k,p,temp", [(8, 152064, 40, 0.95, 0.8), (6, 1000, 40, 0.9, 0.7),
+                                                 (5, 777, 1, 0.55, 1.3), (6, 5000, 48, 1.0, 0.8),
+                                                 (5, 300, 40, 0.95, 0.8), (64, 32000, 20, 0.8, 1.0)])
+def test_sample_filtered_is_top_k_top_p_and_the_draw(ops, rows, vocab, k, p, temp):
+    """The fused kernels give the tokens of the three whole-row kernels one after the other, with
+    ties at the k-th value, with fewer finite entries than k, and for a constant row (more equal
+    values than the lists hold: the whole-row kernels run inside); they leave the logits alone
+    where they can."""
+    l = logits_rows(rows, vocab, 11)
+    l[1, :50] = 9.0                                            # ties that reach into the k largest
+    l[2] = float("-inf")
+    l[2, [3, vocab // 2, vocab - 1]] = torch.tensor([0.5, 1.5, 1.0])     # fewer finite entries than k
+    l[3] = 0.25                                                # a constant row
+    rs = np.random.default_rng(12).random(rows).astype(np.float32)
+    rs[0], rs[4] = 0.0, 0.99999994
+    forced = torch.from_numpy(rs).to(DEV)
+    keys = torch.zeros(rows, dtype=torch.int64, device=DEV)
+    steps = torch.zeros(rows, dtype=torch.int32, device=DEV)
+    chain = l.to(DEV).clone()
+    want = torch.empty(rows, dtype=torch.int32, device=DEV)
+    ops.top_k(chain, k)
+    ops.top_p(chain, p)
+    ops.sample(chain, temp, 0, keys, steps, want, forced)
+    d = l.to(DEV).clone()
+    got = torch.empty(rows, dtype=torch.int32, device=DEV)
+    assert ops.sample_filtered_takes(vocab, k, temp)
+    ops.sample_filtered(d, k, p, temp, 0, keys, steps, got, forced)
+    assert got.cpu().tolist() == want.cpu().tolist()
+    untouched = [i for i in range(rows) if i != 3]
+    assert torch.equal(d[untouched].cpu(), l[untouched])
+    # and the tokens are the plain sampler's (but for the constant row, where a walk over the
+    # whole vocabulary in 32 bits, as the plain sampler does it, drifts, and for the draw next to 1,
+    # where the last bit of the probabilities' sum decides between the last kept token and the
+    # fallback)
+    for i in untouched:
+        if i != 4:
+            assert int(got[i]) == pq.sample(l[i].numpy(), temp, float(rs[i]), k, p, 1.0, 0.0, 0.0, [])
+    # without forced draws: the generator's uniform, as `sample` takes it
+    keys = torch.arange(rows, dtype=torch.int64, device=DEV) + 5
+    steps = torch.arange(rows, dtype=torch.int32, device=DEV)
+    chain = l.to(DEV).clone()
+    ops.top_k(chain, k)
+    ops.top_p(chain, p)
+    ops.sample(chain, temp, 77, keys, steps, want)
+    ops.sample_filtered(l.to(DEV).clone(), k, p, temp, 77, keys, steps, got)
+    assert got.cpu().tolist() == want.cpu().tolist()
+
+
 def test_device_uniform_is_the_host_uniform_and_draws_follow_softmax(ops):
     rows, vocab = 4000, 3
     small = torch.tensor([0.0, 1.0, 2.0]).repeat(rows, 1).to(DEV)
