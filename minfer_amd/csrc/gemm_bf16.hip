@@ -122,9 +122,18 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const 
                                                    const bf16* __restrict__ W, int ldw,
                                                    const float* __restrict__ bias, void* __restrict__ C,
                                                    int ldc, int M, int N, int K, int epi, int tiles_m,
-                                                   int xcd_remap) {
+                                                   int xcd_remap, int k_per_split) {
   constexpr int NTHR = 64 * (BM / WM) * (BN / WN);
   constexpr int LDS_LD = BK + 8;
+  if (k_per_split > 0) {
+    // K split over blockIdx.y: this block multiplies k_per_split of K and stores its sums, 32-bit
+    // and without bias, into its own [M][N] slab of C; another kernel adds the slabs
+    const int kb = blockIdx.y * k_per_split;
+    A += kb;
+    W += kb;
+    K = min(k_per_split, K - kb);
+    C = (float*)C + (size_t)blockIdx.y * M * N;
+  }
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int RP = NTHR / (BK / 8);         // rows per load pass
   constexpr int PA = BM / RP, PW = BN / RP;
@@ -408,7 +417,7 @@ int launch_tile_dma(const bf16* A, int lda, const bf16* W, int ldw, const float*
 
 template <int BM, int BN, int WM, int WN, int BK, bool VEC>
 int launch_tile_v(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
-                  int M, int N, int K, int epi, hipStream_t stream) {
+                  int M, int N, int K, int epi, hipStream_t stream, int splits = 1, int k_per_split = 0) {
   constexpr int smem = 2 * (BM + BN) * (BK + 8) * (int)sizeof(bf16);
   constexpr int NTHR = 64 * (BM / WM) * (BN / WN);
   static bool configured = false;
@@ -421,16 +430,20 @@ int launch_tile_v(const bf16* A, int lda, const bf16* W, int ldw, const float* b
   }
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   static const int remap = getenv("MF_NO_XCD_REMAP") ? 0 : 1;
-  kern<<<tiles_m * tiles_n, NTHR, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, tiles_m,
-                                                  remap && tiles_m * tiles_n >= 16);
+  kern<<<dim3(tiles_m * tiles_n, splits), NTHR, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi,
+                                                                tiles_m, remap && tiles_m * tiles_n >= 16,
+                                                                k_per_split);
   return mf_launch_status();
 }
 
 template <int BM, int BN, int WM, int WN, int BK = 64>
 int launch_tile(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
-                int M, int N, int K, int epi, int vec_ok, hipStream_t stream) {
-  return vec_ok ? launch_tile_v<BM, BN, WM, WN, BK, true>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, stream)
-                : launch_tile_v<BM, BN, WM, WN, BK, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, stream);
+                int M, int N, int K, int epi, int vec_ok, hipStream_t stream, int splits = 1,
+                int k_per_split = 0) {
+  return vec_ok ? launch_tile_v<BM, BN, WM, WN, BK, true>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, stream,
+                                                          splits, k_per_split)
+                : launch_tile_v<BM, BN, WM, WN, BK, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, stream,
+                                                           splits, k_per_split);
 }
 
 // ------------------------------------------------------------------ skinny kernel
@@ -1403,6 +1416,29 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
       return launch_tile_dma(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
   }
   return (int)hipErrorInvalidValue;
+}
+
+// Few rows for the tile kernel (a prompt of a few hundred tokens against 3584 weight rows makes
+// some 50 tiles for 256 CUs): K is split over `splits` blocks per tile, which store 32-bit sums
+// into part[splits][M][N], and skinny_reduce_kernel adds them and runs the epilogue.
+// k_per_split is a multiple of 64.
+MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
+                               int ldc, float* part, int M, int N, int K, int splits, int k_per_split,
+                               int epi, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > 3 || splits < 2 || !part || k_per_split % 64 != 0 ||
+      (long)splits * k_per_split < K || (long)(splits - 1) * k_per_split >= K)
+    return (int)hipErrorInvalidValue;
+  if (epi == EPI_SWIGLU ? (N % 64 != 0 || ldc > N / 2 || ldc <= N / 2 - 32 || bias) : ldc < N)
+    return (int)hipErrorInvalidValue;
+  const int vec_ok = (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) &&
+                     ((uintptr_t)W % 16 == 0) && (K % 8 == 0);
+  int rc = launch_tile<128, 128, 64, 64>((const bf16*)A, lda, (const bf16*)W, ldw, nullptr, part, N, M, N, K,
+                                         EPI_F32, vec_ok, stream, splits, k_per_split);
+  if (rc) return rc;
+  dim3 g2(((epi == EPI_SWIGLU ? ldc : N) + 255) / 256, M);
+  skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, splits, epi);
+  return mf_launch_status();
 }
 
 // The register-resident kernel for the shapes it is built for (K = 256 NS with enough tiles to

@@ -44,6 +44,7 @@ _PROTOTYPES = {
     },
     "gemm_bf16": {
         "mf_gemm_bf16": [_P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_gemm_bf16_splitk": [_P, c_int, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_gemm_bf16_skinny": [_P, c_int, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int,
                                 c_int, c_int, _P],
         "mf_gemm_bf16_normed": [_P, c_int, _P, _P, c_float, _P, c_int, _P, _P, c_int, c_int, c_int, c_int,
@@ -272,6 +273,21 @@ def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None) -> 
     return (chunks + per - 1) // per, per * 256
 
 
+def tile_split_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None) -> Tuple[int, int]:
+    """(splits, k_per_split) of the tile product; (1, k) where its 128 x 128 tiles alone fill the
+    chip.  A prompt of a few hundred tokens against a few thousand weight rows makes some 50 tiles
+    for 256 CUs and is bound by the weight stream: K is split so that there are about two blocks
+    per CU, each with at least 512 of K, and a second kernel adds the parts."""
+    cu = target_blocks if target_blocks is not None else cu_count()
+    tiles = ((m + 127) // 128) * ((n + 127) // 128)
+    chunks = (k + 255) // 256
+    splits = min(chunks // 2, (2 * cu) // max(1, tiles))
+    if tiles >= cu or splits < 2:
+        return 1, k
+    per = (chunks + splits - 1) // splits
+    return (chunks + per - 1) // per, per * 256
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
            accumulate: bool = False, variant: int = 0) -> None:
     """out (+)= x @ weight^T (+ bias).  weight is [out][in].  float32 weights take the true
@@ -303,6 +319,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
                                                         _ptr(out), n, _ptr(part), m, n, k, splits, per,
                                                         epi, _stream()), "gemm_bf16_skinny")
         return
+    if variant == 0:
+        splits, per = tile_split_plan(m, n, k)
+        if splits > 1:
+            part = workspace("skinny", splits * m * n, x.device)
+            _check(_fn("gemm_bf16", "mf_gemm_bf16_splitk")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n,
+                                                            _ptr(part), m, n, k, splits, per, epi, _stream()),
+                   "gemm_bf16_splitk")
+            return
     _check(_fn("gemm_bf16", "mf_gemm_bf16")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n, m,
                                              n, k, epi, variant, _stream()), "gemm_bf16")
 
@@ -339,6 +363,14 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, vari
                                                         _ptr(part), m, n, k, splits, per, EPI_SWIGLU, _stream()),
                "gemm_bf16_skinny(swiglu)")
         return
+    if variant == 0:
+        splits, per = tile_split_plan(m, n, k)
+        if splits > 1:
+            part = workspace("skinny", splits * m * n, x.device)
+            _check(_fn("gemm_bf16", "mf_gemm_bf16_splitk")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
+                                                            _ptr(part), m, n, k, splits, per, EPI_SWIGLU,
+                                                            _stream()), "gemm_bf16_splitk(swiglu)")
+            return
     _check(_fn("gemm_bf16", "mf_gemm_bf16")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf, m, n, k,
                                              EPI_SWIGLU, variant, _stream()), "gemm_bf16(swiglu)")
 

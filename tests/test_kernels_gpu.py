@@ -200,7 +200,9 @@ def test_gemm_f32(ops, m, n, k):
                                                  # 17..64 rows, whole chunks of K: the ring kernel, with K split
                                                  (20, 200, 768), (50, 1000, 4096),
                                                  # 9..16 rows against a long K: the same kernel
-                                                 (12, 300, 8192), (16, 3584, 18944), (4, 5120, 8192)])
+                                                 (12, 300, 8192), (16, 3584, 18944), (4, 5120, 8192),
+                                                 # more than 64 rows but few tiles: K split over blocks
+                                                 (200, 3584, 18944), (65, 1000, 1100), (512, 777, 2048)])
 def test_gemm_bf16(ops, variant, m, n, k):
     if variant and (m * n * k > 3e9):
         pytest.skip("large shape is covered by the default variant")
@@ -493,7 +495,9 @@ def test_gemm_bf16_wide_few_rows(ops, m, n, k):
                                     (65, 232, 200), (300, 18944, 256), (130, 31, 72),
                                     (8, 1100, 1536), (3, 2100, 3584), (16, 1030, 4096), (1, 1024, 2048),
                                     # 17..64 rows against a wide matrix: one block per CU over the whole of K
-                                    (64, 18944, 512), (33, 16400, 256), (40, 300, 512), (10, 96, 8192)])
+                                    (64, 18944, 512), (33, 16400, 256), (40, 300, 512), (10, 96, 8192),
+                                    # more than 64 rows but few tiles: K split over blocks
+                                    (100, 1000, 1024), (200, 512, 3584)])
 def test_gemm_bf16_swiglu(ops, variant, m, nf, k):
     if variant == 12 and k % 64:
         pytest.skip("the direct-to-LDS pipeline takes k in steps of 64")

@@ -28,6 +28,20 @@ def test_skinny_plan_choices_at_the_model_shapes():
     assert ops.skinny_plan(16, 37888, 3584, target_blocks=256)[0] == 1
 
 
+def test_tile_split_plan():
+    for m, n, k in itertools.product((65, 128, 200, 1024, 2048, 8192), (96, 3584, 4608, 37888), (64, 256, 3584, 18944)):
+        splits, per = ops.tile_split_plan(m, n, k, target_blocks=256)
+        if splits == 1:
+            assert per == k
+            continue
+        assert per % 256 == 0 and per >= 512
+        assert splits * per >= k and (splits - 1) * per < k
+        tiles = ((m + 127) // 128) * ((n + 127) // 128)
+        assert tiles < 256 and splits * tiles <= 512
+    assert ops.tile_split_plan(2048, 3584, 18944, target_blocks=256) == (1, 18944)       # 448 tiles: enough
+    assert ops.tile_split_plan(200, 3584, 18944, target_blocks=256)[0] == 9
+
+
 def test_split_plan_of_the_32_bit_attention():
     for n_tok, nk, group, hd, max_len in itertools.product((1, 8, 64, 300), (1, 2, 4), (1, 5, 7), (16, 128, 256),
                                                            (1, 64, 100, 4096, 32768)):
