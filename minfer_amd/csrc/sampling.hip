@@ -41,6 +41,26 @@ __device__ __forceinline__ float exp_rel(float l, float mx) { return expf(l - mx
 __device__ __forceinline__ float prob_of(float l, float mx, float inv) { return exp_rel(l, mx) * inv; }
 __device__ __forceinline__ float share_of(float l, float mx, float tot) { return exp_rel(l, mx) / tot; }
 
+// f(i, row[i]) for i in [lo, hi) in index order, until f returns false.  A thread's run of
+// consecutive entries is read 16 bytes at a time where the row allows: the lanes of such a load
+// sit in 64 different cache lines, each a look-up of its own in the CU's cache, so four entries a
+// look-up instead of one.
+template <typename F>
+__device__ __forceinline__ void for_run(const float* __restrict__ row, int lo, int hi, F f) {
+  int i = lo;
+  if ((reinterpret_cast<uintptr_t>(row + lo) & 15) == 0) {
+    for (; i + 3 < hi; i += 4) {
+      const float4 v = *reinterpret_cast<const float4*>(row + i);
+      if (!f(i, v.x) || !f(i + 1, v.y) || !f(i + 2, v.z) || !f(i + 3, v.w)) return;
+    }
+  }
+  for (; i < hi; ++i)
+    if (!f(i, row[i])) return;
+}
+
+// entries per thread when a row is cut into runs: a multiple of 4, for the 16-byte reads
+__device__ __forceinline__ int run_length(int vocab) { return (((vocab + NT - 1) / NT) + 3) & ~3; }
+
 __device__ __forceinline__ double wave_sum_d(double v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, MF_WAVE);
@@ -158,21 +178,23 @@ __device__ __forceinline__ void sample_row(const float* __restrict__ row, int ro
     return;
   }
   // contiguous chunk per thread so that the walk is in index order
-  const int chunk = (vocab + NT - 1) / NT;
+  const int chunk = run_length(vocab);
   const int lo = min(vocab, (int)threadIdx.x * chunk), hi = min(vocab, lo + chunk);
   double mine = 0.0;
-  for (int i = lo; i < hi; ++i) {
-    const float l = scaled(row[i], inv_t);
+  for_run(row, lo, hi, [&](int, float x) {
+    const float l = scaled(x, inv_t);
     if (l > -INFINITY) mine += (double)exp_rel(l, mx);
-  }
+    return true;
+  });
   const double total = block_sum_d(mine, s_d);
   const float inv = (float)(1.0 / total);
   // probabilities as the reference forms them: e * (1/sum as f32)
   double pm = 0.0;
-  for (int i = lo; i < hi; ++i) {
-    const float l = scaled(row[i], inv_t);
+  for_run(row, lo, hi, [&](int, float x) {
+    const float l = scaled(x, inv_t);
     if (l > -INFINITY) pm += (double)prob_of(l, mx, inv);
-  }
+    return true;
+  });
   // exclusive scan of pm over threads: within the wave, then over wave totals
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   double incl = pm;
@@ -194,15 +216,15 @@ __device__ __forceinline__ void sample_row(const float* __restrict__ row, int ro
   if (pm > 0.0 && prefix < rr && rr <= prefix + pm) {
     double cum = prefix;
     int pick = -1;
-    for (int i = lo; i < hi; ++i) {
-      const float l = scaled(row[i], inv_t);
-      if (!(l > -INFINITY)) continue;
+    for_run(row, lo, hi, [&](int i, float x) {
+      const float l = scaled(x, inv_t);
+      if (!(l > -INFINITY)) return true;
       const float p = prob_of(l, mx, inv);
-      if (p <= 0.f) continue;
+      if (p <= 0.f) return true;
       cum += (double)p;
       pick = i;
-      if (rr <= cum) break;
-    }
+      return !(rr <= cum);
+    });
     if (pick >= 0) s_found = pick;
   }
   __syncthreads();
@@ -318,11 +340,13 @@ __device__ __forceinline__ void top_p_row(float* __restrict__ row, int vocab, fl
   int amax;
   block_argmax(row, vocab, 1.0f, s_val, s_idx, mx, amax);
   if (!(mx > -INFINITY)) return;
-  const int chunk = (vocab + NT - 1) / NT;
+  const int chunk = run_length(vocab);
   const int lo = min(vocab, (int)threadIdx.x * chunk), hi = min(vocab, lo + chunk);
   double mine = 0.0;
-  for (int i = lo; i < hi; ++i)
-    if (row[i] > -INFINITY) mine += exp((double)(row[i] - mx));
+  for_run(row, lo, hi, [&](int, float x) {
+    if (x > -INFINITY) mine += exp((double)(x - mx));
+    return true;
+  });
   const double total = block_sum_d(mine, s_d);
   const float tot_f = (float)total;
   if (threadIdx.x == 0) { s_prefix = 0; s_above = 0.0; }
@@ -332,15 +356,16 @@ __device__ __forceinline__ void top_p_row(float* __restrict__ row, int vocab, fl
     __syncthreads();
     const uint32_t prefix = s_prefix;
     const uint32_t mask = pass == 0 ? 0u : (0xFFFFFFFFu << (shift + 8));
-    for (int i = lo; i < hi; ++i) {
-      if (!(row[i] > -INFINITY)) continue;
-      const float pr = share_of(row[i], mx, tot_f);
+    for_run(row, lo, hi, [&](int, float x) {
+      if (!(x > -INFINITY)) return true;
+      const float pr = share_of(x, mx, tot_f);
       const uint32_t key = __float_as_uint(pr);        // pr >= 0: bit order is value order
       if ((key & mask) == prefix) {
         atomicAdd(&bin_mass[(key >> shift) & 255u], (double)pr);
         atomicAdd(&bin_count[(key >> shift) & 255u], 1u);
       }
-    }
+      return true;
+    });
     __syncthreads();
     if (threadIdx.x == 0) {
       double above = s_above;
@@ -366,8 +391,10 @@ __device__ __forceinline__ void top_p_row(float* __restrict__ row, int vocab, fl
   }
   // rank of each tie in index order: count per thread chunk, exclusive scan
   unsigned int my_ties = 0;
-  for (int i = lo; i < hi; ++i)
-    if (row[i] > -INFINITY && __float_as_uint(share_of(row[i], mx, tot_f)) == tau_key) ++my_ties;
+  for_run(row, lo, hi, [&](int, float x) {
+    if (x > -INFINITY && __float_as_uint(share_of(x, mx, tot_f)) == tau_key) ++my_ties;
+    return true;
+  });
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   unsigned int incl = my_ties;
 #pragma unroll
@@ -380,13 +407,14 @@ __device__ __forceinline__ void top_p_row(float* __restrict__ row, int vocab, fl
   __syncthreads();
   unsigned int rank = incl - my_ties;
   for (int i = 0; i < w; ++i) rank += s_wave_cnt[i];
-  for (int i = lo; i < hi; ++i) {
-    if (!(row[i] > -INFINITY)) continue;
-    const uint32_t key = __float_as_uint(share_of(row[i], mx, tot_f));
-    if (key > tau_key) continue;
-    if (key == tau_key && rank++ < keep_ties) continue;
+  for_run(row, lo, hi, [&](int i, float x) {
+    if (!(x > -INFINITY)) return true;
+    const uint32_t key = __float_as_uint(share_of(x, mx, tot_f));
+    if (key > tau_key) return true;
+    if (key == tau_key && rank++ < keep_ties) return true;
     row[i] = -INFINITY;
-  }
+    return true;
+  });
   __syncthreads();      // what follows in the same block reads the row
 }
 
