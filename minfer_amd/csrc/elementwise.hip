@@ -35,6 +35,36 @@ MF_API int mf_embed(const void* table, int table_is_bf16, const int* ids, float*
 // ---------------------------------------------------------------- RMSNorm
 // y = x * (1/sqrt(mean(x^2) + eps)) * w  (src/vec_ops.rs:500-522; eps inside the root).
 // Row r of the output reads row row_idx[r] of x when row_idx is given.
+// A row of at most 256 * 4 * KEEP elements stays in registers between the sum and the scaling.
+template <typename OT, int KEEP>
+__device__ __forceinline__ void rmsnorm_row_kept(const float* __restrict__ xr, const float* __restrict__ w,
+                                                 OT* __restrict__ o, int d, float eps, float* scratch) {
+  float4 v[KEEP];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < KEEP; ++c) {
+    const int i = (c * 256 + threadIdx.x) * 4;
+    v[c] = i < d ? *reinterpret_cast<const float4*>(xr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    ss = fmaf(v[c].x, v[c].x, ss);
+    ss = fmaf(v[c].y, v[c].y, ss);
+    ss = fmaf(v[c].z, v[c].z, ss);
+    ss = fmaf(v[c].w, v[c].w, ss);
+  }
+  ss = block_sum<256>(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+  for (int c = 0; c < KEEP; ++c) {
+    const int i = (c * 256 + threadIdx.x) * 4;
+    if (i < d) {
+      const float4 g = w ? *reinterpret_cast<const float4*>(w + i) : make_float4(1.f, 1.f, 1.f, 1.f);
+      o[i + 0] = from_f32<OT>(v[c].x * scale * g.x);
+      o[i + 1] = from_f32<OT>(v[c].y * scale * g.y);
+      o[i + 2] = from_f32<OT>(v[c].z * scale * g.z);
+      o[i + 3] = from_f32<OT>(v[c].w * scale * g.w);
+    }
+  }
+}
+
 template <typename OT>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x,
                                                       const int* __restrict__ row_idx,
@@ -44,33 +74,10 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
   const int row = blockIdx.x;
   const float* xr = x + (size_t)(row_idx ? row_idx[row] : row) * d;
   OT* o = out + (size_t)row * d;
-  // rows up to 256 * 4 * KEEP elements stay in registers between the sum and the scaling
-  constexpr int KEEP = 4;
-  if (d % 4 == 0 && d <= 256 * 4 * KEEP) {
-    float4 v[KEEP];
-    float ss = 0.f;
-#pragma unroll
-    for (int c = 0; c < KEEP; ++c) {
-      const int i = (c * 256 + threadIdx.x) * 4;
-      v[c] = i < d ? *reinterpret_cast<const float4*>(xr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
-      ss = fmaf(v[c].x, v[c].x, ss);
-      ss = fmaf(v[c].y, v[c].y, ss);
-      ss = fmaf(v[c].z, v[c].z, ss);
-      ss = fmaf(v[c].w, v[c].w, ss);
-    }
-    ss = block_sum<256>(ss, scratch);
-    const float scale = 1.0f / sqrtf(ss / (float)d + eps);
-#pragma unroll
-    for (int c = 0; c < KEEP; ++c) {
-      const int i = (c * 256 + threadIdx.x) * 4;
-      if (i < d) {
-        const float4 g = w ? *reinterpret_cast<const float4*>(w + i) : make_float4(1.f, 1.f, 1.f, 1.f);
-        o[i + 0] = from_f32<OT>(v[c].x * scale * g.x);
-        o[i + 1] = from_f32<OT>(v[c].y * scale * g.y);
-        o[i + 2] = from_f32<OT>(v[c].z * scale * g.z);
-        o[i + 3] = from_f32<OT>(v[c].w * scale * g.w);
-      }
-    }
+  if (d % 4 == 0 && d <= 256 * 4 * 16) {
+    if (d <= 256 * 4 * 4) rmsnorm_row_kept<OT, 4>(xr, w, o, d, eps, scratch);
+    else if (d <= 256 * 4 * 8) rmsnorm_row_kept<OT, 8>(xr, w, o, d, eps, scratch);
+    else rmsnorm_row_kept<OT, 16>(xr, w, o, d, eps, scratch);
     return;
   }
   float ss = 0.f;

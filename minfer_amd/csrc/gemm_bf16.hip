@@ -8,8 +8,8 @@
 //    steps of BK through double-buffered LDS, 32x32x16 MFMA, each wave a WM x WN tile.
 //  * `tile_dma_kernel`: the 256 x 256 tile with its k tiles copied straight into LDS; the
 //    choice for large aligned products.
-//  * `stationary16_kernel`: at most 16 rows and K of 1536, 2048, 3584 or 4096 (decode): one
-//    block per CU keeps the activations in registers and walks over weight tiles.
+//  * `stationary16_kernel`: at most 16 rows and K of 1536, 2048, 3584, 4096, 5120 or 8192 (decode):
+//    one block per CU keeps the activations in registers and walks over weight tiles.
 //  * `rolling16_kernel`, `skinny16_kernel`: at most 16 rows, any K (decode).  The time is the
 //    weight stream: the waves of a block split K, each reads weights and activations straight
 //    into MFMA operands (16x16x32) and the partial sums meet in LDS.
@@ -921,7 +921,12 @@ struct NormArgs {
   float eps;
 };
 
-template <int NS, int NT, bool PAIR, bool NORM>
+//
+// RING: how many of a slice's NS steps of weights a wave keeps in flight (a divisor of NS).  With
+// RING = NS the registers hold a whole item; for a long K (5120, 8192) the activations alone take
+// up to half the registers, so the weights go through a shorter ring, and a register is refilled
+// with the step RING further on, of this item or of the next one.
+template <int NS, int RING, int NT, bool PAIR, bool NORM>
 __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restrict__ Av, int lda,
                                                            const bf16* __restrict__ W, int ldw,
                                                            const float* __restrict__ bias,
@@ -932,7 +937,8 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
   constexpr int RS = COLS + 4;             // row stride of the sums in LDS: conflict-free writes
   __shared__ float red[2][NW][16][RS];     // [buffer][wave][activation row][weight row of the item]
   __shared__ float ssq[NW][16];            // NORM: sum of x^2 over a wave's slice, per activation row
-  __shared__ __attribute__((aligned(16))) float gs[NORM ? NW * NS * 32 : 4];   // NORM: the norm's weight
+  extern __shared__ __attribute__((aligned(16))) float gs[];   // NORM: the norm's weight, K floats
+  static_assert(NS % RING == 0, "the ring divides a slice");
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int r16 = lane & 15;
   const int k0 = wid * NS * 32 + (lane >> 4) * 8;         // this lane's k in step 0 of its slice
@@ -953,45 +959,23 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
     }
     return min(c0 + 16 * j + r16, c_end - 1);
   };
-  bf16x8 w[NT][NS];
-  const bf16* wrow[NT];
+  const bf16* Wp = W;            // the weights, through a name whose use can be held back
+  bf16x8 w[NT][RING];
+  const bf16* wrow[NT];          // this lane's rows in the next item
+  const bf16* wcur[NT];          // and in the current one (used when RING < NS)
   const int item = 0;
   auto first_loads = [&](int j) {
-    wrow[j] = W + (size_t)lane_wrow(c_begin, j) * ldw + k0;
+    wcur[j] = Wp + (size_t)lane_wrow(c_begin, j) * ldw + k0;
 #pragma unroll
-    for (int s = 0; s < NS; ++s) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32);
+    for (int s = 0; s < RING; ++s) w[j][s] = *reinterpret_cast<const bf16x8*>(wcur[j] + s * 32);
   };
   bf16x8 afr[NS];
   float ss = 0.f;
   if constexpr (NORM) {
-    // Everything the prologue needs is asked for at once, oldest first in the order it is
-    // used: the norm's weight (staged in LDS for all waves), this lane's x, and the first
-    // item's tile 0, which keeps HBM at work while the activations are converted.  The order is
-    // pinned: left alone, the compiler asks for the weights first and then waits for them
-    // before it stages g.
-    static_assert(NW * NS * 32 <= 2 * NW * 64 * 4, "two float4 of g per thread cover K");
-    const int ge0 = min((int)threadIdx.x * 4, NW * NS * 32 - 4);                 // the last ones twice
-    const int ge1 = min((NW * 64 + (int)threadIdx.x) * 4, NW * NS * 32 - 4);
-    const float4 gt0 = *reinterpret_cast<const float4*>(norm.g + ge0);
-    const float4 gt1 = *reinterpret_cast<const float4*>(norm.g + ge1);
     const int m_src = min(r16, M - 1);
     const float* xrow = (const float*)Av + (size_t)(norm.row_idx ? norm.row_idx[m_src] : m_src) * lda + k0;
-    float4 x[NS][2];
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      x[s][0] = *reinterpret_cast<const float4*>(xrow + s * 32);
-      x[s][1] = *reinterpret_cast<const float4*>(xrow + s * 32 + 4);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    if (item < n_items) first_loads(0);
-    __builtin_amdgcn_sched_barrier(0);
-    *reinterpret_cast<float4*>(&gs[ge0]) = gt0;
-    *reinterpret_cast<float4*>(&gs[ge1]) = gt1;
-    __syncthreads();
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      const float4 x0 = x[s][0], x1 = x[s][1];
+    // step s of the slice: sum of squares, and bf16(x * g) into the operand registers
+    auto convert_step = [&](int s, const float4 x0, const float4 x1) {
       const float4 g0 = *reinterpret_cast<const float4*>(&gs[k0 + s * 32]);
       const float4 g1 = *reinterpret_cast<const float4*>(&gs[k0 + s * 32 + 4]);
       ss = fmaf(x0.x, x0.x, ss); ss = fmaf(x0.y, x0.y, ss); ss = fmaf(x0.z, x0.z, ss); ss = fmaf(x0.w, x0.w, ss);
@@ -1002,7 +986,68 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
       afr[s][6] = (bf16)(x1.z * g1.z); afr[s][7] = (bf16)(x1.w * g1.w);
       // the packed value is wanted here and now (left alone, the compiler keeps x and g
       // alive and converts in front of the first MFMA, at twice the registers)
-      asm volatile("" : "+v"(afr[s]));
+      // (and for a long row the sum as well: put off, it keeps x alive in 32 bits)
+      if constexpr (NS <= 16) asm volatile("" : "+v"(afr[s]));
+      else asm volatile("" : "+v"(afr[s]), "+v"(ss));
+    };
+    if constexpr (NS <= 16) {
+      // Everything the prologue needs is asked for at once, oldest first in the order it is
+      // used: the norm's weight (staged in LDS for all waves), this lane's x, and the first
+      // item's tile 0, which keeps HBM at work while the activations are converted.  The order is
+      // pinned: left alone, the compiler asks for the weights first and then waits for them
+      // before it stages g.
+      static_assert(NS > 16 || NW * NS * 32 <= 2 * NW * 64 * 4, "two float4 of g per thread cover K");
+      const int ge0 = min((int)threadIdx.x * 4, NW * NS * 32 - 4);                 // the last ones twice
+      const int ge1 = min((NW * 64 + (int)threadIdx.x) * 4, NW * NS * 32 - 4);
+      const float4 gt0 = *reinterpret_cast<const float4*>(norm.g + ge0);
+      const float4 gt1 = *reinterpret_cast<const float4*>(norm.g + ge1);
+      float4 x[NS][2];
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        x[s][0] = *reinterpret_cast<const float4*>(xrow + s * 32);
+        x[s][1] = *reinterpret_cast<const float4*>(xrow + s * 32 + 4);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (item < n_items) first_loads(0);
+      __builtin_amdgcn_sched_barrier(0);
+      *reinterpret_cast<float4*>(&gs[ge0]) = gt0;
+      *reinterpret_cast<float4*>(&gs[ge1]) = gt1;
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < NS; ++s) convert_step(s, x[s][0], x[s][1]);
+    } else {
+      // A long row does not fit the registers in 32 bits beside its own bf16 copy: x comes in
+      // sets of XC steps, the next set asked for before this one is converted, and the first
+      // weights wait until the activations are in place.
+      constexpr int XC = 4, SETS = NS / XC;
+      static_assert(NS % XC == 0, "whole sets");
+      float4 x[2][XC][2];
+      const float* xp = xrow;
+      auto load_set = [&](int c, int b) {
+#pragma unroll
+        for (int i = 0; i < XC; ++i) {
+          x[b][i][0] = *reinterpret_cast<const float4*>(xp + (c * XC + i) * 32);
+          x[b][i][1] = *reinterpret_cast<const float4*>(xp + (c * XC + i) * 32 + 4);
+        }
+      };
+      load_set(0, 0);
+      for (int e = (int)threadIdx.x * 4; e < NW * NS * 32; e += NW * 64 * 4)
+        *reinterpret_cast<float4*>(&gs[e]) = *reinterpret_cast<const float4*>(norm.g + e);
+      __syncthreads();
+#pragma unroll
+      for (int c = 0; c < SETS; ++c) {
+        if (c + 1 < SETS) load_set(c + 1, (c + 1) & 1);
+#pragma unroll
+        for (int i = 0; i < XC; ++i) convert_step(c * XC + i, x[c & 1][i][0], x[c & 1][i][1]);
+        // the address of the sets further on hangs on this set's last operand: asked for all at
+        // once (which is what the compiler does with loads off one pointer) the row in 32 bits
+        // would not fit the registers
+        asm volatile("" : "+v"(xp), "+v"(afr[c * XC + XC - 1]));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      asm volatile("" : "+s"(Wp), "+v"(afr[NS - 1]));     // no weights before the activations are in place
+      if (item < n_items) first_loads(0);
     }
     ss += __shfl_xor(ss, 16);
     ss += __shfl_xor(ss, 32);
@@ -1026,7 +1071,7 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
     const bool has_next = it + 1 < n_items;
 #pragma unroll
     for (int j = 0; j < NT; ++j)
-      wrow[j] = W + (has_next ? (size_t)lane_wrow(c0 + CH, j) * ldw : (size_t)0) + k0;
+      wrow[j] = Wp + (has_next ? (size_t)lane_wrow(c0 + CH, j) * ldw : (size_t)0) + k0;
     floatx4 acc[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -1034,11 +1079,20 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
     for (int s = 0; s < NS; ++s) {
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afr[s], w[j][s], acc[j], 0, 0, 0);
-        w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32);
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afr[s], w[j][s % RING], acc[j], 0, 0, 0);
+        // the step RING further on: of this item, or of the next one.  (The load stays behind
+        // the MFMA: moved in front of it, it needs a register of its own.)
+        if constexpr (RING < NS) {
+          asm volatile("" : "+v"(acc[j]) : : "memory");
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        w[j][s % RING] = s + RING < NS ? *reinterpret_cast<const bf16x8*>(wcur[j] + (s + RING) * 32)
+                                       : *reinterpret_cast<const bf16x8*>(wrow[j] + (s + RING - NS) * 32);
         __builtin_amdgcn_sched_barrier(0);      // keep "use a register, then refill it" in this order
       }
     }
+#pragma unroll
+    for (int j = 0; j < NT; ++j) wcur[j] = wrow[j];
     // D[m][n]: n = lane % 16, m = 4 (lane / 16) + r
     const int buf = it & 1;
 #pragma unroll
@@ -1101,13 +1155,26 @@ int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const fl
   const int unit = (!PAIR && cols_total / 32 >= 8 * n_cu) ? 32 : 2;
   const int units = (cols_total + unit - 1) / unit;
   const int grid = units < n_cu ? units : n_cu;
-  if (norm)
-    stationary16_kernel<NS, NT, PAIR, true><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
-                                                                      cols_total, unit, epi, *norm);
-  else
-    stationary16_kernel<NS, NT, PAIR, false><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
-                                                                       cols_total, unit, epi,
-                                                                       NormArgs{nullptr, nullptr, 0.f});
+  // registers: 4 NS for the activations and 4 NT RING for the weights in flight, of 256.  A long
+  // K keeps 8 to 10 loads of 1 KB in flight per wave, far more than a CU has outstanding anyway.
+  constexpr int RING = NS <= 16 ? NS : (NS % 10 == 0 ? 10 : 8 / NT);
+  static_assert(NS % RING == 0 && 4 * NS + 4 * NT * RING <= 200, "activations and weight ring fit the registers");
+  if (norm) {
+    constexpr int smem = 8 * NS * 32 * (int)sizeof(float);       // the norm's weight
+    auto kern = stationary16_kernel<NS, RING, NT, PAIR, true>;
+    static bool configured = false;
+    if (!configured) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+      if (e != hipSuccess) return (int)e;
+      configured = true;
+    }
+    kern<<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, cols_total, unit, epi, *norm);
+  } else {
+    stationary16_kernel<NS, RING, NT, PAIR, false><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
+                                                                             cols_total, unit, epi,
+                                                                             NormArgs{nullptr, nullptr, 0.f});
+  }
   return mf_launch_status();
 }
 
@@ -1448,6 +1515,9 @@ static int stationary16(const void* a, int lda, const bf16* w, int ldw, const fl
   static const int off = getenv("MF_NO_STATIONARY") ? 1 : 0;
   if (off || M > 16 || K % 256 != 0 || (N + 15) / 16 < 128) return MF_NOT_BUILT;
   if (epi == EPI_SWIGLU && N % 64 != 0) return MF_NOT_BUILT;
+  // K of 5120 and 8192 without a norm to fold in (the o product): the rolling kernel measured the
+  // same at 5120 and faster at 8192 (26 us against 30 for 8192 x 8192)
+  if (K > 4096 && !norm && epi != EPI_SWIGLU) return MF_NOT_BUILT;
   // two tiles an item where a block's share is more than one: 128-byte rows of 32-bit output
   const int n_cu = cu_count();
   if (n_cu <= 0) return (int)hipErrorUnknown;
@@ -1459,7 +1529,7 @@ static int stationary16(const void* a, int lda, const bf16* w, int ldw, const fl
            : two ? launch_stationary16<NS_, 2, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, norm, stream) \
                  : launch_stationary16<NS_, 1, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, norm, stream);
   switch (K / 256) {
-    MF_STATIONARY(6) MF_STATIONARY(8) MF_STATIONARY(14) MF_STATIONARY(16)
+    MF_STATIONARY(6) MF_STATIONARY(8) MF_STATIONARY(14) MF_STATIONARY(16) MF_STATIONARY(20) MF_STATIONARY(32)
   }
 #undef MF_STATIONARY
   return MF_NOT_BUILT;

@@ -249,14 +249,25 @@ def cu_count() -> int:
     return _CU_COUNT
 
 
-def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None) -> Tuple[int, int]:
+STATIONARY_K = (1536, 2048, 3584, 4096, 5120, 8192)
+
+
+def stationary_shape(n: int, k: int, folded: bool = False) -> bool:
+    """True where the register-resident decode product is built for [n][k] weights (aligned
+    operands given): K one of a few multiples of 256 and at least 128 tiles of 16 weight rows;
+    a K above 4096 only with a norm or SwiGLU folded in (`folded`)."""
+    return k in STATIONARY_K and (n + 15) // 16 >= 128 and (k <= 4096 or folded)
+
+
+def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None,
+                swiglu: bool = False) -> Tuple[int, int]:
     """(splits, k_per_split) of the decode product.  One split: one kernel, K divided between the
     waves of a block.  More: blocks of 128 weight rows with the activations staged in LDS, K split
     so that there is about one block per CU (measured: with four times as many, the partial sums
     and the start of each block cost a fifth more), and a second kernel that adds the parts.
 
     At most 16 rows take the one-kernel form, except against a long K (which the register-resident
-    kernel does not hold) where it does badly: from 9 rows on (every block reads its own copy of
+    kernel does not hold: it takes 1536 to 8192) where it does badly: from 9 rows on (every block reads its own copy of
     the activations from L2: 42 us at 16 rows of 18944 against 33), and where a CU's share of the
     weight rows fills its 16-row tiles poorly (5120 rows over 256 CUs: 20 each, 87 us against 57)."""
     if target_blocks is None:
@@ -264,7 +275,7 @@ def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None) -> 
     if m <= 16:
         share = (n + target_blocks - 1) // target_blocks          # weight rows of a block in the one-kernel form
         fill = share / float((share + 15) // 16 * 16)
-        if k < 8192 or (m <= 8 and fill >= 0.8):
+        if k < 8192 or (m <= 8 and fill >= 0.8) or stationary_shape(n, k, swiglu):
             return 1, (k + 255) // 256 * 256
     n_blocks = (n + 127) // 128
     chunks = (k + 255) // 256
@@ -357,7 +368,7 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, vari
     if m == 0:
         return
     if m <= 64 and variant == 0:
-        splits, per = skinny_plan(m, n, k)
+        splits, per = skinny_plan(m, n, k, swiglu=True)
         part = workspace("skinny", splits * m * n, x.device) if m > 16 or splits > 1 else None
         _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
                                                         _ptr(part), m, n, k, splits, per, EPI_SWIGLU, _stream()),

@@ -44,7 +44,9 @@ def test_embed(ops, dtype, rows, d, vocab):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,d,eps", [(1, 64, 1e-6), (5, 200, 1e-5), (130, 3584, 1e-6), (3, 1000, 0.1)])
+@pytest.mark.parametrize("rows,d,eps", [(1, 64, 1e-6), (5, 200, 1e-5), (130, 3584, 1e-6), (3, 1000, 0.1),
+                                         (2, 5120, 1e-5), (3, 8192, 1e-5), (2, 12288, 1e-6), (2, 20000, 1e-6),
+                                         (2, 4099, 1e-6)])
 def test_rmsnorm(ops, out_dtype, rows, d, eps):
     x = rnd((rows, d), seed=2, scale=3.0)
     w = rnd((d,), seed=3) + 1.0
@@ -197,6 +199,8 @@ def test_gemm_f32(ops, m, n, k):
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(2048, 512, 256), (1, 152064, 64), (64, 3584, 3584),
                                                  # at most 16 rows with K of 1536..4096: activations in registers
                                                  (1, 2100, 1536), (5, 2050, 2048), (8, 4001, 3584), (16, 2048, 4096),
+                                                 # K of 5120 and 8192: the weights go through a shorter ring
+                                                 (5, 2100, 5120), (8, 4100, 5120), (3, 5000, 8192), (16, 8192, 8192),
                                                  # 17..64 rows, whole chunks of K: the ring kernel, with K split
                                                  (20, 200, 768), (50, 1000, 4096),
                                                  # 9..16 rows against a long K: the same kernel
@@ -494,6 +498,7 @@ def test_gemm_bf16_wide_few_rows(ops, m, n, k):
 @pytest.mark.parametrize("m,nf,k", [(1, 176, 64), (8, 344, 128), (16, 32, 200), (17, 176, 64), (64, 1000, 344),
                                     (65, 232, 200), (300, 18944, 256), (130, 31, 72),
                                     (8, 1100, 1536), (3, 2100, 3584), (16, 1030, 4096), (1, 1024, 2048),
+                                    (8, 1100, 5120), (3, 2100, 8192),
                                     # 17..64 rows against a wide matrix: one block per CU over the whole of K
                                     (64, 18944, 512), (33, 16400, 256), (40, 300, 512), (10, 96, 8192),
                                     # more than 64 rows but few tiles: K split over blocks
@@ -516,7 +521,9 @@ def test_gemm_bf16_swiglu(ops, variant, m, nf, k):
 
 
 @pytest.mark.parametrize("m,n,k,idx", [(1, 2100, 1536, False), (5, 4608, 2048, True), (8, 4001, 3584, False),
-                                       (16, 2048, 4096, True), (3, 152064, 3584, True)])
+                                       (16, 2048, 4096, True), (3, 152064, 3584, True),
+                                       (2, 2100, 5120, True), (9, 5000, 5120, False), (7, 5000, 8192, True),
+                                       (16, 2048, 8192, False)])
 def test_gemm_bf16_normed(ops, m, n, k, idx):
     """RMS norm folded into the few-row product: against the same formula in float64 with the
     kernel's one rounding (tight), and against norm-then-product as the two kernels do it."""
@@ -548,7 +555,8 @@ def test_gemm_bf16_normed(ops, m, n, k, idx):
     close(acc, ref - b.double() + base.double(), 2e-5 * math.sqrt(k), 1e-5)
 
 
-@pytest.mark.parametrize("m,nf,k", [(8, 1100, 1536), (3, 2100, 3584), (16, 1030, 4096), (1, 18944, 3584)])
+@pytest.mark.parametrize("m,nf,k", [(8, 1100, 1536), (3, 2100, 3584), (16, 1030, 4096), (1, 18944, 3584),
+                                    (4, 2100, 5120), (16, 1100, 8192), (1, 2500, 8192)])
 def test_gemm_bf16_normed_swiglu(ops, m, nf, k):
     h = rnd((m, k), seed=50, scale=2.0)
     g = 1.0 + rnd((k,), seed=51, scale=0.2)

@@ -7,7 +7,7 @@ from minfer_amd.kernels import ops
 
 def test_skinny_plan_covers_k_without_empty_splits():
     for m, n, k, target in itertools.product((1, 8, 9, 16, 17, 40, 64), (96, 3584, 4608, 37888, 152064),
-                                             (64, 200, 256, 3584, 18944), (64, 256, 1024)):
+                                             (64, 200, 256, 3584, 8192, 18944), (64, 256, 1024)):
         splits, per = ops.skinny_plan(m, n, k, target_blocks=target)
         assert splits >= 1 and per % 256 == 0
         assert splits * per >= k, (m, n, k, splits, per)
@@ -26,6 +26,10 @@ def test_skinny_plan_choices_at_the_model_shapes():
     assert ops.skinny_plan(1, 5120, 27648, target_blocks=256)[0] > 1
     assert ops.skinny_plan(9, 3584, 18944, target_blocks=256)[0] > 1
     assert ops.skinny_plan(16, 37888, 3584, target_blocks=256)[0] == 1
+    # K of 8192 is held in registers where SwiGLU (or a norm) is folded in: one kernel up to 16 rows
+    assert ops.skinny_plan(16, 59136, 8192, target_blocks=256, swiglu=True)[0] == 1
+    assert ops.skinny_plan(16, 8192, 8192, target_blocks=256)[0] > 1
+    assert ops.skinny_plan(12, 300, 8192, target_blocks=256, swiglu=True)[0] > 1      # too few weight rows for it
 
 
 def test_tile_split_plan():
