@@ -12,7 +12,7 @@ sequence reads positions below its own length only and writes each before readin
 
 Layers with the same needs (kv heads, head size, window) form a group with storage of its
 own: one K tensor `[entries][pages][kv_heads][64][head_dim]`, one V tensor (the same shape in
-32-bit, `[entries][pages][kv_heads][head_dim][64]` in bfloat16, see `v_page_shape`) and one
+32-bit, `[entries][pages][kv_heads][2][head_dim][32]` in bfloat16, see `v_page_shape`) and one
 page pool.
 A group with a window gives pages back as soon as every position in them has left the
 window of all later queries.
@@ -27,12 +27,16 @@ import torch
 PAGE = 64
 
 
-def v_page_shape(n_kv_heads: int, head_dim: int, dtype) -> Tuple[int, int, int]:
-    """One page of V: like K, `[kv_heads][64][head_dim]`, in 32-bit; transposed inside the page,
-    `[kv_heads][head_dim][64]`, in bfloat16, where the attention kernels feed V^T rows to the
-    matrix cores as they are stored."""
+V_HALF = PAGE // 2
+
+
+def v_page_shape(n_kv_heads: int, head_dim: int, dtype) -> Tuple[int, ...]:
+    """One page of V: like K, `[kv_heads][64][head_dim]`, in 32-bit.  In bfloat16 it is transposed
+    in two halves of 32 keys, `[kv_heads][2][head_dim][32]` (key j of the page is element j % 32
+    of half j / 32): the attention kernels feed V^T rows to the matrix cores as they are stored,
+    32 keys at a time, and what 16 lanes-rows of such a step read is one contiguous kilobyte."""
     if dtype == torch.bfloat16:
-        return (n_kv_heads, head_dim, PAGE)
+        return (n_kv_heads, 2, head_dim, V_HALF)
     return (n_kv_heads, PAGE, head_dim)
 
 

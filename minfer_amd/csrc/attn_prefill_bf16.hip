@@ -9,8 +9,9 @@
 // 32-bit, probabilities are rounded to bfloat16 for the second product.
 //
 // A block (4 waves) owns 128 consecutive query tokens of one sequence and one query head;
-// each wave 32 of them.  Per cache page (64 keys): K and V^T go to LDS as stored (the cache
-// keeps a page of V transposed, [head_dim][64 keys]), into one of two buffers.
+// each wave 32 of them.  Per cache page (64 keys): K goes to LDS as stored and V^T as rows of 64
+// keys (the cache keeps a page of V transposed in two halves, [2][head_dim][32 keys], which the
+// copy puts side by side), into one of two buffers.
 //   S^T[key][q] = K Q^T      32x32x16 MFMA, A = K rows from LDS, B = Q held in registers
 //   lane <-> query column, so the row statistics of the softmax are per-lane scalars
 //   O^T[d][q]  += V^T P^T    A = V^T from LDS, B = P^T, which is S^T's own register layout
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
   auto fetch = [&](int page_i) {
     const int page = pt[page_i];
     const bf16* kp = kc + ((size_t)page * nk + hk) * KT * HD;
-    const bf16* vp = vc + ((size_t)page * nk + hk) * HD * KT;     // a page of V is [HD][KT]
+    const bf16* vp = vc + ((size_t)page * nk + hk) * HD * KT;     // a page of V is [2][HD][KT / 2]
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
       const int c = i * 256 + tid;
@@ -103,11 +104,11 @@ __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
     const int n_written = blk_p_hi - page_i * KT + 1;    // keys of this page that exist
 #pragma unroll
     for (int i = 0; i < VCH; ++i) {
-      const int c = i * 256 + tid;                       // chunk: column c / 8, keys 8 (c % 8) ..
+      const int c = i * 256 + tid;         // chunk: half c / (4 HD), column (c / 4) % HD, 8 keys from 8 (c % 4)
       if (c < HD * (KT / 8)) {
         vreg[i] = *reinterpret_cast<const bf16x8*>(vp + (size_t)c * 8);
         if (n_written < KT) {
-          const int k0 = (c % (KT / 8)) * 8;
+          const int k0 = (c / (HD * 4)) * (KT / 2) + (c % 4) * 8;
 #pragma unroll
           for (int e = 0; e < 8; ++e)
             if (k0 + e >= n_written) vreg[i][e] = (bf16)0.f;
@@ -129,7 +130,7 @@ __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
     for (int i = 0; i < VCH; ++i) {
       const int c = i * 256 + tid;
       if (c < HD * (KT / 8)) {
-        bf16* dst = &Vt[(c / (KT / 8)) * VT_LD + (c % (KT / 8)) * 8];
+        bf16* dst = &Vt[((c / 4) % HD) * VT_LD + (c / (HD * 4)) * (KT / 2) + (c % 4) * 8];
         *reinterpret_cast<bf16x4*>(dst) = bf16x4{vreg[i][0], vreg[i][1], vreg[i][2], vreg[i][3]};
         *reinterpret_cast<bf16x4*>(dst + 4) = bf16x4{vreg[i][4], vreg[i][5], vreg[i][6], vreg[i][7]};
       }

@@ -201,8 +201,8 @@ MF_API int mf_rope_table(float* cs, float* sn, int n_pos, int half, double theta
 // token's position before attention reads it (src/graph/cpu_backend.rs:118-149).
 // qkv is [T][(nh + 2 nk) hd] in 32-bit with biases already added.  One block per
 // (token, head of q|k|v).
-// In bfloat16 a page of V is stored transposed, [hd][64 keys], the layout the attention
-// kernels read as a matrix-core operand; in 32-bit it lies like K, [64 keys][hd].
+// In bfloat16 a page of V is stored transposed in two halves, [2][hd][32 keys], the layout the
+// attention kernels read as a matrix-core operand; in 32-bit it lies like K, [64 keys][hd].
 template <typename OT, bool V_TRANSPOSED>
 __global__ __launch_bounds__(64) void rope_kvwrite_kernel(
     const float* __restrict__ qkv, const float* __restrict__ cs, const float* __restrict__ sn,
@@ -236,9 +236,11 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(
       dst[i] = from_f32<OT>(x0 * c - x1 * s);
       dst[i + half] = from_f32<OT>(x0 * s + x1 * c);
     }
-  } else if (V_TRANSPOSED) {      // a page of V is [hd][64 keys]
-    OT* dst = vcache + ((size_t)page * nk + hk) * hd * MF_PAGE + pos % MF_PAGE;
-    for (int i = threadIdx.x; i < hd; i += 64) dst[(size_t)i * MF_PAGE] = from_f32<OT>(src[i]);
+  } else if (V_TRANSPOSED) {      // a page of V is [2][hd][32 keys]
+    constexpr int VH = MF_PAGE / 2;
+    const int off = pos % MF_PAGE;
+    OT* dst = vcache + (((size_t)page * nk + hk) * 2 + off / VH) * hd * VH + off % VH;
+    for (int i = threadIdx.x; i < hd; i += 64) dst[(size_t)i * VH] = from_f32<OT>(src[i]);
   } else {
     OT* dst = vcache + (((size_t)page * nk + hk) * MF_PAGE + pos % MF_PAGE) * hd;
     for (int i = threadIdx.x; i < hd; i += 64) dst[i] = from_f32<OT>(src[i]);

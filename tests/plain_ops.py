@@ -80,7 +80,7 @@ def rope_kvwrite(qkv, cos, sin, positions, seq_of_tok, page_table, q_out, kcache
     assert (page >= 0).all(), "token written to a page that was not reserved"
     kcache[page, :, pos % PAGE, :] = k
     if v_transposed(vcache):
-        vcache[page, :, :, pos % PAGE] = v
+        vcache[page, :, (pos % PAGE) // 32, :, pos % 32] = v
     else:
         vcache[page, :, pos % PAGE, :] = v
 
@@ -131,14 +131,14 @@ def linear_normed_reference(x, norm_weight, eps, row_idx, weight, bias, swiglu=F
 
 
 def v_transposed(vcache):
-    """A bfloat16 cache keeps a page of V as [kv_heads][head_dim][64], a 32-bit one as
-    [kv_heads][64][head_dim] (the product's `v_page_shape`)."""
+    """A bfloat16 cache keeps a page of V as [kv_heads][2][head_dim][32] (key j is element j % 32
+    of half j / 32), a 32-bit one as [kv_heads][64][head_dim] (the product's `v_page_shape`)."""
     return vcache.dtype == torch.bfloat16
 
 
 def v_rows(vcache, page, off):
     """[n][kv_heads][head_dim] rows of V at (page[i], off[i])."""
-    return vcache[page, :, :, off] if v_transposed(vcache) else vcache[page, :, off, :]
+    return vcache[page, :, off // 32, :, off % 32] if v_transposed(vcache) else vcache[page, :, off, :]
 
 
 def gather_cache_rows(cache, page_table_row, length, is_v=False):

@@ -127,8 +127,11 @@ def make_cache(n_pages, nk, hd, dtype, seed=0):
 
 
 def stored_v(v):
-    """A bfloat16 cache keeps a page of V transposed, [kv_heads][head_dim][64]."""
-    return v.transpose(2, 3).contiguous() if v.dtype == torch.bfloat16 else v
+    """A bfloat16 cache keeps a page of V transposed in two halves, [kv_heads][2][head_dim][32]."""
+    if v.dtype != torch.bfloat16:
+        return v
+    pages, nk, _, hd = v.shape
+    return v.view(pages, nk, 2, 32, hd).transpose(3, 4).contiguous()
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -349,7 +352,7 @@ def test_attn_decode_rope(ops, nh, nk, hd, window, write_kv):
         close(torch.nan_to_num(vd.float(), nan=7e7), torch.nan_to_num(vr.float(), nan=7e7), 2e-2, 2e-2)
         for b, l in enumerate(lengths):
             page, off = int(table[b, (l - 1) // 64]), (l - 1) % 64
-            assert not torch.isnan(kd[page, :, off].float()).any() and not torch.isnan(vd[page, :, :, off].float()).any()
+            assert not torch.isnan(kd[page, :, off].float()).any() and not torch.isnan(vd[page, :, off // 32, :, off % 32].float()).any()
     else:
         assert same(kd.cpu(), kc) and same(vd.cpu(), vc)
 
@@ -457,7 +460,7 @@ def test_attn_prefill_far_key_and_window_edge(ops):
     qi, far = 650, 3
     page, row = int(table[0, far // 64]), far % 64
     kc[page, 0, row] = q[qi, :hd] * 4.0
-    vrow = vc[page, 0, :, row].float()             # a bfloat16 page of V is [kv_heads][head_dim][64]
+    vrow = vc[page, 0, row // 32, :, row % 32].float()      # a bfloat16 page of V is [kv_heads][2][head_dim][32]
     for window, seen in ((0, True), (qi - far + 1, True), (qi - far, False)):
         out = torch.empty(q.shape, dtype=torch.bfloat16, device=DEV)
         ops.attn_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), ctx_on(DEV), out, nh, nk, hd, 1.0, window)

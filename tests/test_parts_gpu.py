@@ -315,8 +315,8 @@ class ToyPositionBias(PositionEncoding):
         page = page_table.long()[ctx.seq_of_tok.long(), pos // 64]
         k, v = x[:, n_heads:n_heads + n_kv_heads], x[:, n_heads + n_kv_heads:]
         kcache[page, :, pos % 64, :] = k.to(kcache.dtype)
-        if vcache.shape[-1] == 64 and vcache.dtype == torch.bfloat16:      # a bfloat16 page of V is [hd][64]
-            vcache[page, :, :, pos % 64] = v.to(vcache.dtype)
+        if vcache.dtype == torch.bfloat16:      # a bfloat16 page of V is [2][hd][32] (cache.paged.v_page_shape)
+            vcache[page, :, (pos % 64) // 32, :, pos % 32] = v.to(vcache.dtype)
         else:
             vcache[page, :, pos % 64, :] = v.to(vcache.dtype)
 
