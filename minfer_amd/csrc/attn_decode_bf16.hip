@@ -16,46 +16,23 @@
 // The cache keeps V transposed inside a page in bfloat16, in two halves of 32 keys
 // ([2][head_dim][32 keys]), so V^T rows are contiguous over the keys of a step like K rows are
 // over head_dim, the 16 rows a load takes are one contiguous kilobyte (whole 128-byte lines: with
-// rows of 64 keys a step asked for half of each line, and the CU's limit is lines in flight),
-// and neither operand passes through LDS.  In both results a lane owns one head (lane % 16): the softmax statistics are
+// rows of 64 keys a step asked for half of each line, and what a CU can have in flight is counted
+// in lines: 64 sequences of up to 2,048 keys took 41 us that way and take 30 now), and neither
+// operand passes through LDS.  In both results a lane owns one head (lane % 16): the softmax statistics are
 // per-lane scalars, and the scores a lane holds (8 consecutive keys, by the choice of which
 // key each K row of a tile is) are exactly the 8 k-slots of its B operand in the second
 // product, so P never leaves its registers.
 //
 // A block is (token, kv head, chunk of 16 heads, key split); its 4 waves take the 32-key steps
-// of the split in turn and merge through LDS.  How many splits a token gets follows the lengths
-// of the step: all the tokens' keys together are dealt out in shares of the same size (about
-// one block per CU), a token of many keys gets many blocks and a short one a single block, so
-// that a batch of unequal lengths keeps every CU about equally long at work.  The grid holds
-// `s_max` splits per token; blocks beyond a token's own number leave at once.  A token with one
-// split writes its result, one with several writes unnormalised partials (acc, max, sum) and
-// decode_combine_kernel merges them in a fixed order.
+// of the split in turn and merge through LDS.  The split length follows the token's own
+// length, so every split has work.  With several splits each block writes an unnormalised
+// partial (acc, max, sum) and attn_combine_kernel merges them in a fixed order.
 #include "attn_tokens_impl.h"
 
 namespace {
 
 constexpr int STEP = 32;       // keys per wave step
 static_assert(STEP * 2 == MF_PAGE, "a step is one half of a page of V");
-
-// Splits of token t.  `target` is the number of blocks wanted per (kv head, head chunk) over all
-// tokens: a share is the step's keys / target, in whole rounds of a block (4 waves x 32 keys),
-// and a token gets as many splits as it has shares, at most s_max.  Every wave computes this
-// for itself from the positions (64 per pass); the result is the same in all lanes.
-__device__ __forceinline__ int token_splits(const int* __restrict__ positions, int n_tok, int t, int window,
-                                            int target, int s_max) {
-  if (s_max <= 1) return 1;
-  const int lane = threadIdx.x & 63;
-  long long total = 0;
-  for (int i = lane; i < n_tok; i += 64) {
-    const int len = positions[i] + 1;
-    total += window > 0 ? min(len, window) : len;
-  }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) total += __shfl_xor(total, o, MF_WAVE);
-  const long long share = max(4LL * STEP, ((total + target - 1) / target + 4 * STEP - 1) / (4 * STEP) * (4 * STEP));
-  const int mine = window > 0 ? min(positions[t] + 1, window) : positions[t] + 1;
-  return (int)max(1LL, min((long long)s_max, (mine + share - 1) / share));
-}
 
 // ROPE: the step's q|k|v come as the 32-bit output of their product, [(nh + 2 nk) hd] per token,
 // not yet rotated and not yet in the cache.  The kernel rotates q on the way into its operand
@@ -99,8 +76,8 @@ template <int HD, bool ROPE>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16* __restrict__ q, bf16* kc, bf16* vt,
     const int* __restrict__ page_table, int pt_stride, const int* __restrict__ positions,
-    const int* __restrict__ seq_of_tok, bf16* __restrict__ out, float* __restrict__ part, int n_tok, int nh,
-    int nk, float scale, int window, int s_max, int target, RopeArgs rope) {
+    const int* __restrict__ seq_of_tok, bf16* __restrict__ out, float* __restrict__ part, int nh, int nk,
+    float scale, int window, int n_splits, RopeArgs rope) {
   constexpr int KS = (HD + 31) / 32;      // 32-wide steps over head_dim in the first product
   constexpr int CT = HD / 16;             // 16-wide column tiles of the output
   constexpr int O_LD = HD + 4;
@@ -120,15 +97,22 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int r16 = lane & 15, q4 = lane >> 4;
 
   const int p = positions[t];
-  const int n_splits = token_splits(positions, n_tok, t, window, target, s_max);     // of this token
-  if (split >= n_splits) return;
   const int* pt = page_table + (size_t)seq_of_tok[t] * pt_stride;
   const int lo = window > 0 ? max(0, p - window + 1) : 0;
-  // split length: this token's keys over its splits, in whole block rounds of 4 steps
+  // split length: this token's keys over the splits, in whole block rounds of 4 steps
   const int per = (p + 1 - lo + n_splits - 1) / n_splits;
   const int split_len = (per + 4 * STEP - 1) / (4 * STEP) * (4 * STEP);
   const int j_begin = lo + split * split_len;
   const int j_end = min(p + 1, j_begin + split_len);
+  if (j_begin >= j_end) {
+    // A split past the token's keys (a short sequence under a split count made for long ones):
+    // its partials say "nothing here" (zeros, maximum -inf, sum 0) and the block is done.
+    for (int i = threadIdx.x; i < gcount * (HD + 2); i += 256) {
+      const int g = i / (HD + 2), d = i % (HD + 2);
+      part[(((size_t)t * nh + h0 + g) * n_splits + split) * (HD + 2) + d] = d == HD ? -INFINITY : 0.f;
+    }
+    return;
+  }
 
   // B operand of the first product: row = head r16, 8 elements of head_dim at 32 ks + 8 q4.
   // ROPE: the block rotates its 16 heads once, one 8-element chunk per thread, into LDS.
@@ -215,7 +199,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         kn[a][ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
         if (ks * 32 + q4 * 8 < HD) kn[a][ks] = *reinterpret_cast<const bf16x8*>(kp + (size_t)(4 * a) * HD + ks * 32);
       }
-    const bf16* vp = vt + ((size_t)page * nk + hk) * HD * MF_PAGE + ((size_t)(off / STEP) * HD + r16) * STEP + q4 * 8;
+    const bf16* vp = vt + ((((size_t)page * nk + hk) * 2 + off / STEP) * HD + r16) * STEP + q4 * 8;
 #pragma unroll
     for (int c = 0; c < CT; ++c) vn[c] = *reinterpret_cast<const bf16x8*>(vp + (size_t)(16 * c) * STEP);
   };
@@ -341,7 +325,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       o[d] = (bf16)(a * inv);
     }
   } else {
-    float* o = part + (((size_t)t * nh + h) * s_max + split) * (HD + 2);
+    float* o = part + (((size_t)t * nh + h) * n_splits + split) * (HD + 2);
     for (int d = sub; d < HD; d += 16) {
       float a = 0.f;
 #pragma unroll
@@ -352,52 +336,22 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
-// out[t][h][:] = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M) over the token's own splits
-// (at most 64).  One wave per (token, head): lane s weighs split s, then the lanes share the
-// head's elements.  A token with a single split has its result already.
-__global__ __launch_bounds__(64) void decode_combine_kernel(const float* __restrict__ part, bf16* __restrict__ out,
-                                                            const int* __restrict__ positions, int n_tok, int nh,
-                                                            int hd, int window, int s_max, int target) {
-  __shared__ float wgt[64];
-  const size_t th = blockIdx.x;   // t * nh + h
-  const int n_splits = token_splits(positions, n_tok, (int)(th / nh), window, target, s_max);
-  if (n_splits == 1) return;
-  const float* base = part + th * s_max * (hd + 2);
-  const int lane = threadIdx.x;
-  const float ms = lane < n_splits ? base[(size_t)lane * (hd + 2) + hd] : -INFINITY;
-  const float ls = lane < n_splits ? base[(size_t)lane * (hd + 2) + hd + 1] : 0.f;
-  const float mm = wave_max(ms);
-  wgt[lane] = (ms == -INFINITY) ? 0.f : __expf(ms - mm);
-  __syncthreads();
-  float L = 0.f;       // fixed order: one split after another
-  for (int sp = 0; sp < n_splits; ++sp) L += __shfl(ls, sp, MF_WAVE) * wgt[sp];
-  const float inv = L > 0.f ? 1.0f / L : 0.f;
-  for (int d = lane; d < hd; d += 64) {
-    float a = 0.f;
-#pragma unroll 8
-    for (int sp = 0; sp < n_splits; ++sp) a += base[(size_t)sp * (hd + 2) + d] * wgt[sp];
-    out[th * hd + d] = (bf16)(a * inv);
-  }
-}
-
 template <int HD>
 int launch(const bf16* q, bf16* kc, bf16* vt, const int* page_table, int pt_stride, const int* positions,
            const int* seq_of_tok, bf16* out, float* part, int n_tok, int nh, int nk, float scale, int window,
-           int s_max, int target, const RopeArgs* rope, hipStream_t stream) {
+           int n_splits, const RopeArgs* rope, hipStream_t stream) {
   const int G = nh / nk;
-  dim3 grid(n_tok, nk * ((G + 15) / 16), s_max);
+  dim3 grid(n_tok, nk * ((G + 15) / 16), n_splits);
   if (rope)
     attn_decode_kernel<HD, true><<<grid, 256, 0, stream>>>(q, kc, vt, page_table, pt_stride, positions, seq_of_tok,
-                                                           out, part, n_tok, nh, nk, scale, window, s_max, target,
-                                                           *rope);
+                                                           out, part, nh, nk, scale, window, n_splits, *rope);
   else
     attn_decode_kernel<HD, false><<<grid, 256, 0, stream>>>(q, kc, vt, page_table, pt_stride, positions,
-                                                            seq_of_tok, out, part, n_tok, nh, nk, scale, window,
-                                                            s_max, target, RopeArgs{nullptr, nullptr, nullptr, 0});
+                                                            seq_of_tok, out, part, nh, nk, scale, window, n_splits,
+                                                            RopeArgs{nullptr, nullptr, nullptr, 0});
   int rc = mf_launch_status();
-  if (rc == 0 && s_max > 1) {
-    decode_combine_kernel<<<n_tok * nh, 64, 0, stream>>>(part, out, positions, n_tok, nh, HD, window, s_max,
-                                                         target);
+  if (rc == 0 && n_splits > 1) {
+    attn_tokens::attn_combine_kernel<bf16><<<n_tok * nh, 64, 0, stream>>>(part, out, HD, n_splits);
     rc = mf_launch_status();
   }
   return rc;
@@ -405,16 +359,15 @@ int launch(const bf16* q, bf16* kc, bf16* vt, const int* page_table, int pt_stri
 
 int dispatch(const void* q, void* kc, void* vt, const int* page_table, int pt_stride, const int* positions,
              const int* seq_of_tok, void* out, float* part, int n_tok, int nh, int nk, int hd, float scale,
-             int window, int s_max, int target, const RopeArgs* rope, hipStream_t stream) {
+             int window, int n_splits, const RopeArgs* rope, hipStream_t stream) {
   if (n_tok <= 0) return 0;
-  if (hd % 16 != 0 || hd < 16 || hd > 256 || nk <= 0 || nh % nk != 0 || s_max < 1 || s_max > 64 || target < 1 ||
-      (s_max > 1 && part == nullptr))
+  if (hd % 16 != 0 || hd < 16 || hd > 256 || nk <= 0 || nh % nk != 0 || n_splits < 1 || n_splits > 64 ||
+      (n_splits > 1 && part == nullptr))
     return (int)hipErrorInvalidValue;
 #define MF_CASE(E)                                                                                          \
   case E:                                                                                                   \
     return launch<16 * E>((const bf16*)q, (bf16*)kc, (bf16*)vt, page_table, pt_stride, positions,           \
-                          seq_of_tok, (bf16*)out, part, n_tok, nh, nk, scale, window, s_max, target, rope,  \
-                          stream);
+                          seq_of_tok, (bf16*)out, part, n_tok, nh, nk, scale, window, n_splits, rope, stream);
   switch (hd / 16) {
     MF_CASE(1) MF_CASE(2) MF_CASE(3) MF_CASE(4) MF_CASE(5) MF_CASE(6) MF_CASE(7) MF_CASE(8)
     MF_CASE(9) MF_CASE(10) MF_CASE(11) MF_CASE(12) MF_CASE(13) MF_CASE(14) MF_CASE(15) MF_CASE(16)
@@ -426,14 +379,13 @@ int dispatch(const void* q, void* kc, void* vt, const int* page_table, int pt_st
 }  // namespace
 
 // q, out: [n_tok][nh][hd]; kc: [pages][nk][64][hd]; vt: [pages][nk][2][hd][32] (V transposed inside
-// a page, in two halves of 32 keys); part: n_tok * nh * s_max * (hd + 2) floats when s_max > 1 (at most 64 splits a token);
-// target: blocks wanted per (kv head, chunk of 16 heads) over all tokens.
+// a page, in two halves of 32 keys); part: n_tok * nh * n_splits * (hd + 2) floats when n_splits > 1 (at most 64 splits).
 MF_API int mf_attn_decode_bf16(const void* q, const void* kc, const void* vt, const int* page_table,
                                int pt_stride, const int* positions, const int* seq_of_tok, void* out,
                                float* part, int n_tok, int nh, int nk, int hd, float scale, int window,
-                               int s_max, int target, hipStream_t stream) {
+                               int n_splits, hipStream_t stream) {
   return dispatch(q, const_cast<void*>(kc), const_cast<void*>(vt), page_table, pt_stride, positions, seq_of_tok,
-                  out, part, n_tok, nh, nk, hd, scale, window, s_max, target, nullptr, stream);
+                  out, part, n_tok, nh, nk, hd, scale, window, n_splits, nullptr, stream);
 }
 
 // The same with the rotation and the cache write of the step's own q|k|v folded in: qkv is the
@@ -444,9 +396,9 @@ MF_API int mf_attn_decode_bf16(const void* q, const void* kc, const void* vt, co
 MF_API int mf_attn_decode_rope_bf16(const float* qkv, const float* cs, const float* sn, void* kc, void* vt,
                                     const int* page_table, int pt_stride, const int* positions,
                                     const int* seq_of_tok, void* out, float* part, int n_tok, int nh, int nk,
-                                    int hd, float scale, int window, int s_max, int target, int write_kv,
+                                    int hd, float scale, int window, int n_splits, int write_kv,
                                     hipStream_t stream) {
   const RopeArgs rope{qkv, cs, sn, write_kv};
   return dispatch(nullptr, kc, vt, page_table, pt_stride, positions, seq_of_tok, out, part, n_tok, nh, nk, hd,
-                  scale, window, s_max, target, &rope, stream);
+                  scale, window, n_splits, &rope, stream);
 }

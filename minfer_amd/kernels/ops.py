@@ -56,9 +56,9 @@ _PROTOTYPES = {
     },
     "attn_decode_bf16": {
         "mf_attn_decode_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
-                                c_float, c_int, c_int, c_int, _P],
+                                c_float, c_int, c_int, _P],
         "mf_attn_decode_rope_bf16": [_P, _P, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int,
-                                     c_int, c_float, c_int, c_int, c_int, c_int, _P],
+                                     c_int, c_float, c_int, c_int, c_int, _P],
     },
     "attn_prefill_bf16": {
         "mf_attn_prefill_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int,
@@ -460,25 +460,20 @@ def _need_caches(what: str, kcache: torch.Tensor, vcache: torch.Tensor, dtype, n
                           f"{[kcache.shape[0]] + list(want)}")
 
 
-def decode_split_plan(n_tok: int, n_kv_heads: int, group: int, max_len: int,
-                      target_blocks: Optional[int] = None) -> Tuple[int, int]:
-    """(s_max, target) of the bfloat16 decode attention.  `target` is the number of blocks wanted
-    per (kv head, chunk of 16 heads) over all tokens, about one block per CU in all (measured
-    best at 1, 8 and 64 sequences of 4 kv heads); the kernel deals the step's keys out in equal
-    shares, so a token gets splits in proportion to its own length.  `s_max` bounds the splits
-    of one token (the grid and the partial sums are sized by it): four times a token's even
-    share, so that a sequence four times the mean length is still spread out, no more than one
-    per 128 keys of the longest possible sequence, and at most 64."""
-    chunks = n_kv_heads * ((group + 15) // 16)
-    if target_blocks is None:
-        target_blocks = cu_count()
-    target = max(1, target_blocks // chunks)
-    if os.environ.get("MF_ATTN_TARGET"):
-        target = int(os.environ["MF_ATTN_TARGET"])
+def decode_split_plan(n_tok: int, n_kv_heads: int, group: int, max_len: int, target_blocks: int = 256) -> int:
+    """Key splits of the bfloat16 decode attention: about one block per CU (measured best at
+    1, 8 and 64 sequences of 4 kv heads), at least 256 keys of the longest possible sequence
+    per split, at most 32 (one sequence of 30,000 keys: 22 us with 32 splits, 29 with 16; of
+    2,048 keys: 12.0 against 9.6, the merge reads every split).  The kernel divides each token's
+    own length by this number in rounds of 128 keys; a split left without keys writes an empty
+    partial and ends.  (Dealing the splits out by the tokens' lengths instead, a long
+    sequence many blocks and a short one a single block, measured no faster at 8 and 64
+    sequences of unequal lengths up to 2,048 and up to 30,000 keys, and slower where it made
+    more blocks: the blocks of short sequences end early and leave the memory to the others.)"""
+    blocks = n_tok * n_kv_heads * ((group + 15) // 16)
     if os.environ.get("MF_ATTN_SPLITS"):
-        return int(os.environ["MF_ATTN_SPLITS"]), target
-    s_max = max(1, min((4 * target + n_tok - 1) // n_tok, (max_len + 127) // 128, 64))
-    return s_max, target
+        return int(os.environ["MF_ATTN_SPLITS"])
+    return max(1, min(target_blocks // max(1, blocks), (max_len + 255) // 256, 32))
 
 
 def attn_tokens(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
@@ -501,12 +496,12 @@ def attn_tokens(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
     if max_len > page_table.shape[1] * PAGE:
         raise KernelError(f"attention: max_len {max_len} exceeds the page table ({page_table.shape[1]} pages)")
     if q.dtype == torch.bfloat16:
-        s_max, target = decode_split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, max_len)
-        part = workspace("attn", n_tok * n_heads * s_max * (head_dim + 2), q.device) if s_max > 1 else None
+        n_splits = decode_split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, max_len)
+        part = workspace("attn", n_tok * n_heads * n_splits * (head_dim + 2), q.device) if n_splits > 1 else None
         _check(_fn("attn_decode_bf16", "mf_attn_decode_bf16")(
             _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions),
             _ptr(seq_of_tok), _ptr(out), _ptr(part), n_tok, n_heads, n_kv_heads, head_dim, float(scale),
-            int(window or 0), s_max, target, _stream()), "attn_decode_bf16")
+            int(window or 0), n_splits, _stream()), "attn_decode_bf16")
         return
     n_splits, split_len = split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, head_dim, max_len)
     part = workspace("attn", n_tok * n_heads * n_splits * (head_dim + 2), q.device) if n_splits > 1 else None
@@ -541,12 +536,12 @@ def attn_decode_rope(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, kc
     if max_len > page_table.shape[1] * PAGE or max_len > cos.shape[0]:
         raise KernelError(f"attention: max_len {max_len} exceeds the page table ({page_table.shape[1]} pages) "
                           f"or the rotation table ({cos.shape[0]} positions)")
-    s_max, target = decode_split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, max_len)
-    part = workspace("attn", n_tok * n_heads * s_max * (head_dim + 2), qkv.device) if s_max > 1 else None
+    n_splits = decode_split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, max_len)
+    part = workspace("attn", n_tok * n_heads * n_splits * (head_dim + 2), qkv.device) if n_splits > 1 else None
     _check(_fn("attn_decode_bf16", "mf_attn_decode_rope_bf16")(
         _ptr(qkv), _ptr(cos), _ptr(sin), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1],
         _ptr(positions), _ptr(seq_of_tok), _ptr(out), _ptr(part), n_tok, n_heads, n_kv_heads, head_dim,
-        float(scale), int(window or 0), s_max, target, 1 if write_kv else 0, _stream()), "attn_decode_rope_bf16")
+        float(scale), int(window or 0), n_splits, 1 if write_kv else 0, _stream()), "attn_decode_rope_bf16")
 
 
 def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
