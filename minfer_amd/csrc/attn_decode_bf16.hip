@@ -186,7 +186,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int n_steps = j_begin < j_end ? (j_end - 1) / STEP - step0 + 1 : 0;
   bf16x8 kn[2][KS], vn[CT];
   // The page of a step is looked up a whole step before its keys are asked for, so that the
-  // look-up's latency does not stand in front of every step's loads.
+  // look-up's latency does not stand in front of every step's loads.  (Two steps in flight per
+  // wave instead of one measured the same, 30 us for 64 sequences of up to 2,048 keys and 4.7
+  // TB/s at 30,000, at twice the registers: the waves are not what the memory waits for.)
   auto page_of = [&](int i) { return pt[(step0 + i) * STEP / MF_PAGE]; };
   auto issue = [&](int i, int page) {
     const int jb = (step0 + i) * STEP;
