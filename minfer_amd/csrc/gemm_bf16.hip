@@ -1515,9 +1515,10 @@ static int stationary16(const void* a, int lda, const bf16* w, int ldw, const fl
   static const int off = getenv("MF_NO_STATIONARY") ? 1 : 0;
   if (off || M > 16 || K % 256 != 0 || (N + 15) / 16 < 128) return MF_NOT_BUILT;
   if (epi == EPI_SWIGLU && N % 64 != 0) return MF_NOT_BUILT;
-  // K of 5120 and 8192 without a norm to fold in (the o product): the rolling kernel measured the
-  // same at 5120 and faster at 8192 (26 us against 30 for 8192 x 8192)
-  if (K > 4096 && !norm && epi != EPI_SWIGLU) return MF_NOT_BUILT;
+  // K of 8192 without a norm to fold in (the o product): the rolling kernel measured faster
+  // (26 us against 30 for 8192 x 8192 with one row); at 5120 x 5120 it is the other way round from
+  // 8 rows on (19 us against 15.5)
+  if (K > 5120 && !norm && epi != EPI_SWIGLU) return MF_NOT_BUILT;
   // two tiles an item where a block's share is more than one: 128-byte rows of 32-bit output
   const int n_cu = cu_count();
   if (n_cu <= 0) return (int)hipErrorUnknown;

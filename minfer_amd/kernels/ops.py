@@ -255,8 +255,8 @@ STATIONARY_K = (1536, 2048, 3584, 4096, 5120, 8192)
 def stationary_shape(n: int, k: int, folded: bool = False) -> bool:
     """True where the register-resident decode product is built for [n][k] weights (aligned
     operands given): K one of a few multiples of 256 and at least 128 tiles of 16 weight rows;
-    a K above 4096 only with a norm or SwiGLU folded in (`folded`)."""
-    return k in STATIONARY_K and (n + 15) // 16 >= 128 and (k <= 4096 or folded)
+    a K above 5120 only with a norm or SwiGLU folded in (`folded`)."""
+    return k in STATIONARY_K and (n + 15) // 16 >= 128 and (k <= 5120 or folded)
 
 
 def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None,
