@@ -279,9 +279,18 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
                                                        const bf16* __restrict__ W, int ldw,
                                                        const float* __restrict__ bias, void* __restrict__ C,
                                                        int ldc, int M, int N, int K, int epi, int tiles_m,
-                                                       int xcd_remap) {
+                                                       int xcd_remap, int k_per_split) {
   constexpr int TM = 4, TN = 2;
   constexpr int ROW = DMA_BK * 2;              // bytes of a row in LDS
+  if (k_per_split > 0) {
+    // K split over blockIdx.y (k_per_split a multiple of 64): this block multiplies its part of K
+    // and stores 32-bit sums into its own [M][N] slab of C; another kernel adds the slabs
+    const int kb = blockIdx.y * k_per_split;
+    A += kb;
+    W += kb;
+    K = min(k_per_split, K - kb);
+    C = (float*)C + (size_t)blockIdx.y * M * N;
+  }
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   int tile = blockIdx.x;
   if (xcd_remap) {
@@ -399,7 +408,7 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
 }
 
 int launch_tile_dma(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc, int M,
-                    int N, int K, int epi, hipStream_t stream) {
+                    int N, int K, int epi, hipStream_t stream, int splits = 1, int k_per_split = 0) {
   constexpr int smem = DMA_STAGES * DMA_STAGE_BYTES;
   static bool configured = false;
   if (!configured) {
@@ -410,8 +419,8 @@ int launch_tile_dma(const bf16* A, int lda, const bf16* W, int ldw, const float*
   }
   const int tiles_m = (M + DMA_BM - 1) / DMA_BM, tiles_n = (N + DMA_BN - 1) / DMA_BN;
   static const int remap = getenv("MF_NO_XCD_REMAP") ? 0 : 1;
-  tile_dma_kernel<<<tiles_m * tiles_n, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, tiles_m,
-                                                            remap && tiles_m * tiles_n >= 16);
+  tile_dma_kernel<<<dim3(tiles_m * tiles_n, splits), 512, smem, stream>>>(
+      A, lda, W, ldw, bias, C, ldc, M, N, K, epi, tiles_m, remap && tiles_m * tiles_n >= 16, k_per_split);
   return mf_launch_status();
 }
 
@@ -1491,7 +1500,7 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
 // k_per_split is a multiple of 64.
 MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
                                int ldc, float* part, int M, int N, int K, int splits, int k_per_split,
-                               int epi, hipStream_t stream) {
+                               int epi, int big_tiles, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > 3 || splits < 2 || !part || k_per_split % 64 != 0 ||
       (long)splits * k_per_split < K || (long)(splits - 1) * k_per_split >= K)
@@ -1500,8 +1509,13 @@ MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, c
     return (int)hipErrorInvalidValue;
   const int vec_ok = (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) &&
                      ((uintptr_t)W % 16 == 0) && (K % 8 == 0);
-  int rc = launch_tile<128, 128, 64, 64>((const bf16*)A, lda, (const bf16*)W, ldw, nullptr, part, N, M, N, K,
-                                         EPI_F32, vec_ok, stream, splits, k_per_split);
+  // big_tiles: 256 x 256 tiles through the direct-to-LDS pipeline (many rows against few weight
+  // rows and a long K: the down product of a prompt); else 128 x 128 (few rows)
+  if (big_tiles && (!vec_ok || K % DMA_BK != 0)) return (int)hipErrorInvalidValue;
+  int rc = big_tiles ? launch_tile_dma((const bf16*)A, lda, (const bf16*)W, ldw, nullptr, part, N, M, N, K,
+                                       EPI_F32, stream, splits, k_per_split)
+                     : launch_tile<128, 128, 64, 64>((const bf16*)A, lda, (const bf16*)W, ldw, nullptr, part, N, M,
+                                                     N, K, EPI_F32, vec_ok, stream, splits, k_per_split);
   if (rc) return rc;
   dim3 g2(((epi == EPI_SWIGLU ? ldc : N) + 255) / 256, M);
   skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, splits, epi);

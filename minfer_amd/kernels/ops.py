@@ -44,7 +44,8 @@ _PROTOTYPES = {
     },
     "gemm_bf16": {
         "mf_gemm_bf16": [_P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
-        "mf_gemm_bf16_splitk": [_P, c_int, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+        "mf_gemm_bf16_splitk": [_P, c_int, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_int,
+                                c_int, _P],
         "mf_gemm_bf16_skinny": [_P, c_int, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int,
                                 c_int, c_int, _P],
         "mf_gemm_bf16_normed": [_P, c_int, _P, _P, c_float, _P, c_int, _P, _P, c_int, c_int, c_int, c_int,
@@ -284,19 +285,41 @@ def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None,
     return (chunks + per - 1) // per, per * 256
 
 
-def tile_split_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None) -> Tuple[int, int]:
-    """(splits, k_per_split) of the tile product; (1, k) where its 128 x 128 tiles alone fill the
-    chip.  A prompt of a few hundred tokens against a few thousand weight rows makes some 50 tiles
-    for 256 CUs and is bound by the weight stream: K is split so that there are about two blocks
-    per CU, each with at least 512 of K, and a second kernel adds the parts."""
+def tile_split_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None) -> Tuple[int, int, bool]:
+    """(splits, k_per_split, big) of the tile product; (1, k, False) where its tiles alone fill the
+    chip.  Two cases split K over blocks, with a second kernel that adds the parts:
+
+    * many rows whose 256 x 256 tiles leave CUs idle or a last round nearly empty (the down product
+      of a prompt: 2,048 x 3584 is 112 such tiles for 256 CUs, or 448 of 128 x 128 at a lower rate):
+      the big tiles (`big`) with K cut in s parts, s chosen by the rounds it takes (a round of big
+      tiles costs 28.5 ns per unit of K, one of 128 x 128 tiles 18.2 ns, measured at K 18944; the
+      parts are added at about 3.5 TB/s), each part at least 2,048 of K;
+    * a prompt of a few hundred tokens against a few thousand weight rows (some 50 tiles of
+      128 x 128, bound by the weight stream): those tiles with about two blocks per CU, each with
+      at least 512 of K."""
     cu = target_blocks if target_blocks is not None else cu_count()
-    tiles = ((m + 127) // 128) * ((n + 127) // 128)
     chunks = (k + 255) // 256
+
+    def cut(splits):
+        per = (chunks + splits - 1) // splits
+        return (chunks + per - 1) // per, per * 256
+
+    t256 = ((m + 255) // 256) * ((n + 255) // 256)
+    tiles = ((m + 127) // 128) * ((n + 127) // 128)
+    if m >= 768 and k % 64 == 0 and not os.environ.get("MF_NO_BIG_SPLIT"):
+        rounds = lambda blocks, slots: (blocks + slots - 1) // slots
+        whole = min(rounds(t256, cu) * 28.5e-9 * k, rounds(tiles, 2 * cu) * 18.2e-9 * k)
+        best, best_s = whole, 1
+        for parts in range(2, min(8, k // 2048) + 1):
+            t = rounds(t256 * parts, cu) * 28.5e-9 * k / parts + (parts + 2) * m * n * 4 / 3.5e12
+            if t < 0.92 * best:
+                best, best_s = t, parts
+        if best_s > 1:
+            return cut(best_s) + (True,)
     splits = min(chunks // 2, (2 * cu) // max(1, tiles))
     if tiles >= cu or splits < 2:
-        return 1, k
-    per = (chunks + splits - 1) // splits
-    return (chunks + per - 1) // per, per * 256
+        return 1, k, False
+    return cut(splits) + (False,)
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -331,12 +354,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
                                                         epi, _stream()), "gemm_bf16_skinny")
         return
     if variant == 0:
-        splits, per = tile_split_plan(m, n, k)
+        splits, per, big = tile_split_plan(m, n, k)
+        if big and (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8):
+            splits = 1                           # the big tiles take aligned operands only
         if splits > 1:
             part = workspace("skinny", splits * m * n, x.device)
             _check(_fn("gemm_bf16", "mf_gemm_bf16_splitk")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n,
-                                                            _ptr(part), m, n, k, splits, per, epi, _stream()),
-                   "gemm_bf16_splitk")
+                                                            _ptr(part), m, n, k, splits, per, epi, 1 if big else 0,
+                                                            _stream()), "gemm_bf16_splitk")
             return
     _check(_fn("gemm_bf16", "mf_gemm_bf16")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n, m,
                                              n, k, epi, variant, _stream()), "gemm_bf16")
@@ -375,11 +400,11 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, vari
                "gemm_bf16_skinny(swiglu)")
         return
     if variant == 0:
-        splits, per = tile_split_plan(m, n, k)
-        if splits > 1:
+        splits, per, big = tile_split_plan(m, n, k)
+        if splits > 1 and not big:
             part = workspace("skinny", splits * m * n, x.device)
             _check(_fn("gemm_bf16", "mf_gemm_bf16_splitk")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
-                                                            _ptr(part), m, n, k, splits, per, EPI_SWIGLU,
+                                                            _ptr(part), m, n, k, splits, per, EPI_SWIGLU, 0,
                                                             _stream()), "gemm_bf16_splitk(swiglu)")
             return
     _check(_fn("gemm_bf16", "mf_gemm_bf16")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf, m, n, k,

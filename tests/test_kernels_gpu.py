@@ -209,7 +209,9 @@ def test_gemm_f32(ops, m, n, k):
                                                  # 9..16 rows against a long K: the same kernel
                                                  (12, 300, 8192), (16, 3584, 18944), (4, 5120, 8192),
                                                  # more than 64 rows but few tiles: K split over blocks
-                                                 (200, 3584, 18944), (65, 1000, 1100), (512, 777, 2048)])
+                                                 (200, 3584, 18944), (65, 1000, 1100), (512, 777, 2048),
+                                                 # many rows, few big tiles, a long K: K split over 256 x 256 tiles
+                                                 (800, 300, 4096), (1030, 777, 6144)])
 def test_gemm_bf16(ops, variant, m, n, k):
     if variant and (m * n * k > 3e9):
         pytest.skip("large shape is covered by the default variant")

@@ -33,17 +33,25 @@ def test_skinny_plan_choices_at_the_model_shapes():
 
 
 def test_tile_split_plan():
-    for m, n, k in itertools.product((65, 128, 200, 1024, 2048, 8192), (96, 3584, 4608, 37888), (64, 256, 3584, 18944)):
-        splits, per = ops.tile_split_plan(m, n, k, target_blocks=256)
+    for m, n, k in itertools.product((65, 128, 200, 512, 1024, 2048, 8192), (96, 3584, 4608, 37888),
+                                     (64, 256, 3584, 18944)):
+        splits, per, big = ops.tile_split_plan(m, n, k, target_blocks=256)
         if splits == 1:
-            assert per == k
+            assert per == k and not big
             continue
         assert per % 256 == 0 and per >= 512
         assert splits * per >= k and (splits - 1) * per < k
-        tiles = ((m + 127) // 128) * ((n + 127) // 128)
-        assert tiles < 256 and splits * tiles <= 512
-    assert ops.tile_split_plan(2048, 3584, 18944, target_blocks=256) == (1, 18944)       # 448 tiles: enough
-    assert ops.tile_split_plan(200, 3584, 18944, target_blocks=256)[0] == 9
+        if big:
+            t256 = ((m + 255) // 256) * ((n + 255) // 256)
+            assert m >= 768 and k % 64 == 0 and per >= 2048 and splits <= 8
+        else:
+            tiles = ((m + 127) // 128) * ((n + 127) // 128)
+            assert tiles < 256 and splits * tiles <= 512
+    assert ops.tile_split_plan(2048, 3584, 18944, target_blocks=256) == (2, 9472, True)   # 112 big tiles, twice
+    assert ops.tile_split_plan(2048, 3584, 3584, target_blocks=256) == (1, 3584, False)   # K too short to split
+    assert ops.tile_split_plan(2048, 37888, 3584, target_blocks=256) == (1, 3584, False)
+    assert ops.tile_split_plan(200, 3584, 18944, target_blocks=256)[0::2] == (9, False)
+    assert ops.tile_split_plan(2048, 5120, 27648, target_blocks=256)[0::2] == (3, True)   # 160 big tiles: 480 blocks, two rounds
 
 
 def test_split_plan_of_the_32_bit_attention():
