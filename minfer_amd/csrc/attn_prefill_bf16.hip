@@ -33,7 +33,8 @@ __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ page_table, int pt_stride, const int* __restrict__ cu_seqlens,
     const int* __restrict__ start_pos, const int* __restrict__ tile_seq,
-    const int* __restrict__ tile_q0, bf16* __restrict__ out, int nh, int nk, float scale, int window) {
+    const int* __restrict__ tile_q0, bf16* __restrict__ out, int n_tiles, int nh, int nk, float scale, int window,
+    int pair_slots) {
   constexpr int HD = NKS * 16;
   constexpr int NDT = (NKS + 1) / 2;          // 32-wide output tiles over head_dim
   constexpr int HDP = NDT * 32;
@@ -43,8 +44,18 @@ __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
   bf16* const kv = reinterpret_cast<bf16*>(smem);        // two such buffers
   bf16* Os = reinterpret_cast<bf16*>(smem);              // [4][32][K_LD], after the last step
 
-  const int b = tile_seq[blockIdx.x], q0 = tile_q0[blockIdx.x];
-  const int h = blockIdx.y, hk = h / (nh / nk);
+  // Work items are (tile, head) with the tiles longest first (the host sorts them), one block
+  // each, in this order: the longest start first and the short ones fill in behind them.  Where
+  // all items are on the chip at once, two to a CU (a prompt of 2,048 tokens and 28 heads: 448),
+  // nothing fills in, and what counts is which two share a CU: blocks i and i + CUs do, so the
+  // second lot runs shortest first and every CU gets about the same number of pages (the
+  // longest and the shortest tile together: 34 pages where two of the longest were 64).
+  const int n_items = n_tiles * nh;
+  int item = blockIdx.x;
+  if (pair_slots > 0 && n_items <= 2 * pair_slots && item >= pair_slots) item = n_items - 1 - (item - pair_slots);
+  const int tile = item / nh;
+  const int b = tile_seq[tile], q0 = tile_q0[tile];
+  const int h = item % nh, hk = h / (nh / nk);
   const int tok0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - tok0, start = start_pos[b];
   const int* pt = page_table + (size_t)b * pt_stride;
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
@@ -262,6 +273,14 @@ int launch(const bf16* q, const bf16* kc, const bf16* vc, const int* page_table,
            const int* cu_seqlens, const int* start_pos, const int* tile_seq, const int* tile_q0, bf16* out,
            int n_tiles, int nh, int nk, float scale, int window, hipStream_t stream) {
   constexpr int HD = NKS * 16, HDP = ((NKS + 1) / 2) * 32, K_LD = HD + 8;
+  static int n_cu = 0;                 // compute units of the device (asked once)
+  if (n_cu == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return (int)hipErrorUnknown;
+    n_cu = prop.multiProcessorCount;
+  }
+  const int pair_slots = NKS <= 8 ? n_cu : 0;      // where two blocks share a CU (head sizes up to 128)
   constexpr int kv_bytes = 2 * (KT * K_LD + HDP * VT_LD) * 2;      // two buffers
   constexpr int o_bytes = 4 * 32 * K_LD * 2;
   constexpr int smem = kv_bytes > o_bytes ? kv_bytes : o_bytes;
@@ -273,8 +292,8 @@ int launch(const bf16* q, const bf16* kc, const bf16* vc, const int* page_table,
     if (e != hipSuccess) return (int)e;
     configured = true;
   }
-  kern<<<dim3(n_tiles, nh), 256, smem, stream>>>(q, kc, vc, page_table, pt_stride, cu_seqlens, start_pos,
-                                                 tile_seq, tile_q0, out, nh, nk, scale, window);
+  kern<<<n_tiles * nh, 256, smem, stream>>>(q, kc, vc, page_table, pt_stride, cu_seqlens, start_pos, tile_seq,
+                                            tile_q0, out, n_tiles, nh, nk, scale, window, pair_slots);
   return mf_launch_status();
 }
 
