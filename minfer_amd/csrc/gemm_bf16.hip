@@ -266,7 +266,11 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const 
 // Measured on the 2048 x 37888 x 3584 product (0.95 PFLOP/s): without the copies 1.1, without
 // copies and fragment reads 1.3 (the matrix cores alone, with the epilogue's 310 MB of output),
 // at a clock of 2.0 GHz under this load; asking for a tile in four parts spread over a tile's
-// products, or leaving the barrier out, changed nothing.
+// products, or leaving the barrier out, changed nothing, and neither did three stages for the W
+// tiles (which come from HBM) beside two for the A tiles, five times 32 KB, so that a W tile has
+// two tile times to arrive: it is not the copies' latency that the matrix cores wait for.
+// Counters on that product: the matrix cores busy 53% of the cycles at 1.93 GHz, LDS 16%, no bank
+// conflicts, waves 1.6% of their time waiting for LDS.
 constexpr int DMA_BM = 256, DMA_BN = 256, DMA_BK = 64, DMA_STAGES = 2;
 constexpr int DMA_STAGE_BYTES = (DMA_BM + DMA_BN) * DMA_BK * 2;
 
