@@ -274,8 +274,10 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const 
 constexpr int DMA_BM = 256, DMA_BN = 256, DMA_BK = 64, DMA_STAGES = 2;
 constexpr int DMA_STAGE_BYTES = (DMA_BM + DMA_BN) * DMA_BK * 2;
 
-__device__ __forceinline__ void dma16(const bf16* g, unsigned lds_byte) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte)
+// 16 bytes per lane from base + off (a wave-uniform base and a 32-bit byte offset per lane: one
+// register where a 64-bit address takes two, and no address arithmetic per copy)
+__device__ __forceinline__ void dma16(const bf16* base, unsigned off, unsigned lds_byte) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds_byte)
                : "memory", "m0");
 }
 
@@ -321,23 +323,24 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
   // and 24 + wid (8 rows each) of the A tile and of the W tile; the lane fetches row
   // 8 b + lane / 8, the chunk that belongs at position lane % 8
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
-  const bf16* ga[4];
-  const bf16* gw[4];
+  unsigned ga[4], gw[4];                       // byte offsets from A and W (the host checks that they fit)
 #pragma unroll
   for (int jj = 0; jj < 4; ++jj) {
     const int r = 8 * (jj * 8 + wid) + (lane >> 3);
     const int chunk = (lane & 7) ^ ((r >> 1) & 7);
-    ga[jj] = A + (size_t)min(m0 + r, M - 1) * lda + chunk * 8;
-    gw[jj] = W + (size_t)min(n0 + r, N - 1) * ldw + chunk * 8;
+    ga[jj] = ((unsigned)min(m0 + r, M - 1) * (unsigned)lda + chunk * 8) * 2u;
+    gw[jj] = ((unsigned)min(n0 + r, N - 1) * (unsigned)ldw + chunk * 8) * 2u;
   }
-  auto issue = [&](int kt) {
+  // copy q of a wave's eight for tile kt: four blocks of the A tile, then four of the W tile
+  auto issue_one = [&](int kt, int q) {
     const unsigned st = lds0 + (unsigned)(kt % DMA_STAGES) * DMA_STAGE_BYTES + wid * 1024;
     const int k = kt * DMA_BK;
+    if (q < 4) dma16(A + k, ga[q], __builtin_amdgcn_readfirstlane(st + q * 8192));
+    else dma16(W + k, gw[q - 4], __builtin_amdgcn_readfirstlane(st + DMA_BM * ROW + (q - 4) * 8192));
+  };
+  auto issue = [&](int kt) {
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) dma16(ga[jj] + k, __builtin_amdgcn_readfirstlane(st + jj * 8192));
-#pragma unroll
-    for (int jj = 0; jj < 4; ++jj)
-      dma16(gw[jj] + k, __builtin_amdgcn_readfirstlane(st + DMA_BM * ROW + jj * 8192));
+    for (int q = 0; q < 8; ++q) issue_one(kt, q);
   };
   // fragment reads: row R of a tile, chunk 4 half + 2 ks + fk of its 8, at position chunk ^ ((R >> 1) & 7)
   const int sw = (fr >> 1) & 7;
@@ -384,7 +387,11 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
   __syncthreads();
   read_frags(0, S0{});
   int stage = 0;                               // of tile kt
-  for (int kt = 0; kt < nkt; ++kt) {
+  // All tiles but the last run the same straight line of code, the last one a copy without the
+  // barrier section.  (With that section under an `if` inside one loop, the compiler joins the
+  // two paths in front of the last eight products and waits there for every LDS read in flight,
+  // the next tile's fragments included, which those products do not use.)
+  for (int kt = 0; kt + 1 < nkt; ++kt) {
     // first half, from set 0; the second half of the same stage goes into set 1
     multiply(0, S0{});
     __builtin_amdgcn_sched_barrier(0);
@@ -396,18 +403,23 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
     // this tile's stage free
     multiply(0, S1{});
     __builtin_amdgcn_sched_barrier(0);
-    if (kt + 1 < nkt) {
-      if (issued > kt + 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
-      if (issued + 1 < nkt) { issue(issued + 1); ++issued; }      // into the stage of tile kt
-      stage ^= 1;
-      read_frags(stage, S0{});
-    }
+    if (issued > kt + 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (issued + 1 < nkt) { issue(issued + 1); ++issued; }      // into the stage of tile kt
+    stage ^= 1;
+    read_frags(stage, S0{});
     __builtin_amdgcn_sched_barrier(0);
     multiply(1, S1{});
     __builtin_amdgcn_sched_barrier(0);
   }
+  multiply(0, S0{});
+  __builtin_amdgcn_sched_barrier(0);
+  read_frags(stage, S1{});
+  __builtin_amdgcn_sched_barrier(0);
+  multiply(1, S0{});
+  multiply(0, S1{});
+  multiply(1, S1{});
   tile_epilogue<TM, TN>(acc, bias, C, ldc, M, N, epi, m0, wm, n0, wn, lane);
 }
 
@@ -1470,7 +1482,8 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
                      ((uintptr_t)W % 16 == 0) && (K % 8 == 0);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
-  const bool dma_ok = vec_ok && K % DMA_BK == 0;
+  // the direct-to-LDS kernel addresses its operands with 32-bit byte offsets
+  const bool dma_ok = vec_ok && K % DMA_BK == 0 && (size_t)M * lda * 2 < (1ull << 32) && (size_t)N * ldw * 2 < (1ull << 32);
   if (variant == 0) {
     // 256x256 tiles run one block per CU at about 0.95 PFLOP/s through the direct-to-LDS pipeline
     // (0.88 through registers), 128x128 tiles two blocks per CU at about 0.80: the number of
@@ -1515,7 +1528,9 @@ MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, c
                      ((uintptr_t)W % 16 == 0) && (K % 8 == 0);
   // big_tiles: 256 x 256 tiles through the direct-to-LDS pipeline (many rows against few weight
   // rows and a long K: the down product of a prompt); else 128 x 128 (few rows)
-  if (big_tiles && (!vec_ok || K % DMA_BK != 0)) return (int)hipErrorInvalidValue;
+  if (big_tiles && (!vec_ok || K % DMA_BK != 0 || (size_t)M * lda * 2 >= (1ull << 32) ||
+                    (size_t)N * ldw * 2 >= (1ull << 32)))
+    return (int)hipErrorInvalidValue;
   int rc = big_tiles ? launch_tile_dma((const bf16*)A, lda, (const bf16*)W, ldw, nullptr, part, N, M, N, K,
                                        EPI_F32, stream, splits, k_per_split)
                      : launch_tile<128, 128, 64, 64>((const bf16*)A, lda, (const bf16*)W, ldw, nullptr, part, N, M,
