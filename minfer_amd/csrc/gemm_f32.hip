@@ -2,6 +2,10 @@
 // out[t][o] = dot(W[o][:], x[t][:]) + b[o], as src/graph/cpu_backend.rs:214-248 of
 // yusiwen/minfer.  Plain fp32 FMA, no reduced-precision matrix mode: this is the path
 // that shows faults bfloat16 hides.  Any M, N, K; vector loads only where they are aligned.
+// A dot product is summed in blocks of 128 terms whose sums are then added up: the rounding
+// error of one long chain grows with the root of its length (18944 terms in the down product;
+// the reference's scalar path sums in 64 bits, src/vec_ops.rs:31-35), that of blocks with the
+// roots of the block's and of the number of blocks.
 #include "common.h"
 
 namespace {
@@ -38,7 +42,9 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   const int lrow = tid >> 2, lk = (tid & 3) * 4;   // 64 rows x 4 chunks of 4 k
   const int ty = tid >> 4, tx = tid & 15;
-  float acc[4][4] = {};
+  constexpr int FLUSH = 128 / BK;                   // chunks per block of the sum
+  float acc[4][4] = {}, tot[4][4] = {};
+  int chunk = 0;
   for (int k0 = 0; k0 < K; k0 += BK) {
     const float4 a = load4(A, lda, m0 + lrow, M, k0 + lk, K, vec_ok);
     const float4 w = load4(W, ldw, n0 + lrow, N, k0 + lk, K, vec_ok);
@@ -57,7 +63,21 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(ar[i], wr[j], acc[i][j]);
     }
+    if (++chunk == FLUSH) {
+      chunk = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          tot[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+    }
   }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] += tot[i][j];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int m = m0 + ty * 4 + i;
