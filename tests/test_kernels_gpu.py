@@ -159,6 +159,18 @@ def test_rope_kvwrite(ops, dtype, nh, nk, hd):
     close(vd, vr, tol, tol)
     # untouched rows stay untouched
     assert torch.equal(kd.cpu()[1], kc[1]) and torch.equal(vd.cpu()[4], vc[4])
+    # the same from a q|k|v buffer that starts 4 bytes off a 16-byte boundary: the kernel
+    # without 16-byte loads, same result up to how the compiler fuses the multiply-adds
+    flat = torch.empty(qkv.numel() + 1, device=DEV)
+    odd = flat[1:].view(qkv.shape)
+    odd.copy_(qkv)
+    assert odd.data_ptr() % 16 == 4 and odd.is_contiguous()
+    q2 = torch.empty(t, nh * hd, dtype=dtype, device=DEV)
+    kd2, vd2 = kc.to(DEV), vc.to(DEV)
+    ops.rope_kvwrite(odd, cs.to(DEV), sn.to(DEV), pos.to(DEV), seq.to(DEV), table.to(DEV), q2, kd2, vd2, nh, nk, hd)
+    close(q2, q_ref, tol, tol)
+    close(kd2, kr, tol, tol)
+    close(vd2, vr, tol, tol)
 
 
 def test_rope_position_zero_is_identity_and_pairs_are_half_split(ops):
