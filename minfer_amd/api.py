@@ -13,7 +13,9 @@ from __future__ import annotations
 
 from typing import Any, Dict, List, Optional, Sequence, Union
 
+from .cache.paged import PAGE
 from .engine import Engine, GenerationResult, generate, load_model, random_model
+from .engine.engine import cache_bytes_per_token, tokens_that_fit
 from .sampling import SamplingParams
 
 
@@ -24,8 +26,10 @@ class LLM:
                  device: str = "cuda:0"):
         """`model`: folder with config.json and model.safetensors.  With `random_weights`, the
         configuration comes from `config` (a dict or a config.json path) or from the folder's
-        config.json, and weights are made on the device from `weight_seed`.  The cache holds
-        `max_tokens` tokens (default n_slots x n_ctx); a sequence ends at `n_ctx` positions."""
+        config.json, and weights are made on the device from `weight_seed`.  A sequence ends at
+        `n_ctx` positions.  The cache holds `max_tokens` tokens; by default as many as `n_slots`
+        sequences of `n_ctx` positions need, or what fits into the device memory that is free
+        once the weights are loaded if that is less (`cache_plan` says which)."""
         if random_weights:
             from .config.base import read_config_json
             src = config if config is not None else model
@@ -39,7 +43,16 @@ class LLM:
             self.model = load_model(model, dtype=dtype, device=device)
         self.config = self.model.config
         self.n_ctx = min(int(n_ctx), self.model.spec.max_positions)
-        self.engine = Engine(self.model, max_tokens=max_tokens or self.n_ctx * n_slots, max_seqs=n_slots)
+        wanted = n_slots * ((self.n_ctx + PAGE - 1) // PAGE * PAGE)
+        fits = None
+        if max_tokens is None:
+            fits = tokens_that_fit(self.model)
+            max_tokens = min(wanted, fits)
+        self.engine = Engine(self.model, max_tokens=max_tokens, max_seqs=n_slots)
+        per_token = cache_bytes_per_token(self.model.cache_requests(), self.model.rt.dtype)
+        self.cache_plan = dict(tokens=self.engine.capacity_tokens(), slots=n_slots, context=self.n_ctx,
+                               bytes=self.engine.capacity_tokens() * per_token, bytes_per_token=per_token,
+                               fits=fits, limited_by_memory=fits is not None and fits < wanted)
 
     @classmethod
     def from_pretrained(cls, folder: str, **kw) -> "LLM":
@@ -58,6 +71,10 @@ class LLM:
 
     def step(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], want="last"):
         return self.engine.step(slots, tokens, want)
+
+    def truncate(self, slot: int, length: int) -> None:
+        """Rolls a sequence back to its first `length` tokens (see `Engine.truncate`)."""
+        self.engine.truncate(slot, length)
 
     def generate(self, prompts: Sequence[Sequence[int]], max_new: int = 512, temp: float = 0.8,
                  top_k: int = 40, top_p: float = 0.95, repeat_penalty: float = 1.1,

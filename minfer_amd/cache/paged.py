@@ -259,7 +259,23 @@ class Cache:
         i = g.index_of[entry]
         return g.k[i], g.v[i], g
 
+    def store_kv(self, entry: int, qkv: torch.Tensor, ctx, n_heads: int, q_out: torch.Tensor) -> None:
+        """Stores the step's keys and values into the entry's pages at the tokens' positions and
+        leaves q, rounded to the run type, in `q_out`.  `qkv` is the 32-bit
+        `[tokens][(n_heads + 2 kv_heads) head_dim]` row of q|k|v with every position encoding
+        already applied.  The page layout (`v_page_shape`) is known here and in the kernels only:
+        a mixer or a position encoding never indexes pages itself."""
+        from ..kernels import ops
+        k, v, group = self.kv(entry)
+        req = group.request
+        ops.rope_kvwrite(qkv, None, None, ctx.positions, ctx.seq_of_tok, ctx.page_table(group), q_out, k, v,
+                         n_heads, req.n_kv_heads, req.head_dim, True)
+
     def state(self, entry: int) -> torch.Tensor:
+        """The entry's fixed-size state of every slot, `[max_seqs] + shape`.  A step addresses its
+        sequences' rows with `ctx.slot_ids` (int32 on the device), e.g.
+        `state.index_select(0, ctx.slot_ids.long())` and `state.index_copy_`: the slots are data,
+        so a captured decode step serves whichever slots it is bound to."""
         return self.states[entry]
 
     def page_rows(self, group: KVGroup, slots: Sequence[int], n_cols: int) -> List[List[int]]:

@@ -26,17 +26,22 @@ OPTIONS:
   --config <FILE>         config.json to use with --random-weights
   --weight-seed <N>       seed of the random weights (default 0)
   --dtype <T>             bfloat16 (default) or float32
-  --temp <T>              sampling temperature (default 0.8; 0 = greedy)
-  --greedy                greedy decoding (--temp 0)
-  --top-k <K>             top-K sampling (default 40; 0 = off)
-  --top-p <P>             top-P nucleus sampling (default 0.95)
-  --repeat-penalty <N>    penalize repeated tokens (default 1.1; 1.0 = off)
-  --frequency-penalty <N> penalize by token count in the window (default 0.0)
-  --presence-penalty <N>  penalize any token present in the window (default 0.0)
-  --stop-token <ID>       stop generation at this token id (repeatable; default: the
-                          model's eos ids)
-  -n, --n-predict <N>     max tokens to generate (default 512); also --max-new
-  --seed <N>              RNG seed for sampling (default 42)
+  --temp <T>              temperature of the draw; below 1e-6 the largest logit is taken
+                          (default 0.8)
+  --greedy                the same as --temp 0
+  --top-k <K>             draw among the K largest logits only; 0 keeps all (default 40)
+  --top-p <P>             draw among the most probable tokens that together reach P; values
+                          outside (0, 1) keep all (default 0.95)
+  --repeat-penalty <N>    logits of the last 64 tokens are divided by N (multiplied if
+                          negative); 1.0 leaves them (default 1.1)
+  --frequency-penalty <N> N times a token's count among the last 64 is taken off its logit
+                          (default 0.0)
+  --presence-penalty <N>  N is taken off the logit of every token among the last 64
+                          (default 0.0)
+  --stop-token <ID>       a token id that ends a sequence and is not emitted; may be given
+                          several times (default: the model's eos ids)
+  -n, --n-predict <N>     most tokens generated per prompt (default 512); also --max-new
+  --seed <N>              seed of the sampler's random streams (default 42)
   --n-ctx <N>             context per sequence (default 4096)
   --n-slots <N>           sequences decoded together (default: number of prompts, at most 64)
   --no-graph              do not capture the decode step as a HIP graph

@@ -141,6 +141,11 @@ class Qwen2Config:
             max_positions=self.max_position_embeddings,
             stop_tokens=self.eos_token_ids)
 
+    def ignored_tensors(self) -> Tuple[str, ...]:
+        """Tensors a file may hold that this configuration does not use: a stored copy of the
+        head when it is tied to the embedding table."""
+        return ("lm_head.weight",) if self.tie_word_embeddings else ()
+
     def random_init_std(self, tensor_name: str) -> float:
         """Standard deviation for random weights; norm gains are set to one instead."""
         return self.initializer_range

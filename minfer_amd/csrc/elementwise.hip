@@ -3,6 +3,7 @@
 // seeded normal fill.  Formulas follow yusiwen/minfer's CPU path; each kernel names its
 // source.  Statistics, angles and the residual stream are 32-bit.
 #include "common.h"
+#include "random_normal.h"
 
 // ---------------------------------------------------------------- embedding
 // h[t][:] = table[ids[t]][:], no scaling (src/graph/cpu_backend.rs:269-285).  The host
@@ -198,7 +199,9 @@ MF_API int mf_rope_table(float* cs, float* sn, int n_pos, int half, double theta
 
 // Half-split rotation of q and k (pair i with i + hd/2; x0' = x0 c - x1 s, x1' = x0 s + x1 c;
 // src/graph/cpu_backend.rs:421-431), v copied, k and v stored into the paged cache at the
-// token's position before attention reads it (src/graph/cpu_backend.rs:118-149).
+// token's position before attention reads it (src/graph/cpu_backend.rs:118-149).  Without
+// tables (cs null) nothing is rotated: the kernel then only rounds q and stores k and v that
+// some other position encoding has already treated.
 // qkv is [T][(nh + 2 nk) hd] in 32-bit with biases already added.  One block per
 // (token, head of q|k|v).
 // In bfloat16 a page of V is stored transposed in two halves, [2][hd][32 keys], the layout the
@@ -216,7 +219,7 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(
   if (head < nh) {
     OT* dst = q_out + ((size_t)t * nh + head) * hd;
     for (int i = threadIdx.x; i < half; i += 64) {
-      const float c = cs[(size_t)pos * half + i], s = sn[(size_t)pos * half + i];
+      const float c = cs ? cs[(size_t)pos * half + i] : 1.f, s = cs ? sn[(size_t)pos * half + i] : 0.f;
       const float x0 = src[i], x1 = src[i + half];
       dst[i] = from_f32<OT>(x0 * c - x1 * s);
       dst[i + half] = from_f32<OT>(x0 * s + x1 * c);
@@ -231,7 +234,7 @@ __global__ __launch_bounds__(64) void rope_kvwrite_kernel(
   if (is_k) {
     OT* dst = kcache + (((size_t)page * nk + hk) * MF_PAGE + pos % MF_PAGE) * hd;
     for (int i = threadIdx.x; i < half; i += 64) {
-      const float c = cs[(size_t)pos * half + i], s = sn[(size_t)pos * half + i];
+      const float c = cs ? cs[(size_t)pos * half + i] : 1.f, s = cs ? sn[(size_t)pos * half + i] : 0.f;
       const float x0 = src[i], x1 = src[i + half];
       dst[i] = from_f32<OT>(x0 * c - x1 * s);
       dst[i + half] = from_f32<OT>(x0 * s + x1 * c);
@@ -280,8 +283,8 @@ __global__ __launch_bounds__(256) void rope_kvwrite_vec_kernel(
     const float* src = row + (size_t)head * hd;
     const float4 x0 = *reinterpret_cast<const float4*>(src + i);
     const float4 x1 = *reinterpret_cast<const float4*>(src + i + half);
-    const float4 c = *reinterpret_cast<const float4*>(cs + (size_t)pos * half + i);
-    const float4 s = *reinterpret_cast<const float4*>(sn + (size_t)pos * half + i);
+    const float4 c = cs ? *reinterpret_cast<const float4*>(cs + (size_t)pos * half + i) : make_float4(1.f, 1.f, 1.f, 1.f);
+    const float4 s = cs ? *reinterpret_cast<const float4*>(sn + (size_t)pos * half + i) : make_float4(0.f, 0.f, 0.f, 0.f);
     OT* dst = head < nh ? q_out + ((size_t)t * nh + head) * hd
                         : kcache + (((size_t)page * nk + (head - nh)) * MF_PAGE + off) * hd;
     store4<OT>(dst + i, x0.x * c.x - x1.x * s.x, x0.y * c.y - x1.y * s.y, x0.z * c.z - x1.z * s.z,
@@ -307,11 +310,39 @@ __global__ __launch_bounds__(256) void rope_kvwrite_vec_kernel(
   }
 }
 
+// The rotation alone, in place, on the first n_rot heads of every token's [n_heads_total][hd] row
+// of 32-bit values (q and k of a q|k|v row; v is left as it is).
+__global__ __launch_bounds__(256) void rope_inplace_kernel(float* __restrict__ x, const float* __restrict__ cs,
+                                                           const float* __restrict__ sn,
+                                                           const int* __restrict__ positions, int n_rot,
+                                                           int n_heads_total, int hd) {
+  const int t = blockIdx.x, half = hd >> 1;
+  const int pos = positions[t];
+  float* row = x + (size_t)t * n_heads_total * hd;
+  for (int it = threadIdx.x; it < n_rot * half; it += 256) {
+    const int head = it / half, i = it % half;
+    const float c = cs[(size_t)pos * half + i], s = sn[(size_t)pos * half + i];
+    float* p = row + (size_t)head * hd;
+    const float x0 = p[i], x1 = p[i + half];
+    p[i] = x0 * c - x1 * s;
+    p[i + half] = x0 * s + x1 * c;
+  }
+}
+
+MF_API int mf_rope_inplace(float* x, const float* cs, const float* sn, const int* positions, int n_tok, int n_rot,
+                           int n_heads_total, int hd, hipStream_t stream) {
+  if (n_tok <= 0 || n_rot <= 0) return 0;
+  if (hd % 2 != 0 || n_rot > n_heads_total || !cs || !sn) return (int)hipErrorInvalidValue;
+  rope_inplace_kernel<<<n_tok, 256, 0, stream>>>(x, cs, sn, positions, n_rot, n_heads_total, hd);
+  return mf_launch_status();
+}
+
 MF_API int mf_rope_kvwrite(const float* qkv, const float* cs, const float* sn, const int* positions,
                            const int* seq_of_tok, const int* page_table, int pt_stride, void* q_out,
                            void* kcache, void* vcache, int is_bf16, int n_tok, int nh, int nk, int hd,
                            int write_kv, hipStream_t stream) {
   if (n_tok <= 0) return 0;
+  if ((cs == nullptr) != (sn == nullptr)) return (int)hipErrorInvalidValue;
   const bool vec = hd % 8 == 0 && (uintptr_t)qkv % 16 == 0 && (uintptr_t)cs % 16 == 0 && (uintptr_t)sn % 16 == 0 &&
                    (uintptr_t)q_out % 16 == 0 && (uintptr_t)kcache % 16 == 0 && (uintptr_t)vcache % 16 == 0;
   if (vec) {
@@ -339,33 +370,40 @@ MF_API int mf_rope_kvwrite(const float* qkv, const float* cs, const float* sn, c
 }
 
 // ---------------------------------------------------------------- seeded normal fill
-// value(i) depends only on (seed, i): two hashed uniforms through Box-Muller.
-__device__ __forceinline__ uint64_t mix64(uint64_t z) {
-  z += 0x9E3779B97F4A7C15ull;
-  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-  return z ^ (z >> 31);
-}
-
+// value(i) depends only on (seed, i) and is the same bits as the host's fill of the same
+// (seed, i) (random_normal.h, host_random.cpp).  A thread makes both members of a pair.
 template <typename OT>
 __global__ __launch_bounds__(256) void fill_normal_kernel(OT* __restrict__ out, size_t n, uint64_t seed,
-                                                          float std) {
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
-    const uint64_t h = mix64(seed ^ mix64(i));
-    const float u1 = ((float)(uint32_t)(h >> 40) + 1.0f) * (1.0f / 16777216.0f);   // (0,1]
-    const float u2 = (float)(uint32_t)((h >> 8) & 0xFFFFFF) * (1.0f / 16777216.0f);  // [0,1)
-    const float r = sqrtf(-2.0f * logf(u1));
-    out[i] = from_f32<OT>(r * cosf(6.28318530717958647692f * u2) * std);
+                                                          float std, int round_bf16) {
+  const size_t pairs = (n + 1) / 2;
+  for (size_t j = (size_t)blockIdx.x * 256 + threadIdx.x; j < pairs; j += (size_t)gridDim.x * 256) {
+    double z0, z1;
+    mf_normal_pair(seed, j, &z0, &z1);
+    float v0, v1;
+    {
+#pragma clang fp contract(off)
+      v0 = (float)z0 * std;
+      v1 = (float)z1 * std;
+    }
+    if (round_bf16) {
+      v0 = mf_bf16_value(mf_bf16_bits(v0));
+      v1 = mf_bf16_value(mf_bf16_bits(v1));
+    }
+    out[2 * j] = from_f32<OT>(v0);
+    if (2 * j + 1 < n) out[2 * j + 1] = from_f32<OT>(v1);
   }
 }
 
-MF_API int mf_fill_normal(void* out, int is_bf16, size_t n, uint64_t seed, float std,
+// `round_bf16`: a float32 output holds values that bfloat16 represents (what a tensor written in
+// bfloat16 and widened gives); a bfloat16 output is rounded in any case.
+MF_API int mf_fill_normal(void* out, int is_bf16, size_t n, uint64_t seed, float std, int round_bf16,
                           hipStream_t stream) {
   if (n == 0) return 0;
-  const int blocks = (int)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  const size_t pairs = (n + 1) / 2;
+  const int blocks = (int)((pairs + 255) / 256 < 16384 ? (pairs + 255) / 256 : 16384);
   if (is_bf16)
-    fill_normal_kernel<bf16><<<blocks, 256, 0, stream>>>((bf16*)out, n, seed, std);
+    fill_normal_kernel<bf16><<<blocks, 256, 0, stream>>>((bf16*)out, n, seed, std, 1);
   else
-    fill_normal_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, n, seed, std);
+    fill_normal_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, n, seed, std, round_bf16);
   return mf_launch_status();
 }

@@ -30,6 +30,7 @@
 // are 32 apart inside one wave's tile; the epilogue writes bfloat16 y[M][ldc], ldc = number
 // of outputs, straight from the 32-bit accumulators and the [M][2 nf] intermediate is never
 // stored.
+#include <stdio.h>
 #include <stdlib.h>
 
 #include "common.h"
@@ -446,9 +447,8 @@ int launch_tile_dma(const bf16* A, int lda, const bf16* W, int ldw, const float*
     configured = true;
   }
   const int tiles_m = (M + DMA_BM - 1) / DMA_BM, tiles_n = (N + DMA_BN - 1) / DMA_BN;
-  static const int remap = getenv("MF_NO_XCD_REMAP") ? 0 : 1;
   tile_dma_kernel<<<dim3(tiles_m * tiles_n, splits), 512, smem, stream>>>(
-      A, lda, W, ldw, bias, C, ldc, M, N, K, epi, tiles_m, remap && tiles_m * tiles_n >= 16, k_per_split);
+      A, lda, W, ldw, bias, C, ldc, M, N, K, epi, tiles_m, tiles_m * tiles_n >= 16, k_per_split);
   return mf_launch_status();
 }
 
@@ -466,10 +466,8 @@ int launch_tile_v(const bf16* A, int lda, const bf16* W, int ldw, const float* b
     configured = true;
   }
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  static const int remap = getenv("MF_NO_XCD_REMAP") ? 0 : 1;
   kern<<<dim3(tiles_m * tiles_n, splits), NTHR, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi,
-                                                                tiles_m, remap && tiles_m * tiles_n >= 16,
-                                                                k_per_split);
+                                                                tiles_m, tiles_m * tiles_n >= 16, k_per_split);
   return mf_launch_status();
 }
 
@@ -782,6 +780,48 @@ static int cu_count() {
     n_cu = prop.multiProcessorCount;
   }
   return n_cu;
+}
+
+// ---- which shapes each decode kernel takes (the launchers and `mf_gemm_bf16_plan` both ask here)
+
+// K = 256 NS for which the register-resident kernel is instantiated
+#define MF_STATIONARY_NS(X) X(4) X(6) X(8) X(10) X(12) X(14) X(16) X(20) X(24) X(28) X(32)
+
+// weights in flight per wave of the register-resident kernel: a whole slice up to NS 16, else the
+// largest divisor of NS that leaves the activations (4 NS registers) and the ring within budget
+constexpr int stationary_ring(int NS, int NT) {
+  if (NS <= 16) return NS;
+  for (int r = 10; r > 1; --r)
+    if (NS % r == 0 && 4 * NS + 4 * NT * r <= 176) return r;
+  return 1;
+}
+
+bool stationary_takes(int M, int N, int K, int epi, bool normed) {
+  if (M > 16 || K % 256 != 0 || (N + 15) / 16 < 128) return false;
+  if (epi == EPI_SWIGLU && N % 64 != 0) return false;
+  // a K above 5120 without a norm or SwiGLU to fold in (the o product of the widest models): the
+  // rolling kernel is the faster one there
+  if (K > 5120 && !normed && epi != EPI_SWIGLU) return false;
+  switch (K / 256) {
+#define MF_X(NS_) case NS_:
+    MF_STATIONARY_NS(MF_X)
+#undef MF_X
+    return true;
+  }
+  return false;
+}
+
+// one block per CU over the whole of K, for 17 to 64 rows against a matrix that gives every CU at
+// least 8 tiles of 16 weight rows
+bool panel_takes(int M, int N, int K, bool aligned, int epi, int n_cu) {
+  if (M <= 16 || M > 64 || K % 256 != 0 || !aligned) return false;
+  if (epi == EPI_SWIGLU && N % 64 != 0) return false;
+  return (N + 31) / 32 >= 4 * n_cu;
+}
+
+// the ring form of the K-split kernel needs whole chunks of 256 in every split
+bool ring_takes(bool aligned, int K, int splits, int k_per_split) {
+  return aligned && K % 256 == 0 && (long)(splits - 1) * k_per_split < K;
 }
 
 // The same split of the work as skinny16_kernel (a block owns 16 NT weight rows, its waves split
@@ -1194,7 +1234,7 @@ int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const fl
   const int grid = units < n_cu ? units : n_cu;
   // registers: 4 NS for the activations and 4 NT RING for the weights in flight, of 256.  A long
   // K keeps 8 to 10 loads of 1 KB in flight per wave, far more than a CU has outstanding anyway.
-  constexpr int RING = NS <= 16 ? NS : (NS % 10 == 0 ? 10 : 8 / NT);
+  constexpr int RING = stationary_ring(NS, NT);
   static_assert(NS % RING == 0 && 4 * NS + 4 * NT * RING <= 200, "activations and weight ring fit the registers");
   if (norm) {
     constexpr int smem = 8 * NS * 32 * (int)sizeof(float);       // the norm's weight
@@ -1407,8 +1447,7 @@ int launch_skinny_v(const bf16* A, int lda, const bf16* W, int ldw, const float*
   }
   dim3 grid((N + 127) / 128, splits);
   const bool two_pass = splits > 1 || epi == EPI_SWIGLU;   // gate and up columns sit in different waves
-  static const int no_ring = getenv("MF_NO_SKINNY_RING") ? 1 : 0;
-  if (VEC && !no_ring && K % KC == 0 && (long)(splits - 1) * k_per_split < K) {      // whole chunks only
+  if (ring_takes(VEC, K, splits, k_per_split)) {
     constexpr int smem_ring = smem + MT * 16 * SR_LD * (int)sizeof(float);
     static bool ring_configured = false;
     if (!ring_configured) {
@@ -1462,21 +1501,60 @@ int launch_panel_mt(const bf16* A, int lda, const bf16* W, int ldw, const float*
 
 int launch_panel(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc, int M, int N,
                  int K, int epi, hipStream_t stream) {
-  static const int off = getenv("MF_NO_PANEL") ? 1 : 0;
-  if (off || M <= 16 || M > 64 || K % KC != 0 || ldw % 8 != 0 || (uintptr_t)W % 16 != 0 || lda % 8 != 0 ||
-      (uintptr_t)A % 16 != 0)
-    return MF_NOT_BUILT;
-  if (epi == EPI_SWIGLU && N % 64 != 0) return MF_NOT_BUILT;
   const int n_cu = cu_count();
   if (n_cu <= 0) return (int)hipErrorUnknown;
+  const bool aligned = ldw % 8 == 0 && (uintptr_t)W % 16 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0;
+  if (!panel_takes(M, N, K, aligned, epi, n_cu)) return MF_NOT_BUILT;
   const int units = (N + 31) / 32;
-  if (units < 4 * n_cu) return MF_NOT_BUILT;
   switch ((M + 15) / 16) {
     case 2: return launch_panel_mt<2>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
     case 3: return launch_panel_mt<3>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
     case 4: return launch_panel_mt<4>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
   }
   return MF_NOT_BUILT;
+}
+
+// The tile kernel of a product with many rows: 256 x 256 tiles run one block per CU (faster
+// through the direct-to-LDS pipeline than through registers), 128 x 128 tiles two blocks per CU at a
+// somewhat lower rate each; the number of rounds the tiles take over the CUs decides.  Tiny
+// problems take 64 x 64.
+int tile_variant(int M, int N, bool dma_ok, int epi, int n_cu) {
+  const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+  const long t128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+  const long slots = n_cu > 0 ? n_cu : 1;
+  const double cost256 = (double)((t256 + slots - 1) / slots) * (256. * 256.) / (dma_ok ? 0.95 : 0.88);
+  const double cost128 = (t128 <= slots ? 1. : 2. * (double)((t128 + 2 * slots - 1) / (2 * slots))) *
+                         (128. * 128.) / 0.80;
+  int variant;
+  if (cost256 < cost128) variant = dma_ok ? 12 : 9;
+  else variant = (t128 >= 64 || M > 64) ? 2 : 3;
+  if (epi == EPI_SWIGLU && variant == 3) variant = 2;
+  return variant;
+}
+
+// Which kernel a product of at most 64 rows takes.
+enum SkinnyChoice {
+  SK_STATIONARY, SK_ROLLING, SK_GUARDED_PAIR, SK_GUARDED_4X2, SK_GUARDED_8X2, SK_GUARDED_8X1, SK_PANEL, SK_RING,
+  SK_STAGED
+};
+
+SkinnyChoice skinny_choice(int M, int N, int K, bool aligned, int epi, int splits, int k_per_split, int n_cu) {
+  if (M <= 16 && splits == 1) {
+    // the register-resident kernel where it is built; other aligned shapes the rolling K-split
+    // kernel; the rest (and SwiGLU outside the first) the guarded kernel
+    if (aligned && stationary_takes(M, N, K, epi, false)) return SK_STATIONARY;
+    if (aligned && K % 32 == 0 && epi != EPI_SWIGLU) return SK_ROLLING;
+    if (epi == EPI_SWIGLU) return SK_GUARDED_PAIR;
+    // many weight rows: 4 waves with two 16-row tiles each (less activation traffic per weight
+    // byte); a row count that would leave a short second round of 16-row blocks: 8 waves with
+    // two tiles; otherwise 8 waves, one tile
+    const int blocks16 = (N + 15) / 16;
+    if (blocks16 >= 1024) return SK_GUARDED_4X2;
+    if (blocks16 > 256 && blocks16 <= 512) return SK_GUARDED_8X2;
+    return SK_GUARDED_8X1;
+  }
+  if (M > 16 && panel_takes(M, N, K, aligned, epi, n_cu)) return SK_PANEL;
+  return ring_takes(aligned, K, splits, k_per_split) ? SK_RING : SK_STAGED;
 }
 
 }  // namespace
@@ -1496,19 +1574,7 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
   const bf16* w = (const bf16*)W;
   // the direct-to-LDS kernel addresses its operands with 32-bit byte offsets
   const bool dma_ok = vec_ok && K % DMA_BK == 0 && (size_t)M * lda * 2 < (1ull << 32) && (size_t)N * ldw * 2 < (1ull << 32);
-  if (variant == 0) {
-    // 256x256 tiles run one block per CU at about 0.95 PFLOP/s through the direct-to-LDS pipeline
-    // (0.88 through registers), 128x128 tiles two blocks per CU at about 0.80: the number of
-    // rounds decides (measured at 512, 2048 and 8192 rows); tiny problems take 64x64
-    const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-    const long t128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-    const long slots = cu_count();
-    const double cost256 = (double)((t256 + slots - 1) / slots) * (256. * 256.) / (dma_ok ? 0.95 : 0.88);
-    const double cost128 = (t128 <= slots ? 1. : 2. * (double)((t128 + 2 * slots - 1) / (2 * slots))) *
-                           (128. * 128.) / 0.80;
-    if (cost256 < cost128) variant = dma_ok ? 12 : 9;
-    else variant = (t128 >= 64 || M > 64) ? 2 : 3;
-  }
+  if (variant == 0) variant = tile_variant(M, N, dma_ok, epi, cu_count());
   if (epi == EPI_SWIGLU && variant == 3) variant = 2;      // needs two 32-column tiles per wave
   switch (variant) {
     case 1: return launch_tile<256, 256, 128, 128>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
@@ -1557,13 +1623,7 @@ MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, c
 // go round); MF_NOT_BUILT for any other, and nothing is launched.
 static int stationary16(const void* a, int lda, const bf16* w, int ldw, const float* bias, void* C, int ldc, int M,
                  int N, int K, int epi, const NormArgs* norm, hipStream_t stream) {
-  static const int off = getenv("MF_NO_STATIONARY") ? 1 : 0;
-  if (off || M > 16 || K % 256 != 0 || (N + 15) / 16 < 128) return MF_NOT_BUILT;
-  if (epi == EPI_SWIGLU && N % 64 != 0) return MF_NOT_BUILT;
-  // K of 8192 without a norm to fold in (the o product): the rolling kernel measured faster
-  // (26 us against 30 for 8192 x 8192 with one row); at 5120 x 5120 it is the other way round from
-  // 8 rows on (19 us against 15.5)
-  if (K > 5120 && !norm && epi != EPI_SWIGLU) return MF_NOT_BUILT;
+  if (!stationary_takes(M, N, K, epi, norm != nullptr)) return MF_NOT_BUILT;
   // two tiles an item where a block's share is more than one: 128-byte rows of 32-bit output
   const int n_cu = cu_count();
   if (n_cu <= 0) return (int)hipErrorUnknown;
@@ -1574,9 +1634,7 @@ static int stationary16(const void* a, int lda, const bf16* w, int ldw, const fl
                ? launch_stationary16<NS_, 2, true>(a, lda, w, ldw, bias, C, ldc, M, N, epi, norm, stream)   \
            : two ? launch_stationary16<NS_, 2, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, norm, stream) \
                  : launch_stationary16<NS_, 1, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, norm, stream);
-  switch (K / 256) {
-    MF_STATIONARY(6) MF_STATIONARY(8) MF_STATIONARY(14) MF_STATIONARY(16) MF_STATIONARY(20) MF_STATIONARY(32)
-  }
+  switch (K / 256) { MF_STATIONARY_NS(MF_STATIONARY) }
 #undef MF_STATIONARY
   return MF_NOT_BUILT;
 }
@@ -1596,30 +1654,16 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
                      ((uintptr_t)W % 16 == 0) && (K % 8 == 0);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
-  if (M <= 16 && splits == 1) {
-    // the register-resident kernel where it is built; other aligned shapes the rolling K-split
-    // kernel; the rest (and SwiGLU outside the first) the guarded kernel
-    if (vec_ok) {
-      const int rc = stationary16(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, nullptr, stream);
-      if (rc != MF_NOT_BUILT) return rc;
-    }
-    if (vec_ok && K % 32 == 0 && epi != EPI_SWIGLU)
-      return launch_rolling16<8, 1, 16>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
-    if (epi == EPI_SWIGLU)
-      return launch_skinny16<4, 2, 4, true>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    // Measured at 3584..152064 weight rows: many rows -> 4 waves with two 16-row tiles each
-    // (less activation traffic per weight byte); a row count that would leave a short second
-    // round of 16-row blocks -> 8 waves with two tiles; otherwise 8 waves, one tile.
-    const int blocks16 = (N + 15) / 16;
-    if (blocks16 >= 1024)
-      return launch_skinny16<4, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    if (blocks16 > 256 && blocks16 <= 512)
-      return launch_skinny16<8, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    return launch_skinny16<8, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-  }
-  if (M > 16) {
-    const int rc = launch_panel(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
-    if (rc != MF_NOT_BUILT) return rc;
+  const SkinnyChoice choice = skinny_choice(M, N, K, vec_ok, epi, splits, k_per_split, cu_count());
+  switch (choice) {
+    case SK_STATIONARY: return stationary16(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, nullptr, stream);
+    case SK_ROLLING: return launch_rolling16<8, 1, 16>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+    case SK_GUARDED_PAIR: return launch_skinny16<4, 2, 4, true>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case SK_GUARDED_4X2: return launch_skinny16<4, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case SK_GUARDED_8X2: return launch_skinny16<8, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case SK_GUARDED_8X1: return launch_skinny16<8, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
+    case SK_PANEL: return launch_panel(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+    default: break;
   }
   switch ((M + 15) / 16) {
     case 1: return launch_skinny<1>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
@@ -1643,4 +1687,39 @@ MF_API int mf_gemm_bf16_normed(const float* x, int ldx, const int* row_idx, cons
     return MF_NOT_BUILT;
   const NormArgs norm{g, row_idx, eps};
   return stationary16(x, ldx, (const bf16*)W, ldw, bias, C, ldc, M, N, K, epi, &norm, stream);
+}
+
+// The name of the kernel that a product of this shape takes, without launching anything: `rows`
+// activation rows against `N` weight rows of length `K`; `aligned`: 16-byte aligned operands with
+// row strides and K in multiples of 8; `splits`, `k_per_split`, `big_tiles`: the caller's K split
+// (1, K, 0 for none); `normed`: the RMS norm is to be folded in (an empty name then means "no such
+// kernel": norm and product run one after the other); `n_cu`: compute units of the device.
+MF_API int mf_gemm_bf16_plan(int M, int N, int K, int aligned, int epi, int splits, int k_per_split,
+                             int big_tiles, int normed, int n_cu, char* name, int cap) {
+  if (!name || cap < 48 || M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 3 || n_cu <= 0) return (int)hipErrorInvalidValue;
+  const char* what = "";
+  if (normed) {
+    what = (aligned && stationary_takes(M, N, K, epi, true)) ? "stationary16_kernel(norm)" : "";
+  } else if (M <= 64) {
+    switch (skinny_choice(M, N, K, aligned != 0, epi, splits, k_per_split, n_cu)) {
+      case SK_STATIONARY: what = "stationary16_kernel"; break;
+      case SK_ROLLING: what = "rolling16_kernel"; break;
+      case SK_GUARDED_PAIR: case SK_GUARDED_4X2: case SK_GUARDED_8X2: case SK_GUARDED_8X1: what = "skinny16_kernel"; break;
+      case SK_PANEL: what = "panel_kernel"; break;
+      case SK_RING: what = "skinny_ring_kernel"; break;
+      case SK_STAGED: what = "skinny_kernel"; break;
+    }
+  } else if (splits > 1) {
+    what = big_tiles ? "tile_dma_kernel(split K)" : "tile_kernel<128,128>(split K)";
+  } else {
+    const bool dma_ok = aligned && K % DMA_BK == 0 && (size_t)M * K * 2 < (1ull << 32) && (size_t)N * K * 2 < (1ull << 32);
+    switch (tile_variant(M, N, dma_ok, epi, n_cu)) {
+      case 12: what = "tile_dma_kernel"; break;
+      case 9: what = "tile_kernel<256,256>"; break;
+      case 2: what = "tile_kernel<128,128>"; break;
+      default: what = "tile_kernel<64,64>"; break;
+    }
+  }
+  snprintf(name, (size_t)cap, "%s", what);
+  return 0;
 }

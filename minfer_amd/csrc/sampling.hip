@@ -29,9 +29,11 @@ __device__ __forceinline__ uint64_t mix64(uint64_t z) {
   return z ^ (z >> 31);
 }
 
-// uniform in [0,1) with 24 bits; mirrored by minfer_amd.sampling.rng.uniform
-__device__ __forceinline__ float uniform01(uint64_t seed, uint64_t key, uint64_t step) {
-  const uint64_t h = mix64(mix64(seed ^ mix64(key)) ^ step);
+// uniform in [0,1) with 24 bits; mirrored by minfer_amd.sampling.rng.uniform.  `stream` is the
+// host's mix64(seed ^ mix64(key)) of a sequence (minfer_amd.sampling.rng.stream): the seed reaches
+// the kernels as data, so a captured step serves every seed.
+__device__ __forceinline__ float uniform01(uint64_t stream, uint64_t step) {
+  const uint64_t h = mix64(stream ^ step);
   return (float)(uint32_t)(h >> 40) * (1.0f / 16777216.0f);
 }
 
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restric
 
 // temperature draw; temp < 1e-6 falls back to greedy (src/sampler.rs:225-227)
 __device__ __forceinline__ void sample_row(const float* __restrict__ row, int rowi, int vocab, float temp,
-                                           uint64_t seed, const long long* __restrict__ keys,
+                                           const long long* __restrict__ streams,
                                            const int* __restrict__ steps, const float* __restrict__ forced_r,
                                            int* __restrict__ out) {
   __shared__ float s_val[NT / 64];
@@ -211,7 +213,7 @@ __device__ __forceinline__ void sample_row(const float* __restrict__ row, int ro
   for (int i = 0; i < w; ++i) before += s_wave_tot[i];
   const double prefix = before + incl - pm;
   float r = forced_r ? forced_r[rowi]
-                     : uniform01(seed, (uint64_t)keys[rowi], (uint64_t)(uint32_t)steps[rowi]);
+                     : uniform01((uint64_t)streams[rowi], (uint64_t)(uint32_t)steps[rowi]);
   const double rr = fmax((double)r, 1e-30);
   if (pm > 0.0 && prefix < rr && rr <= prefix + pm) {
     double cum = prefix;
@@ -232,12 +234,12 @@ __device__ __forceinline__ void sample_row(const float* __restrict__ row, int ro
 }
 
 __global__ __launch_bounds__(NT) void sample_kernel(const float* __restrict__ logits, int ld, int vocab,
-                                                    float temp, uint64_t seed,
-                                                    const long long* __restrict__ keys,
+                                                    float temp,
+                                                    const long long* __restrict__ streams,
                                                     const int* __restrict__ steps,
                                                     const float* __restrict__ forced_r,
                                                     int* __restrict__ out) {
-  sample_row(logits + (size_t)blockIdx.x * ld, blockIdx.x, vocab, temp, seed, keys, steps, forced_r, out);
+  sample_row(logits + (size_t)blockIdx.x * ld, blockIdx.x, vocab, temp, streams, steps, forced_r, out);
 }
 
 // penalties in place; prev is [rows][max_prev], n_prev[row] entries are used
@@ -514,8 +516,8 @@ __global__ __launch_bounds__(256) void topk_candidates_kernel(const float* __res
 }
 
 __global__ __launch_bounds__(NT) void sample_filtered_kernel(float* __restrict__ logits, int ld, int vocab, int k,
-                                                             float top_p, float temp, uint64_t seed,
-                                                             const long long* __restrict__ keys,
+                                                             float top_p, float temp,
+                                                             const long long* __restrict__ streams,
                                                              const int* __restrict__ steps,
                                                              const float* __restrict__ forced_r,
                                                              const float* __restrict__ cand_val,
@@ -583,7 +585,7 @@ __global__ __launch_bounds__(NT) void sample_filtered_kernel(float* __restrict__
   if (s_over) {            // too many equal values for the lists: the whole-row kernels, in place
     top_k_row(row, vocab, k);
     top_p_row(row, vocab, top_p);
-    sample_row(row, rowi, vocab, temp, seed, keys, steps, forced_r, out);
+    sample_row(row, rowi, vocab, temp, streams, steps, forced_r, out);
     return;
   }
   const int n = s_n;       // survivors, largest first, equal values in index order
@@ -663,7 +665,7 @@ __global__ __launch_bounds__(NT) void sample_filtered_kernel(float* __restrict__
   __syncthreads();
   if (tid == 0) {
     const float rnd = forced_r ? forced_r[rowi]
-                               : uniform01(seed, (uint64_t)keys[rowi], (uint64_t)(uint32_t)steps[rowi]);
+                               : uniform01((uint64_t)streams[rowi], (uint64_t)(uint32_t)steps[rowi]);
     const double rr = fmax((double)rnd, 1e-30);
     double cum = 0.0;
     int pick = vocab - 1;                // fallback: the last index (src/sampler.rs:266)
@@ -720,12 +722,12 @@ MF_API int mf_argmax(const float* logits, int ld, int rows, int vocab, int* out,
   return mf_launch_status();
 }
 
-MF_API int mf_sample(const float* logits, int ld, int rows, int vocab, float temp, uint64_t seed,
-                     const long long* keys, const int* steps, const float* forced_r, int* out,
+MF_API int mf_sample(const float* logits, int ld, int rows, int vocab, float temp,
+                     const long long* streams, const int* steps, const float* forced_r, int* out,
                      hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0 || ld < vocab) return (int)hipErrorInvalidValue;
-  sample_kernel<<<rows, NT, 0, stream>>>(logits, ld, vocab, temp, seed, keys, steps, forced_r, out);
+  sample_kernel<<<rows, NT, 0, stream>>>(logits, ld, vocab, temp, streams, steps, forced_r, out);
   return mf_launch_status();
 }
 
@@ -733,7 +735,7 @@ MF_API int mf_sample(const float* logits, int ld, int rows, int vocab, float tem
 // kernels that read the row once; `work` holds rows * 32 * 64 floats, as many ints, and rows * 32
 // ints.  The logits stay as they are unless a row has more equal values than the lists hold.
 MF_API int mf_sample_filtered(float* logits, int ld, int rows, int vocab, int k, float top_p, float temp,
-                              uint64_t seed, const long long* keys, const int* steps, const float* forced_r,
+                              const long long* streams, const int* steps, const float* forced_r,
                               void* work, int* out, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0 || ld < vocab || k < 1 || k > FAST_K_MAX || !(temp >= 1e-6f) || !work ||
@@ -746,7 +748,7 @@ MF_API int mf_sample_filtered(float* logits, int ld, int rows, int vocab, int k,
                                                                       cand_n);
   int rc = mf_launch_status();
   if (rc) return rc;
-  sample_filtered_kernel<<<rows, NT, 0, stream>>>(logits, ld, vocab, k, top_p, temp, seed, keys, steps, forced_r,
+  sample_filtered_kernel<<<rows, NT, 0, stream>>>(logits, ld, vocab, k, top_p, temp, streams, steps, forced_r,
                                                   cand_val, cand_idx, cand_n, out);
   return mf_launch_status();
 }

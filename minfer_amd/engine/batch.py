@@ -30,10 +30,10 @@ class StepContext:
     max_len: int                         # bound on position + 1 over the step's tokens
     max_new: int                         # longest run of new tokens of one sequence
     all_decode: bool                     # every sequence brings exactly one token
-    # host copies, for parts that plan on the host (and for toy parts in tests)
-    host_slots: List[int] = field(default_factory=list)
-    host_new: List[int] = field(default_factory=list)
-    host_start: List[int] = field(default_factory=list)
+    # host copies of the ragged layout, for parts that plan their launches on the host.  Which
+    # slot a sequence lives in is not among them: slots are addressed through `slot_ids` only.
+    host_new: List[int] = field(default_factory=list)        # new tokens of each sequence
+    host_start: Optional[List[int]] = None                   # tokens each held before (None in a decode step)
     new_lengths: Dict[int, int] = field(default_factory=dict)   # slot -> tokens held after the step
     _memo: Dict = field(default_factory=dict, repr=False)
 

@@ -16,20 +16,24 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from ..cache.paged import PAGE
-from ..kernels import ops
+from ..kernels import ops, tuning
 from ..sampling.params import REPEAT_LAST_N
 from .batch import StepContext
 
 
 class DecodeSession:
     """Buffers (and, once captured, the graph) for `n_seqs` sequences decoding up to
-    `max_len` positions.  `bind` points it at a set of live sequences."""
+    `max_len` positions.  `bind` points it at a set of live sequences: which slots they live in,
+    their page tables, their random streams (the sampling seed folded with each sequence's key)
+    and their positions are all data in device buffers, so one captured step serves any set of
+    sequences and any seed.  What is baked into a capture is the batch size, the reach and the
+    sampling options other than the seed."""
 
     def __init__(self, engine, n_seqs: int, max_len: int, sampler, use_graph: bool = True):
         self.engine, self.n, self.sampler = engine, n_seqs, sampler
         self.max_len = max_len
         self.n_cols = (max_len + PAGE - 1) // PAGE
-        self.use_graph = use_graph and engine.device.type == "cuda"
+        self.use_graph = use_graph and engine.device.type == "cuda" and not tuning.DEBUG_SYNC
         dev = engine.device
         i32 = dict(dtype=torch.int32, device=dev)
         self.token_ids = torch.zeros(n_seqs, **i32)
@@ -39,7 +43,7 @@ class DecodeSession:
         self.slot_ids = torch.zeros(n_seqs, **i32)
         self.tables: Dict[int, torch.Tensor] = {
             id(g): torch.full((n_seqs, self.n_cols), -1, **i32) for g in engine.cache.groups}
-        self.keys = torch.zeros(n_seqs, dtype=torch.int64, device=dev)
+        self.streams = torch.zeros(n_seqs, dtype=torch.int64, device=dev)
         self.steps = torch.zeros(n_seqs, **i32)
         self.sampled = torch.zeros(n_seqs, **i32)
         self.prev = torch.zeros((n_seqs, REPEAT_LAST_N), **i32)
@@ -52,16 +56,36 @@ class DecodeSession:
             self._events = [torch.cuda.Event() for _ in range(2)]
         self._host_out: List[Optional[List[int]]] = [None, None]
         self._launched = self._collected = 0
+        self.last_logits: Optional[torch.Tensor] = None
         self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self._graph_generation = -1          # ops.workspace_generation() the graph was captured under
         self.warm = False
         self.slots: List[int] = []
         self._host_tables: Dict[int, List[List[int]]] = {}
         engine.model.prepare(max_len)
 
     # ------------------------------------------------------------ binding
+    def abandon(self) -> None:
+        """After an error: waits for whatever is in flight and forgets it, so the session can be
+        bound again."""
+        if self.engine.device.type == "cuda":
+            torch.cuda.synchronize(self.engine.device)
+        self._collected = self._launched
+
+    def release(self) -> None:
+        """Gives up the captured graph and with it the memory pool it holds."""
+        self.graph = None
+        self.warm = False
+
     def bind(self, slots: Sequence[int], next_tokens: Sequence[int], keys: Sequence[int],
-             steps: Sequence[int]) -> None:
-        """The sequences in `slots` will each be fed `next_tokens[i]` at their current length."""
+             steps: Sequence[int], sampler=None) -> None:
+        """The sequences in `slots` will each be fed `next_tokens[i]` at their current length.
+        `keys[i]` names sequence i's random stream under the sampler's seed; `sampler` replaces
+        the session's (same options, any seed)."""
+        if sampler is not None:
+            if sampler.structure != self.sampler.structure:
+                raise ValueError("decode session bound with other sampling options than it was made for")
+            self.sampler = sampler
         if len(slots) != self.n:
             raise ValueError(f"session is for {self.n} sequences, got {len(slots)}")
         cache, dev = self.engine.cache, self.engine.device
@@ -70,7 +94,7 @@ class DecodeSession:
         self.token_ids.copy_(torch.tensor(list(next_tokens), dtype=torch.int32))
         self.positions.copy_(torch.tensor(lengths, dtype=torch.int32))
         self.slot_ids.copy_(torch.tensor(self.slots, dtype=torch.int32))
-        self.keys.copy_(torch.tensor(list(keys), dtype=torch.int64))
+        self.streams.copy_(torch.tensor(self.sampler.streams(keys), dtype=torch.int64))
         self.steps.copy_(torch.tensor(list(steps), dtype=torch.int32))
         self._host_tables = {}
         if self._launched != self._collected:
@@ -93,12 +117,12 @@ class DecodeSession:
             cache=self.engine.cache, n_tokens=self.n, n_seqs=self.n, token_ids=self.token_ids,
             positions=self.positions, seq_of_tok=self.seq_of_tok, cu_seqlens=self.cu_seqlens,
             start_pos=self.positions, slot_ids=self.slot_ids, logit_rows=None, page_tables=self.tables,
-            max_len=self.max_len, max_new=1, all_decode=True, host_slots=list(self.slots),
-            host_new=[1] * self.n, host_start=None)
+            max_len=self.max_len, max_new=1, all_decode=True, host_new=[1] * self.n, host_start=None)
 
     def _run(self) -> None:
         logits = self.engine.model.forward(self._context())
-        self.sampler(logits, self.keys, self.steps, self.sampled, self.prev, self.n_prev)
+        self.last_logits = logits          # float32 [n_seqs][vocab] of the step run last (penalties applied in place)
+        self.sampler(logits, self.streams, self.steps, self.sampled, self.prev, self.n_prev)
         ops.advance(self.token_ids, self.sampled, self.positions, self.steps, self.prev, self.n_prev, self.cursor)
 
     def step(self) -> List[int]:
@@ -129,6 +153,8 @@ class DecodeSession:
                 if self._host_tables.get(id(g)) != rows:
                     self.tables[id(g)].copy_(torch.tensor(rows, dtype=torch.int32))
                     self._host_tables[id(g)] = rows
+        if self.graph is not None and self._graph_generation != ops.workspace_generation():
+            self.release()                   # a buffer the graph points at was replaced: capture again
         if not self.use_graph:
             self._run()
         elif self.graph is not None:
@@ -141,6 +167,7 @@ class DecodeSession:
             with torch.cuda.graph(graph):
                 self._run()
             self.graph = graph
+            self._graph_generation = ops.workspace_generation()
             graph.replay()
         k = self._launched % 2
         if self._pinned is not None:

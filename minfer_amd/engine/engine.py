@@ -10,6 +10,7 @@ sequence index as data.  There is no padding: only the tokens given are run.
 """
 from __future__ import annotations
 
+from collections import OrderedDict
 from typing import Dict, List, Optional, Sequence, Union
 
 import numpy as np
@@ -26,20 +27,63 @@ class StepError(ValueError):
     """A step that cannot run: the message says which sequence and why.  Nothing changed."""
 
 
+# Decode sessions an engine keeps (each holds a captured graph with a memory pool of its own: the
+# logits of its batch size and the activations of a step); the least recently used one goes first.
+MAX_SESSIONS = 8
+
+# Device memory left alone when the cache is sized from what is free: the activations and logits
+# of the largest step, workspaces of the kernels, the pools of captured graphs.
+RESERVE_BYTES_MIN = 2 << 30
+RESERVE_FRACTION = 0.06
+
+
+def cache_bytes_per_token(requests: Dict[int, object], dtype: torch.dtype) -> int:
+    """Bytes one token of one sequence takes in the cache: K and V of every entry."""
+    from ..cache.paged import KVRequest
+    elem = torch.empty((), dtype=dtype).element_size()
+    return sum(2 * r.n_kv_heads * r.head_dim * elem for r in requests.values() if isinstance(r, KVRequest))
+
+
+def tokens_that_fit(model: DecoderModel, max_step_tokens: int = 8192) -> int:
+    """How many tokens the cache can hold in the device memory that is free now (the weights are
+    loaded), after a reserve for everything else a step needs.  The reference divides a given
+    context over its slots (src/server/slot.rs:27-32 of yusiwen/minfer); here the given is what
+    the GPU has left."""
+    if model.rt.device.type != "cuda":
+        return 1 << 30                       # (tests drive the engine through stand-ins on the host)
+    free, total = torch.cuda.mem_get_info(model.rt.device)
+    s = model.spec
+    step = max_step_tokens * s.hidden_size * 4 * 12          # residual, q|k|v, feed-forward rows of a large step
+    reserve = max(RESERVE_BYTES_MIN, int(RESERVE_FRACTION * total)) + step
+    per_token = max(1, cache_bytes_per_token(model.cache_requests(), model.rt.dtype))
+    tokens = (free - reserve) // per_token // PAGE * PAGE
+    if tokens < PAGE:
+        raise CacheError(f"no room for a cache: {free >> 20} MiB free, {reserve >> 20} MiB held back, "
+                         f"{per_token} bytes a token")
+    return int(tokens)
+
+
 class Engine:
-    def __init__(self, model: DecoderModel, max_tokens: int, max_seqs: Optional[int] = None,
+    def __init__(self, model: DecoderModel, max_tokens: Optional[int] = None, max_seqs: Optional[int] = None,
                  poison_cache: bool = False):
+        """`max_tokens`: the most tokens all live sequences hold together (each rounded up to whole
+        pages of 64); None: as many as fit into the device memory that is free after the weights
+        (`tokens_that_fit`)."""
         if not model.loaded:
             raise RuntimeError("Engine needs a model with weights")
         self.model = model
         self.device = model.rt.device
+        if max_tokens is None:
+            max_tokens = tokens_that_fit(model)
+            if max_seqs:
+                max_tokens = min(max_tokens, int(max_seqs) * ((model.spec.max_positions + PAGE - 1) // PAGE * PAGE))
         n_pages = (max_tokens + PAGE - 1) // PAGE
         self.max_seqs = int(max_seqs) if max_seqs else max(1, min(n_pages, 1024))
         self.cache = Cache(model.cache_requests(), max_tokens, self.max_seqs, model.rt.dtype, self.device,
                            poison=poison_cache)
         self.vocab_size = model.spec.vocab_size
         self.max_positions = model.spec.max_positions
-        self._sessions = {}
+        self._sessions: "OrderedDict" = OrderedDict()
 
     # ------------------------------------------------------------ sequences
     def new_sequence(self) -> int:
@@ -57,20 +101,38 @@ class Engine:
         """Tokens the cache can hold when nothing is live (whole pages)."""
         return self.cache.n_pages * PAGE
 
+    def truncate(self, slot: int, length: int) -> None:
+        """Rolls a sequence back to its first `length` tokens; the next step continues from there
+        (the reference's rollback of a conversation turn, src/conversation.rs:334-349 of
+        yusiwen/minfer).  Refused for models with per-sequence state and once a windowed layer
+        has given up pages the shorter sequence would need."""
+        try:
+            self.cache.truncate(slot, length)
+        except CacheError as e:
+            raise StepError(str(e)) from None
+
     def stop_tokens(self):
-        """The model's own stop tokens (config.json eos_token_id; the reference stops on
-        eos or <|im_end|>, src/main.rs:626-628 of yusiwen/minfer)."""
-        return tuple(self.model.spec.stop_tokens)
+        """The model's own stop tokens: config.json's eos_token_id and, where the model folder has
+        one, generation_config.json's (the reference stops on eos or <|im_end|>,
+        src/main.rs:626-628 of yusiwen/minfer)."""
+        return tuple(getattr(self.model, "stop_tokens", self.model.spec.stop_tokens))
 
     def decode_session(self, n_seqs: int, max_len: int, sampler, use_graph: bool = True):
         """A `DecodeSession` for this batch size, reused (with its captured graph) while the
-        size, the reach and the sampling options stay the same."""
+        size, the reach and the sampling options other than the seed stay the same.  At most
+        MAX_SESSIONS are kept; the one unused for longest gives up its graph and buffers."""
         from .decode import DecodeSession
         max_len = min(self.max_positions, (max_len + 255) // 256 * 256)
-        key = (n_seqs, max_len, sampler.params, use_graph)
-        if key not in self._sessions:
-            self._sessions[key] = DecodeSession(self, n_seqs, max_len, sampler, use_graph)
-        return self._sessions[key]
+        key = (n_seqs, max_len, sampler.structure, use_graph)
+        session = self._sessions.get(key)
+        if session is None:
+            while len(self._sessions) >= MAX_SESSIONS:
+                _, old = self._sessions.popitem(last=False)
+                old.release()
+            session = self._sessions[key] = DecodeSession(self, n_seqs, max_len, sampler, use_graph)
+        else:
+            self._sessions.move_to_end(key)
+        return session
 
     # ------------------------------------------------------------ one step
     def build_context(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], want: Want) -> StepContext:
@@ -140,8 +202,7 @@ class Engine:
             cache=self.cache, n_tokens=n_tok, n_seqs=n_seq, token_ids=views[0], positions=views[1],
             seq_of_tok=views[2], cu_seqlens=views[3], start_pos=views[4], slot_ids=views[5],
             logit_rows=None if rows is None else views[6], page_tables=tables, max_len=max_len,
-            max_new=max(n_new), all_decode=all(n == 1 for n in n_new),
-            host_slots=list(slots), host_new=n_new, host_start=start)
+            max_new=max(n_new), all_decode=all(n == 1 for n in n_new), host_new=n_new, host_start=start)
         ctx.new_lengths = new_len
         return ctx
 

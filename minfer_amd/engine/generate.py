@@ -18,6 +18,7 @@ from typing import Callable, Dict, List, Optional, Sequence
 import torch
 
 from ..cache.paged import PAGE
+from ..kernels import tuning
 from ..sampling.params import REPEAT_LAST_N, SamplingParams
 from ..sampling.sampler import Sampler
 
@@ -31,6 +32,8 @@ class GenerationResult:
     decode_tokens: int = 0                  # tokens produced by decode steps
     decode_seconds: float = 0.0
     batches: List[List[int]] = field(default_factory=list)   # request indices of each batch
+    forward_seconds: float = 0.0            # with MF_TIMING: decode time spent in the model's step
+    sample_seconds: float = 0.0             # with MF_TIMING: decode time spent sampling
 
     @property
     def prefill_rate(self) -> float:
@@ -91,6 +94,15 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: Optional[Sampling
     result.batches = plan_batches([len(p) for p in prompts], max_new, capacity, max_batch, limit)
     dev = engine.device
 
+    held = set()                             # slots this call has taken and not yet given back
+    timing = tuning.TIMING
+    if timing:
+        use_graph = False                    # the split needs a stop between the step and the sampling
+
+    def release(slot: int) -> None:
+        held.discard(slot)
+        engine.end_sequence(slot)
+
     def decide(req: int, tok: int, slot: int, live: Dict[int, int], length: Optional[int] = None) -> None:
         """After sampling `tok` for request `req`: stop, emit, or emit and end.  `length` is what
         the sequence held after the step that gave `tok` (default: what it holds now)."""
@@ -106,10 +118,13 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: Optional[Sampling
                 live[req] = slot
                 return
             result.finish_reasons[req] = "length"
-        engine.end_sequence(slot)
+        release(slot)
 
-    for batch in result.batches:
-        slots = {r: engine.new_sequence() for r in batch}
+    def run_batch(batch: List[int]) -> None:
+        slots = {}
+        for r in batch:
+            slots[r] = engine.new_sequence()
+            held.add(slots[r])
         windows = {r: list(prompts[r])[-REPEAT_LAST_N:] for r in batch}
         _sync(engine)
         t0 = time.perf_counter()
@@ -131,9 +146,16 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: Optional[Sampling
                 live = _decode_bound(engine, sampler, params, order, live, next_tok, windows, prompts, result,
                                      max_new, limit, decide)
             else:
+                t1 = time.perf_counter()
                 logits = engine.step([live[r] for r in order], [[next_tok[r]] for r in order], "last")
+                if timing:
+                    _sync(engine)
+                    t2 = time.perf_counter()
+                    result.forward_seconds += t2 - t1
                 toks = _sample(sampler, logits, order, [len(result.tokens[r]) for r in order],
                                [windows[r] for r in order], dev)
+                if timing:
+                    result.sample_seconds += time.perf_counter() - t2
                 result.decode_tokens += len(order)
                 was, live = live, {}
                 for r, tok in zip(order, toks):
@@ -142,6 +164,26 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: Optional[Sampling
             next_tok = {r: result.tokens[r][-1] for r in live}
         _sync(engine)
         result.decode_seconds += time.perf_counter() - t0
+
+    try:
+        for batch in result.batches:
+            run_batch(batch)
+    finally:
+        # whatever ended the loop (an error in a step, in `on_token`, an interrupt): no slot of
+        # this call stays taken, so the engine is as free for the next call as before this one
+        for slot in list(held):
+            try:
+                release(slot)
+            except Exception:
+                pass
+    if timing and result.decode_tokens:
+        import sys
+        both = result.forward_seconds + result.sample_seconds
+        print(f"[MF_TIMING] over {result.decode_tokens} tokens: sample "
+              f"{result.sample_seconds / result.decode_tokens * 1e3:6.2f} ms/tok "
+              f"({100.0 * result.sample_seconds / both:4.1f}%), forward "
+              f"{result.forward_seconds / result.decode_tokens * 1e3:6.2f} ms/tok "
+              f"({100.0 * result.forward_seconds / both:4.1f}%)", file=sys.stderr)
     return result
 
 
@@ -155,7 +197,7 @@ def _decode_bound(engine, sampler, params, order, live, next_tok, windows, promp
     cap = max(min(len(prompts[r]) + max_new, limit) for r in order)
     session = engine.decode_session(len(order), cap, sampler)
     session.bind([live[r] for r in order], [next_tok[r] for r in order], order,
-                 [len(result.tokens[r]) for r in order])
+                 [len(result.tokens[r]) for r in order], sampler=sampler)
     if params.has_penalties:
         session.set_windows([windows[r] for r in order])
     slots = dict(live)
@@ -174,6 +216,15 @@ def _decode_bound(engine, sampler, params, order, live, next_tok, windows, promp
             decide(r, tok, slots[r], now, held[r])
         alive.intersection_update(now)
 
+    try:
+        _run_bound(session, order, result, max_new, limit, held, alive, take)
+    except BaseException:
+        session.abandon()
+        raise
+    return {r: slots[r] for r in order if r in alive}
+
+
+def _run_bound(session, order, result, max_new, limit, held, alive, take) -> None:
     pending = session.launch()
     while True:
         ahead = None
@@ -188,7 +239,6 @@ def _decode_bound(engine, sampler, params, order, live, next_tok, windows, promp
             take(session.collect(ahead))
             break
         pending = ahead
-    return {r: slots[r] for r in order if r in alive}
 
 
 def _sample(sampler: Sampler, logits: torch.Tensor, keys: Sequence[int], steps: Sequence[int],
@@ -204,6 +254,6 @@ def _sample(sampler: Sampler, logits: torch.Tensor, keys: Sequence[int], steps: 
                 flat[i, :len(w)] = torch.tensor(w, dtype=torch.int32)
         prev = flat.to(device)
         n_prev = torch.tensor([min(len(w), REPEAT_LAST_N) for w in windows], dtype=torch.int32, device=device)
-    sampler(logits, torch.tensor(list(keys), dtype=torch.int64, device=device),
+    sampler(logits, torch.tensor(sampler.streams(keys), dtype=torch.int64, device=device),
             torch.tensor(list(steps), dtype=torch.int32, device=device), out, prev, n_prev)
     return out.cpu().tolist()

@@ -6,16 +6,18 @@ src/models/qwen2/loader.rs:215-350 of yusiwen/minfer).
 """
 from __future__ import annotations
 
+import json
+import os
 import warnings
-import zlib
-from typing import Any, Dict, Union
+from typing import Any, Dict, Tuple, Union
 
 import torch
 
-from ..config.base import read_config_json
+from ..config.base import ConfigError, read_config_json
 from ..kernels import ops
 from ..registry import config_from_dict
 from ..weights.loader import FolderWeights
+from ..weights.random_init import tensor_seed
 from .model import DecoderModel
 
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
@@ -36,27 +38,56 @@ def require_gpu(device) -> torch.device:
     return device
 
 
+def generation_stop_tokens(folder: str, vocab_size: int) -> Tuple[int, ...]:
+    """The `eos_token_id` entries of the folder's generation_config.json (an id or a list of
+    ids), if there is such a file.  A chat model's end-of-turn token is listed there and not in
+    config.json; the reference stops on either (eos or <|im_end|>, src/main.rs:626-628 of
+    yusiwen/minfer)."""
+    path = os.path.join(folder, "generation_config.json")
+    if not os.path.isfile(path):
+        return ()
+    try:
+        with open(path) as f:
+            raw = json.load(f)
+    except (OSError, json.JSONDecodeError) as e:
+        raise ConfigError(f"{path}: cannot be read as JSON ({e})") from None
+    v = raw.get("eos_token_id") if isinstance(raw, dict) else None
+    if v is None:
+        return ()
+    ids = v if isinstance(v, (list, tuple)) else [v]
+    for t in ids:
+        if isinstance(t, bool) or not isinstance(t, int) or not 0 <= t < vocab_size:
+            raise ConfigError(f"{path}: 'eos_token_id' must hold token ids below {vocab_size}, found {v!r}")
+    return tuple(int(t) for t in ids)
+
+
 def load_model(folder: str, dtype="bfloat16", device="cuda:0") -> DecoderModel:
-    """config.json picks the architecture; model.safetensors gives the tensors by name."""
+    """config.json picks the architecture; model.safetensors gives the tensors by name.  Stop
+    tokens are config.json's, joined by generation_config.json's where the folder has one."""
     device = require_gpu(device)
     config = config_from_dict(read_config_json(folder))
     model = DecoderModel(config.model_spec(), run_dtype(dtype), device)
     model.config = config
     expected = model.expected_tensors()
-    ignore = ()
-    if model.spec.head_name is None:
-        ignore = ("lm_head.weight",)     # tied: a stored copy of the head is not used
+    # tensors a file may hold without the model wanting them (a stored copy of a tied head)
+    ignore = tuple(getattr(config, "ignored_tensors", lambda: ())())
     source = FolderWeights(folder, expected, model.rt.dtype, device, ignore=ignore)
-    if any(n in source.files for n in ignore):
-        warnings.warn("tie_word_embeddings is set: lm_head.weight in the file is ignored")
+    found = [n for n in ignore if n in source.files and n not in expected]
+    if found:
+        warnings.warn(f"{', '.join(found)} in the file is not used by this configuration and is ignored")
     model.load(source.get)
+    spec_stops = tuple(model.spec.stop_tokens)
+    extra = tuple(t for t in generation_stop_tokens(folder, model.spec.vocab_size) if t not in spec_stops)
+    model.stop_tokens = spec_stops + extra
     return model
 
 
 def random_model(config: Union[Dict[str, Any], Any], seed: int = 0, dtype="bfloat16",
                  device="cuda:0") -> DecoderModel:
-    """Random weights made on the device (no file): matrices, tables and biases N(0, std of
-    the configuration), norm gains one; a tensor's values depend on (seed, its name)."""
+    """Random weights made on the device (no file): the tensors that `write_random_model` writes
+    for the same configuration and seed (in bfloat16) and `load_model` reads back, value for
+    value: matrices, tables and biases N(0, std of the configuration) rounded to bfloat16, norm
+    gains one; a tensor's values depend on (seed, its name, the index)."""
     device = require_gpu(device)
     if isinstance(config, dict):
         config = config_from_dict(config)
@@ -68,9 +99,12 @@ def random_model(config: Union[Dict[str, Any], Any], seed: int = 0, dtype="bfloa
     def get(name: str) -> torch.Tensor:
         ts = expected[name]
         if ts.init == "ones":
-            return torch.ones(ts.shape, dtype=torch.float32, device=device)
+            return torch.ones(ts.shape, dtype=dt, device=device)
+        if ts.init == "zeros":
+            return torch.zeros(ts.shape, dtype=dt, device=device)
         t = torch.empty(ts.shape, dtype=dt, device=device)
-        ops.fill_normal(t, (int(seed) << 32) ^ zlib.crc32(name.encode()), config.random_init_std(name))
+        ops.fill_normal(t, tensor_seed(seed, name), config.random_init_std(name), round_bf16=True)
         return t
     model.load(get)
+    model.stop_tokens = tuple(model.spec.stop_tokens)
     return model

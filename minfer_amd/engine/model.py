@@ -13,8 +13,8 @@ from typing import Callable, Dict, List, Optional
 import torch
 
 from ..kernels import ops
-from ..parts.base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Normed, Runtime, make_part)
-from ..parts.linear import Linear
+from ..parts.base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, Normed, Runtime, make_part,
+                          normed_input)
 from ..parts.spec import BlockSpec, ModelSpec
 from ..weights.loader import TensorSpec
 
@@ -37,17 +37,20 @@ class DecoderModel:
         self.rt = Runtime(dtype=dtype, device=torch.device(device))
         self.blocks = [_build_block(bs, self.rt) for bs in spec.blocks]
         self.final_norm = make_part(NORMS, spec.final_norm, self.rt, "norm")
-        self.embedding: Optional[torch.Tensor] = None
-        self.head: Optional[Linear] = None
+        self.embedding = make_part(EMBEDDINGS, spec.embedding, self.rt, "embedding")
+        self.head = make_part(HEADS, spec.head, self.rt, "head")
+        self.stop_tokens = tuple(spec.stop_tokens)      # a loader may add to them (generation_config.json)
         self.loaded = False
 
     # ------------------------------------------------------------ tensors
     def expected_tensors(self) -> Dict[str, TensorSpec]:
         s = self.spec
-        out = {s.embedding_name: TensorSpec((s.vocab_size, s.hidden_size))}
-        if s.head_name is not None:
-            out[s.head_name] = TensorSpec((s.vocab_size, s.hidden_size))
-        out.update(self.final_norm.tensor_specs())
+        out: Dict[str, TensorSpec] = {}
+        for part in (self.embedding, self.head, self.final_norm):
+            for name, ts in part.tensor_specs().items():
+                if name in out:
+                    raise ValueError(f"tensor {name!r} is claimed by two parts")
+                out[name] = ts
         for bs, block in zip(s.blocks, self.blocks):
             for part in block.parts():
                 for name, ts in part.tensor_specs().items():
@@ -60,9 +63,9 @@ class DecoderModel:
     def load(self, get: Callable[[str], torch.Tensor]) -> None:
         """`get(full name)` returns a device tensor in its storage type."""
         s = self.spec
-        self.embedding = get(s.embedding_name).contiguous()
-        # tied head: the same storage, no second copy (src/models/qwen2/loader.rs:260)
-        self.head = Linear(self.embedding if s.head_name is None else get(s.head_name))
+        self.embedding.load(get)
+        self.head.load(get)
+        self.head.tie(self.embedding)        # a tied head takes the table's storage, no second copy
         self.final_norm.load(get)
         for bs, block in zip(s.blocks, self.blocks):
             for part in block.parts():
@@ -76,6 +79,8 @@ class DecoderModel:
                 for e in self.spec.schedule if e.writes_cache}
 
     def prepare(self, max_len: int) -> None:
+        for part in (self.embedding, self.head, self.final_norm):
+            part.prepare(max_len)
         for block in self.blocks:
             for part in block.parts():
                 part.prepare(max_len)
@@ -87,7 +92,7 @@ class DecoderModel:
             raise RuntimeError("model has no weights yet")
         s = self.spec
         h = torch.empty((ctx.n_tokens, s.hidden_size), dtype=torch.float32, device=self.rt.device)
-        ops.embed(self.embedding, ctx.token_ids, h)
+        self.embedding.forward(ctx.token_ids, h)
         rows = ctx.logit_rows
         last = len(s.schedule) - 1
         for n, e in enumerate(s.schedule):
@@ -97,7 +102,7 @@ class DecoderModel:
             kept = torch.empty((rows.numel(), s.hidden_size), dtype=torch.float32, device=h.device)
             ops.gather_rows(h, rows, kept)
             h = kept
-        return self.head(Normed(self.final_norm, h), out_dtype=torch.float32)
+        return self.head.forward(normed_input(self.final_norm, self.head, h))
 
 
 def expected_tensors(spec: ModelSpec) -> Dict[str, TensorSpec]:

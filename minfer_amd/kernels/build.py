@@ -20,8 +20,10 @@ from typing import Dict, List
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 LIB_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "_lib")
 
-# library name -> source file; HEADERS: what each includes (default: common.h)
+# library name -> source file; HEADERS: what each includes (default: common.h).  A `.cpp` source is
+# host code only and is built with the host compiler.
 LIBRARIES: Dict[str, str] = {
+    "host_random": "host_random.cpp",
     "elementwise": "elementwise.hip",
     "gemm_f32": "gemm_f32.hip",
     "gemm_bf16": "gemm_bf16.hip",
@@ -30,12 +32,15 @@ LIBRARIES: Dict[str, str] = {
     "attn_prefill_bf16": "attn_prefill_bf16.hip",
     "sampling": "sampling.hip",
 }
-HEADERS = {"attn_tokens_f32": ["common.h", "attn_tokens_impl.h"],
+HEADERS = {"host_random": ["random_normal.h"],
+           "elementwise": ["common.h", "random_normal.h"],
+           "attn_tokens_f32": ["common.h", "attn_tokens_impl.h"],
            "attn_decode_bf16": ["common.h", "attn_tokens_impl.h"]}
 
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-shared", "-std=c++17",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-command-line-argument"]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-pthread", "-ffp-contract=off", "-Wno-unknown-pragmas"]
 
 
 class KernelBuildError(RuntimeError):
@@ -50,9 +55,20 @@ def _hipcc() -> str:
                            "kernels cannot be built and there is no other backend")
 
 
+def is_host_library(name: str) -> bool:
+    return LIBRARIES[name].endswith(".cpp")
+
+
+def _host_compiler() -> str:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++")):
+        if cand and (os.path.exists(cand) or shutil.which(cand)):
+            return cand
+    raise KernelBuildError("no host C++ compiler found (looked at $CXX, g++, c++, clang++)")
+
+
 def source_hash(name: str) -> str:
     h = hashlib.sha256()
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(HOST_FLAGS if is_host_library(name) else HIPCC_FLAGS).encode())
     for fname in [LIBRARIES[name]] + HEADERS.get(name, ["common.h"]):
         with open(os.path.join(CSRC, fname), "rb") as f:
             h.update(fname.encode())
@@ -102,9 +118,12 @@ def compile_library(name: str, quiet: bool = False) -> str:
     """Compiles one library; prints a line at start and every 15 s while hipcc runs."""
     so = lib_path(name)
     tmp = f"{so}.{os.getpid()}.tmp"
-    cmd = [_hipcc()] + HIPCC_FLAGS + ["-I", CSRC, os.path.join(CSRC, LIBRARIES[name]), "-o", tmp]
+    if is_host_library(name):
+        cmd = [_host_compiler()] + HOST_FLAGS + ["-I", CSRC, os.path.join(CSRC, LIBRARIES[name]), "-o", tmp]
+    else:
+        cmd = [_hipcc()] + HIPCC_FLAGS + ["-I", CSRC, os.path.join(CSRC, LIBRARIES[name]), "-o", tmp]
     if not quiet:
-        _say(f"compiling {LIBRARIES[name]} for gfx950 ...")
+        _say(f"compiling {LIBRARIES[name]}" + ("" if is_host_library(name) else " for gfx950") + " ...")
     t0 = time.time()
     env = dict(os.environ)
     env.setdefault("TMPDIR", "/tmp")
@@ -122,7 +141,7 @@ def compile_library(name: str, quiet: bool = False) -> str:
         if os.path.exists(tmp):
             os.remove(tmp)
         lines = [l for l in out.splitlines() if "packed-fp32-ops" not in l]
-        raise KernelBuildError(f"hipcc failed on {LIBRARIES[name]}:\n" + "\n".join(lines[-60:]))
+        raise KernelBuildError(f"{os.path.basename(cmd[0])} failed on {LIBRARIES[name]}:\n" + "\n".join(lines[-60:]))
     os.replace(tmp, so)
     with open(so + ".hash", "w") as f:
         f.write(source_hash(name))

@@ -5,15 +5,14 @@ cached workspaces below.
 """
 from __future__ import annotations
 
-import os
-
 import ctypes
-from ctypes import c_double, c_float, c_int, c_size_t, c_uint64, c_void_p
+import sys
+from ctypes import c_char_p, c_double, c_float, c_int, c_size_t, c_uint64, c_void_p
 from typing import Dict, Optional, Tuple
 
 import torch
 
-from . import build
+from . import build, tuning
 from ..cache.paged import v_page_shape
 
 PAGE = 64          # tokens per cache page (MF_PAGE in csrc/common.h)
@@ -37,7 +36,11 @@ _PROTOTYPES = {
         "mf_rope_table": [_P, _P, c_int, c_int, c_double, c_double, _P],
         "mf_rope_kvwrite": [_P, _P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int,
                             c_int, c_int, _P],
-        "mf_fill_normal": [_P, c_int, c_size_t, c_uint64, c_float, _P],
+        "mf_rope_inplace": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
+        "mf_fill_normal": [_P, c_int, c_size_t, c_uint64, c_float, c_int, _P],
+    },
+    "host_random": {
+        "mf_fill_normal_host": [_P, c_int, c_size_t, c_uint64, c_float, c_int, c_int],
     },
     "gemm_f32": {
         "mf_gemm_f32": [_P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
@@ -50,6 +53,7 @@ _PROTOTYPES = {
                                 c_int, c_int, _P],
         "mf_gemm_bf16_normed": [_P, c_int, _P, _P, c_float, _P, c_int, _P, _P, c_int, c_int, c_int, c_int,
                                 c_int, _P],
+        "mf_gemm_bf16_plan": [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_char_p, c_int],
     },
     "attn_tokens_f32": {
         "mf_attn_tokens_f32": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
@@ -67,11 +71,11 @@ _PROTOTYPES = {
     },
     "sampling": {
         "mf_argmax": [_P, c_int, c_int, c_int, _P, _P, c_int, _P],
-        "mf_sample": [_P, c_int, c_int, c_int, c_float, c_uint64, _P, _P, _P, _P, _P],
+        "mf_sample": [_P, c_int, c_int, c_int, c_float, _P, _P, _P, _P, _P],
         "mf_penalties": [_P, c_int, c_int, c_int, _P, c_int, _P, c_float, c_float, c_float, _P],
         "mf_top_k": [_P, c_int, c_int, c_int, c_int, _P],
         "mf_top_p": [_P, c_int, c_int, c_int, c_float, _P],
-        "mf_sample_filtered": [_P, c_int, c_int, c_int, c_int, c_float, c_float, c_uint64, _P, _P, _P, _P, _P, _P],
+        "mf_sample_filtered": [_P, c_int, c_int, c_int, c_int, c_float, c_float, _P, _P, _P, _P, _P, _P],
         "mf_advance": [_P, _P, _P, _P, c_int, _P, c_int, _P, _P, _P],
     },
 }
@@ -93,9 +97,18 @@ def _stream() -> c_void_p:
 
 
 def _check(rc: int, what: str) -> None:
+    """Raises on a launch error.  With MF_DEBUG_SYNC the stream is synchronised after every launch,
+    so a fault inside a kernel is reported here, under the name of the launch that caused it
+    (the reference's debug_sync, src/cuda.rs:378-395 of yusiwen/minfer)."""
     if rc != 0:
         raise KernelError(f"{what}: HIP error {rc}"
                           + (" (invalid argument: a size the kernel does not take)" if rc == 1 else ""))
+    if tuning.DEBUG_SYNC and not torch.cuda.is_current_stream_capturing():
+        try:
+            torch.cuda.current_stream().synchronize()
+        except RuntimeError as e:
+            raise KernelError(f"{what}: failed on the device: {e}") from None
+        print(f"[minfer_amd] {what} OK", file=sys.stderr, flush=True)
 
 
 def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
@@ -123,23 +136,35 @@ _FLOATS = (torch.float32, torch.bfloat16)
 
 # ------------------------------------------------------------------ workspaces
 _workspaces: Dict[Tuple[str, int], torch.Tensor] = {}
-
-
-_retired: list = []
+_workspace_generation = 0
 
 
 def workspace(tag: str, n_floats: int, device) -> torch.Tensor:
     """A float32 scratch tensor of at least n_floats, kept per (tag, device) and grown when
-    needed.  Kernels that use one run in stream order, so sharing it is safe.  A tensor that
-    was outgrown is kept alive: a captured graph may still hold its address."""
+    needed.  Kernels that use one run in stream order, so sharing it is safe.  When one grows,
+    the old tensor is given up and `workspace_generation()` moves on: a captured graph holds the
+    old address, so whoever keeps a graph compares the generation it captured under with the
+    current one and captures again when they differ (`DecodeSession` does)."""
+    global _workspace_generation
     key = (tag, torch.device(device).index or 0)
     w = _workspaces.get(key)
     if w is None or w.numel() < n_floats:
         if w is not None:
-            _retired.append(w)
+            _workspace_generation += 1
         w = torch.empty(max(n_floats, 1 << 16), dtype=torch.float32, device=device)
         _workspaces[key] = w
     return w
+
+
+def workspace_generation() -> int:
+    return _workspace_generation
+
+
+def note_replaced_buffer() -> None:
+    """For any other buffer whose address a captured graph may hold (a rotation table that was
+    rebuilt longer): moves the generation on, so that graphs are captured again."""
+    global _workspace_generation
+    _workspace_generation += 1
 
 
 # ------------------------------------------------------------------ element-wise
@@ -197,11 +222,26 @@ def convert(src: torch.Tensor, dst: torch.Tensor) -> None:
                                              src.numel(), _stream()), "convert")
 
 
-def fill_normal(out: torch.Tensor, seed: int, std: float) -> None:
+def fill_normal(out: torch.Tensor, seed: int, std: float, round_bf16: bool = True) -> None:
+    """N(0, std) values that depend on (seed, index) only, the same bits as `fill_normal_host`
+    gives.  `round_bf16`: a float32 tensor gets values that bfloat16 represents."""
     _need(out, "fill_normal.out", _FLOATS)
     _check(_fn("elementwise", "mf_fill_normal")(_ptr(out), _is_bf16(out), out.numel(),
-                                                 seed & 0xFFFFFFFFFFFFFFFF, float(std), _stream()),
-           "fill_normal")
+                                                 seed & 0xFFFFFFFFFFFFFFFF, float(std), 1 if round_bf16 else 0,
+                                                 _stream()), "fill_normal")
+
+
+def fill_normal_host(out: torch.Tensor, seed: int, std: float, round_bf16: bool = True, threads: int = 0) -> None:
+    """The same fill into a CPU tensor (host code only; no GPU is touched)."""
+    import os
+    if not isinstance(out, torch.Tensor) or out.is_cuda or not out.is_contiguous() or out.dtype not in _FLOATS:
+        raise KernelError("fill_normal_host: needs a contiguous float32 or bfloat16 tensor on the CPU")
+    threads = threads or max(1, min(16, os.cpu_count() or 1))
+    rc = _fn("host_random", "mf_fill_normal_host")(c_void_p(out.data_ptr()), _is_bf16(out), out.numel(),
+                                                    seed & 0xFFFFFFFFFFFFFFFF, float(std),
+                                                    1 if round_bf16 else 0, threads)
+    if rc != 0:
+        raise KernelError(f"fill_normal_host: error {rc}")
 
 
 def rope_table(n_pos: int, half: int, theta: float, freq_scale: float, device):
@@ -213,18 +253,37 @@ def rope_table(n_pos: int, half: int, theta: float, freq_scale: float, device):
     return cs, sn
 
 
-def rope_kvwrite(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
-                 seq_of_tok: torch.Tensor, page_table: torch.Tensor, q_out: torch.Tensor,
+def rope_inplace(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
+                 n_rot_heads: int, n_heads_total: int, head_dim: int) -> None:
+    """The half-split rotation alone: the first `n_rot_heads` heads of every token's
+    `[n_heads_total][head_dim]` row of 32-bit values are rotated in place."""
+    n_tok = positions.numel()
+    _need(qkv, "rope_inplace.qkv", torch.float32, (n_tok, n_heads_total * head_dim))
+    _need(cos, "rope_inplace.cos", torch.float32)
+    _need(sin, "rope_inplace.sin", torch.float32, tuple(cos.shape))
+    if cos.shape[1] != head_dim // 2 or head_dim % 2 or n_rot_heads > n_heads_total:
+        raise KernelError(f"rope_inplace: table {tuple(cos.shape)}, head_dim {head_dim}, {n_rot_heads} of {n_heads_total} heads")
+    _need(positions, "rope_inplace.positions", torch.int32, (n_tok,))
+    _check(_fn("elementwise", "mf_rope_inplace")(_ptr(qkv), _ptr(cos), _ptr(sin), _ptr(positions), n_tok,
+                                                  n_rot_heads, n_heads_total, head_dim, _stream()), "rope_inplace")
+
+
+def rope_kvwrite(qkv: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                 positions: torch.Tensor, seq_of_tok: torch.Tensor, page_table: torch.Tensor, q_out: torch.Tensor,
                  kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor], n_heads: int,
                  n_kv_heads: int, head_dim: int, write_kv: bool = True) -> None:
     """Rotates q and k, and stores k and v of the tokens at their positions in the cache pages
-    (`v_page_shape` says how V lies in a page)."""
+    (`v_page_shape` says how V lies in a page).  Without tables (cos and sin None) nothing is
+    rotated: q is rounded into q_out and k, v are stored as they come."""
     n_tok = positions.numel()
     _need(qkv, "rope.qkv", torch.float32, (n_tok, (n_heads + 2 * n_kv_heads) * head_dim))
-    _need(cos, "rope.cos", torch.float32)
-    _need(sin, "rope.sin", torch.float32, tuple(cos.shape))
-    if cos.shape[1] != head_dim // 2:
-        raise KernelError(f"rope: table has {cos.shape[1]} frequencies, head_dim {head_dim} needs {head_dim // 2}")
+    if (cos is None) != (sin is None):
+        raise KernelError("rope: cos and sin come together or not at all")
+    if cos is not None:
+        _need(cos, "rope.cos", torch.float32)
+        _need(sin, "rope.sin", torch.float32, tuple(cos.shape))
+        if cos.shape[1] != head_dim // 2:
+            raise KernelError(f"rope: table has {cos.shape[1]} frequencies, head_dim {head_dim} needs {head_dim // 2}")
     _need(positions, "rope.positions", torch.int32, (n_tok,))
     _need(seq_of_tok, "rope.seq_of_tok", torch.int32, (n_tok,))
     _need(page_table, "rope.page_table", torch.int32)
@@ -250,29 +309,30 @@ def cu_count() -> int:
     return _CU_COUNT
 
 
-STATIONARY_K = (1536, 2048, 3584, 4096, 5120, 8192)
+# K = 256 NS for which the register-resident decode product is instantiated
+# (MF_STATIONARY_NS in csrc/gemm_bf16.hip; `plan_linear` asks the library itself)
+STATIONARY_NS = (4, 6, 8, 10, 12, 14, 16, 20, 24, 28, 32)
 
 
 def stationary_shape(n: int, k: int, folded: bool = False) -> bool:
     """True where the register-resident decode product is built for [n][k] weights (aligned
-    operands given): K one of a few multiples of 256 and at least 128 tiles of 16 weight rows;
+    operands given): K = 256 NS for one of the NS above and at least 128 tiles of 16 weight rows;
     a K above 5120 only with a norm or SwiGLU folded in (`folded`)."""
-    return k in STATIONARY_K and (n + 15) // 16 >= 128 and (k <= 5120 or folded)
+    return k % 256 == 0 and k // 256 in STATIONARY_NS and (n + 15) // 16 >= 128 and (k <= 5120 or folded)
 
 
 def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None,
                 swiglu: bool = False) -> Tuple[int, int]:
-    """(splits, k_per_split) of the decode product.  One split: one kernel, K divided between the
-    waves of a block.  More: blocks of 128 weight rows with the activations staged in LDS, K split
-    so that there is about one block per CU (measured: with four times as many, the partial sums
-    and the start of each block cost a fifth more), and a second kernel that adds the parts.
+    """(splits, k_per_split) of a product with at most 64 rows.  One split: one kernel, K divided
+    between the waves of a block.  More: blocks of 128 weight rows with the activations staged in
+    LDS, K split so that there is about one block per CU, and a second kernel that adds the parts.
 
-    At most 16 rows take the one-kernel form, except against a long K (which the register-resident
-    kernel does not hold: it takes 1536 to 8192) where it does badly: from 9 rows on (every block reads its own copy of
-    the activations from L2: 42 us at 16 rows of 18944 against 33), and where a CU's share of the
-    weight rows fills its 16-row tiles poorly (5120 rows over 256 CUs: 20 each, 87 us against 57)."""
+    At most 16 rows take the one-kernel form, except against a K of 8192 and more that the
+    register-resident kernel does not hold, where it does badly from 9 rows on (every block reads
+    its own copy of the activations from L2) and where a CU's share of the weight rows fills its
+    16-row tiles poorly."""
     if target_blocks is None:
-        target_blocks = int(os.environ.get("MF_SKINNY_TARGET", 0)) or cu_count()
+        target_blocks = tuning.SKINNY_TARGET or cu_count()
     if m <= 16:
         share = (n + target_blocks - 1) // target_blocks          # weight rows of a block in the one-kernel form
         fill = share / float((share + 15) // 16 * 16)
@@ -290,10 +350,10 @@ def tile_split_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None)
     chip.  Two cases split K over blocks, with a second kernel that adds the parts:
 
     * many rows whose 256 x 256 tiles leave CUs idle or a last round nearly empty (the down product
-      of a prompt: 2,048 x 3584 is 112 such tiles for 256 CUs, or 448 of 128 x 128 at a lower rate):
-      the big tiles (`big`) with K cut in s parts, s chosen by the rounds it takes (a round of big
-      tiles costs 28.5 ns per unit of K, one of 128 x 128 tiles 18.2 ns, measured at K 18944; the
-      parts are added at about 3.5 TB/s), each part at least 2,048 of K;
+      of a prompt of 2,048 tokens at a width of 3584: 112 such tiles for 256 CUs): the big tiles
+      (`big`) with K cut in s parts, s chosen by an estimate of the rounds it takes (cost per unit
+      of K of a round of big and of 128 x 128 tiles, and of adding the parts), each part at least
+      2,048 of K;
     * a prompt of a few hundred tokens against a few thousand weight rows (some 50 tiles of
       128 x 128, bound by the weight stream): those tiles with about two blocks per CU, each with
       at least 512 of K."""
@@ -306,7 +366,7 @@ def tile_split_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None)
 
     t256 = ((m + 255) // 256) * ((n + 255) // 256)
     tiles = ((m + 127) // 128) * ((n + 127) // 128)
-    if m >= 768 and k % 64 == 0 and not os.environ.get("MF_NO_BIG_SPLIT"):
+    if m >= 768 and k % 64 == 0 and not tuning.NO_BIG_SPLIT:
         rounds = lambda blocks, slots: (blocks + slots - 1) // slots
         whole = min(rounds(t256, cu) * 28.5e-9 * k, rounds(tiles, 2 * cu) * 18.2e-9 * k)
         best, best_s = whole, 1
@@ -320,6 +380,40 @@ def tile_split_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None)
     if tiles >= cu or splits < 2:
         return 1, k, False
     return cut(splits) + (False,)
+
+
+def _k_split(m: int, n: int, k: int, swiglu: bool, aligned: bool, n_cu: Optional[int] = None) -> Tuple[int, int, bool]:
+    """(splits, k_per_split, big tiles) as `linear` and `linear_swiglu` cut a bfloat16 product."""
+    if m <= 64:
+        target = tuning.SKINNY_TARGET or n_cu
+        return skinny_plan(m, n, k, target_blocks=target, swiglu=swiglu) + (False,)
+    splits, per, big = tile_split_plan(m, n, k, target_blocks=n_cu)
+    if big and (swiglu or not aligned or k % 8):
+        return 1, k, False                     # the big tiles take aligned operands and no SwiGLU epilogue
+    return splits, per, big
+
+
+def plan_linear(m: int, n: int, k: int, swiglu: bool = False, normed: bool = False, aligned: bool = True,
+                out_bf16: bool = False, accumulate: bool = False, n_cu: Optional[int] = None) -> Dict[str, object]:
+    """Which kernel `linear` / `linear_swiglu` / `linear_normed` runs for a bfloat16 product of
+    `m` rows against `[n][k]` weights, as the library itself decides it, without launching
+    anything: {'kernel': name, 'splits': s, 'k_per_split': per}.  With `normed` an empty name
+    means that no kernel folds the norm in at this shape (norm and product then run one after
+    the other).  `n` counts the interleaved gate|up rows for `swiglu`."""
+    n_cu = n_cu or cu_count()
+    epi = EPI_SWIGLU if swiglu else (EPI_BF16 if out_bf16 else (EPI_ACC_F32 if accumulate else EPI_F32))
+    splits, per, big = 1, k, False
+    if normed:
+        if m > 16 or tuning.NO_FOLD:
+            return dict(kernel="", splits=1, k_per_split=k)
+    else:
+        splits, per, big = _k_split(m, n, k, swiglu, aligned, n_cu)
+    name = ctypes.create_string_buffer(64)
+    rc = _fn("gemm_bf16", "mf_gemm_bf16_plan")(m, n, k, 1 if aligned else 0, epi, splits, per, 1 if big else 0,
+                                               1 if normed else 0, n_cu, name, 64)
+    if rc != 0:
+        raise KernelError(f"plan_linear: error {rc} for m {m}, n {n}, k {k}")
+    return dict(kernel=name.value.decode(), splits=splits, k_per_split=per)
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -346,17 +440,16 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
     if accumulate and out.dtype != torch.float32:
         raise KernelError("linear: accumulation needs a float32 output")
     epi = EPI_BF16 if out.dtype == torch.bfloat16 else (EPI_ACC_F32 if accumulate else EPI_F32)
+    aligned = not (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8)
     if m <= 64 and variant == 0:
-        splits, per = skinny_plan(m, n, k)
+        splits, per, _ = _k_split(m, n, k, False, aligned)
         part = workspace("skinny", splits * m * n, x.device) if splits > 1 else None
         _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(bias),
                                                         _ptr(out), n, _ptr(part), m, n, k, splits, per,
                                                         epi, _stream()), "gemm_bf16_skinny")
         return
     if variant == 0:
-        splits, per, big = tile_split_plan(m, n, k)
-        if big and (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8):
-            splits = 1                           # the big tiles take aligned operands only
+        splits, per, big = _k_split(m, n, k, False, aligned)
         if splits > 1:
             part = workspace("skinny", splits * m * n, x.device)
             _check(_fn("gemm_bf16", "mf_gemm_bf16_splitk")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n,
@@ -392,16 +485,17 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, vari
     _need(out, "linear_swiglu.out", torch.bfloat16, (m, nf))
     if m == 0:
         return
+    aligned = not (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8)
     if m <= 64 and variant == 0:
-        splits, per = skinny_plan(m, n, k, swiglu=True)
+        splits, per, _ = _k_split(m, n, k, True, aligned)
         part = workspace("skinny", splits * m * n, x.device) if m > 16 or splits > 1 else None
         _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
                                                         _ptr(part), m, n, k, splits, per, EPI_SWIGLU, _stream()),
                "gemm_bf16_skinny(swiglu)")
         return
     if variant == 0:
-        splits, per, big = tile_split_plan(m, n, k)
-        if splits > 1 and not big:
+        splits, per, big = _k_split(m, n, k, True, aligned)
+        if splits > 1:
             part = workspace("skinny", splits * m * n, x.device)
             _check(_fn("gemm_bf16", "mf_gemm_bf16_splitk")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
                                                             _ptr(part), m, n, k, splits, per, EPI_SWIGLU, 0,
@@ -448,7 +542,7 @@ def linear_normed(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, row_id
         ldc = n
     if m == 0:
         return True
-    if m > 16 or os.environ.get("MF_NO_FOLD"):
+    if m > 16 or tuning.NO_FOLD:
         return False
     rc = _fn("gemm_bf16", "mf_gemm_bf16_normed")(_ptr(x), k, _ptr(row_idx), _ptr(norm_weight), float(eps),
                                                  _ptr(weight), k, _ptr(bias), _ptr(out), ldc, m, n, k, epi,
@@ -486,18 +580,13 @@ def _need_caches(what: str, kcache: torch.Tensor, vcache: torch.Tensor, dtype, n
 
 
 def decode_split_plan(n_tok: int, n_kv_heads: int, group: int, max_len: int, target_blocks: int = 256) -> int:
-    """Key splits of the bfloat16 decode attention: about one block per CU (measured best at
-    1, 8 and 64 sequences of 4 kv heads), at least 256 keys of the longest possible sequence
-    per split, at most 32 (one sequence of 30,000 keys: 22 us with 32 splits, 29 with 16; of
-    2,048 keys: 12.0 against 9.6, the merge reads every split).  The kernel divides each token's
-    own length by this number in rounds of 128 keys; a split left without keys writes an empty
-    partial and ends.  (Dealing the splits out by the tokens' lengths instead, a long
-    sequence many blocks and a short one a single block, measured no faster at 8 and 64
-    sequences of unequal lengths up to 2,048 and up to 30,000 keys, and slower where it made
-    more blocks: the blocks of short sequences end early and leave the memory to the others.)"""
+    """Key splits of the bfloat16 decode attention: about one block per CU, at least 256 keys of
+    the longest possible sequence per split, at most 32 (the merge reads every split).  The kernel
+    divides each token's own length by this number in rounds of 128 keys; a split left without
+    keys writes an empty partial and ends."""
     blocks = n_tok * n_kv_heads * ((group + 15) // 16)
-    if os.environ.get("MF_ATTN_SPLITS"):
-        return int(os.environ["MF_ATTN_SPLITS"])
+    if tuning.ATTN_SPLITS:
+        return tuning.ATTN_SPLITS
     return max(1, min(target_blocks // max(1, blocks), (max_len + 255) // 256, 32))
 
 
@@ -617,19 +706,19 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
                                          _stream()), "argmax")
 
 
-def sample(logits: torch.Tensor, temp: float, seed: int, keys: torch.Tensor, steps: torch.Tensor,
+def sample(logits: torch.Tensor, temp: float, streams: torch.Tensor, steps: torch.Tensor,
            out: torch.Tensor, forced_r: Optional[torch.Tensor] = None) -> None:
     """Temperature draw per row (greedy when temp < 1e-6).  The uniform of row i is
-    `rng.uniform(seed, keys[i], steps[i])`, or forced_r[i] when given (tests)."""
+    `rng.uniform(seed, key_i, steps[i])` for streams[i] = `rng.stream_i64(seed, key_i)`, or
+    forced_r[i] when given (tests)."""
     rows, vocab = _logit_rows(logits, "sample.logits")
-    _need(keys, "sample.keys", torch.int64, (rows,))
+    _need(streams, "sample.streams", torch.int64, (rows,))
     _need(steps, "sample.steps", torch.int32, (rows,))
     _need(out, "sample.out", torch.int32, (rows,))
     if forced_r is not None:
         _need(forced_r, "sample.forced_r", torch.float32, (rows,))
-    _check(_fn("sampling", "mf_sample")(_ptr(logits), vocab, rows, vocab, float(temp),
-                                         seed & 0xFFFFFFFFFFFFFFFF, _ptr(keys), _ptr(steps),
-                                         _ptr(forced_r), _ptr(out), _stream()), "sample")
+    _check(_fn("sampling", "mf_sample")(_ptr(logits), vocab, rows, vocab, float(temp), _ptr(streams),
+                                         _ptr(steps), _ptr(forced_r), _ptr(out), _stream()), "sample")
 
 
 def penalties(logits: torch.Tensor, prev: torch.Tensor, n_prev: torch.Tensor, repeat: float,
@@ -663,7 +752,7 @@ def sample_filtered_takes(vocab: int, k: int, temp: float) -> bool:
     return 1 <= k <= FILTERED_K_MAX and k < vocab <= FILTERED_VOCAB_MAX and temp >= 1e-6
 
 
-def sample_filtered(logits: torch.Tensor, k: int, p: float, temp: float, seed: int, keys: torch.Tensor,
+def sample_filtered(logits: torch.Tensor, k: int, p: float, temp: float, streams: torch.Tensor,
                     steps: torch.Tensor, out: torch.Tensor, forced_r: Optional[torch.Tensor] = None) -> None:
     """top-k, then top-p (off unless 0 < p < 1), then the temperature draw, as `top_k`, `top_p` and
     `sample` one after the other give it, but reading each row once: its k largest entries and their
@@ -673,15 +762,15 @@ def sample_filtered(logits: torch.Tensor, k: int, p: float, temp: float, seed: i
     rows, vocab = _logit_rows(logits, "sample_filtered.logits")
     if not sample_filtered_takes(vocab, k, temp):
         raise KernelError(f"sample_filtered: k {k}, vocabulary {vocab}, temperature {temp} are outside what it takes")
-    _need(keys, "sample_filtered.keys", torch.int64, (rows,))
+    _need(streams, "sample_filtered.streams", torch.int64, (rows,))
     _need(steps, "sample_filtered.steps", torch.int32, (rows,))
     _need(out, "sample_filtered.out", torch.int32, (rows,))
     if forced_r is not None:
         _need(forced_r, "sample_filtered.forced_r", torch.float32, (rows,))
     work = workspace("sample_filtered", rows * 32 * (2 * 64 + 1), logits.device)
     _check(_fn("sampling", "mf_sample_filtered")(_ptr(logits), vocab, rows, vocab, int(k), float(p), float(temp),
-                                                  seed & 0xFFFFFFFFFFFFFFFF, _ptr(keys), _ptr(steps),
-                                                  _ptr(forced_r), _ptr(work), _ptr(out), _stream()),
+                                                  _ptr(streams), _ptr(steps), _ptr(forced_r), _ptr(work),
+                                                  _ptr(out), _stream()),
            "sample_filtered")
 
 

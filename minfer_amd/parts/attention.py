@@ -73,14 +73,24 @@ class GQAttention(Mixer):
         qkv = self.qkv(x, out_dtype=torch.float32)
         window = 0 if self.window is None else int(self.window)
         o = torch.empty((x.shape[0], self.nh * self.hd), dtype=self.rt.dtype, device=x.device)
-        tables = self.position.rotation_tables(ctx.max_len) if self.rt.is_bf16 and ctx.all_decode else None
-        if tables is not None:         # decode: rotation, cache write and attention in one kernel
+        tables = self.position.rotation_tables(ctx.max_len)
+        if tables is not None and self.rt.is_bf16 and ctx.all_decode:
+            # decode: rotation, cache write and attention in one kernel
             ops.attn_decode_rope(qkv, tables[0], tables[1], kc, vc, table, ctx.positions, ctx.seq_of_tok, o,
                                  self.nh, self.nk, self.hd, self.scale, window, ctx.max_len, writes_cache)
             self.o(o, out=h, accumulate=True)
             return
         q = torch.empty_like(o)
-        self.position.rotate_and_store(qkv, ctx, q, kc, vc, table, self.nh, self.nk, writes_cache)
+        if tables is not None:         # rotation and cache write in one kernel
+            ops.rope_kvwrite(qkv, tables[0], tables[1], ctx.positions, ctx.seq_of_tok, table, q, kc, vc,
+                             self.nh, self.nk, self.hd, writes_cache)
+        else:                          # any other encoding: it treats q and k, the cache stores
+            self.position.encode(qkv, ctx, self.nh, self.nk)
+            if writes_cache:
+                ctx.cache.store_kv(entry, qkv, ctx, self.nh, q)
+            else:
+                ops.rope_kvwrite(qkv, None, None, ctx.positions, ctx.seq_of_tok, table, q, None, None,
+                                 self.nh, self.nk, self.hd, False)
         if self.rt.is_bf16 and not ctx.all_decode and ops.HAVE_PREFILL_ATTENTION:
             ops.attn_prefill(q, kc, vc, table, ctx, o, self.nh, self.nk, self.hd, self.scale, window)
         else:

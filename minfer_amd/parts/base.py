@@ -93,15 +93,19 @@ def normed_input(norm: "Norm", part, h: torch.Tensor, row_idx: Optional[torch.Te
 
 
 class PositionEncoding(Part):
-    def rotate_and_store(self, qkv: torch.Tensor, ctx, q_out: torch.Tensor, kcache, vcache,
-                         page_table, n_heads: int, n_kv_heads: int, write_kv: bool) -> None:
-        """Encodes positions into q (written to q_out) and k, and stores k and v of the
-        step's tokens into the cache pages."""
+    """Puts the tokens' positions into queries and keys.  Storing keys and values is not its
+    business: the cache does that (`Cache.store_kv`), so an encoding knows nothing of pages."""
+
+    def encode(self, qkv: torch.Tensor, ctx, n_heads: int, n_kv_heads: int) -> None:
+        """Encodes `ctx.positions` into the q heads (the first `n_heads`) and the k heads (the next
+        `n_kv_heads`) of the 32-bit `[tokens][(n_heads + 2 n_kv_heads) head_dim]` rows, in place;
+        the v heads stay as they are."""
         raise NotImplementedError
 
     def rotation_tables(self, max_len: int):
-        """(cos, sin) `[positions][head_dim / 2]` float32 tables if this encoding is the
-        half-split rotation the decode attention kernel can apply itself, else None."""
+        """(cos, sin) `[positions][head_dim / 2]` float32 tables if this encoding is the half-split
+        rotation, else None.  A mixer may then use kernels that rotate on the way (rotation and
+        cache write in one, or inside the decode attention) instead of calling `encode`."""
         return None
 
 
@@ -126,6 +130,32 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class Embedding(Part):
+    """Token ids in, rows of the 32-bit residual stream out."""
+
+    def forward(self, token_ids: torch.Tensor, out: torch.Tensor) -> None:
+        """Writes the row of every id (int32 on the device) into `out` (float32 `[tokens][hidden]`)."""
+        raise NotImplementedError
+
+    def table(self) -> Optional[torch.Tensor]:
+        """The `[vocab][hidden]` matrix a tied head multiplies by, if this embedding has one."""
+        return None
+
+
+class Head(Part):
+    """The wanted rows of the residual stream, after the final norm, to float32 logits."""
+
+    def tie(self, embedding: "Embedding") -> None:
+        """Called once after loading when the head shares the embedding's storage."""
+
+    def forward(self, x) -> torch.Tensor:
+        """`x`: the final norm's rows, as a tensor or (when `takes_normed`) a `Normed`.
+        Returns float32 `[rows][vocab]`."""
+        raise NotImplementedError
+
+    takes_normed = False
+
+
 class Block:
     """An arrangement of parts.  `forward` returns the residual stream, reduced to the rows
     `keep_rows` (int32 indices on the device) when given."""
@@ -148,6 +178,8 @@ FEED_FORWARDS: Dict[str, type] = {}
 NORMS: Dict[str, type] = {}
 POSITIONS: Dict[str, type] = {}
 BLOCKS: Dict[str, type] = {}
+EMBEDDINGS: Dict[str, type] = {}
+HEADS: Dict[str, type] = {}
 
 
 def _registrar(table: Dict[str, type], what: str):
@@ -165,6 +197,8 @@ register_feed_forward = _registrar(FEED_FORWARDS, "feed-forward")
 register_norm = _registrar(NORMS, "norm")
 register_position = _registrar(POSITIONS, "position encoding")
 register_block = _registrar(BLOCKS, "block arrangement")
+register_embedding = _registrar(EMBEDDINGS, "embedding")
+register_head = _registrar(HEADS, "head")
 
 
 def make_part(table: Dict[str, type], spec: PartSpec, rt: Runtime, what: str):

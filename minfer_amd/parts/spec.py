@@ -51,17 +51,29 @@ class RunEntry:
 
 @dataclass(frozen=True)
 class ModelSpec:
+    """`embedding` and `head` are parts like the others; a model with the plain table at both
+    ends gives their tensor names instead (`embedding_name`, and `head_name`, None for a head
+    tied to the table) and gets the built-in `token_embedding` and `linear_head`."""
     hidden_size: int
     vocab_size: int
-    embedding_name: str
-    head_name: Optional[str]          # None: the head is the embedding table (tied)
     final_norm: PartSpec
     blocks: Tuple[BlockSpec, ...]
     schedule: Tuple[RunEntry, ...]
     max_positions: int
+    embedding_name: Optional[str] = None
+    head_name: Optional[str] = None   # None: the head is the embedding table (tied)
     stop_tokens: Tuple[int, ...] = ()
+    embedding: Optional[PartSpec] = None
+    head: Optional[PartSpec] = None
 
     def __post_init__(self):
+        sizes = dict(vocab_size=self.vocab_size, hidden_size=self.hidden_size)
+        if self.embedding is None:
+            if self.embedding_name is None:
+                raise ValueError("ModelSpec needs an embedding part or the embedding table's tensor name")
+            object.__setattr__(self, "embedding", PartSpec("token_embedding", dict(sizes, name=self.embedding_name)))
+        if self.head is None:
+            object.__setattr__(self, "head", PartSpec("linear_head", dict(sizes, name=self.head_name)))
         for e in self.schedule:
             if not 0 <= e.block < len(self.blocks):
                 raise ValueError(f"schedule names block {e.block}, model has {len(self.blocks)}")

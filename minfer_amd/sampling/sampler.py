@@ -10,6 +10,7 @@ import torch
 
 from ..kernels import ops
 from .params import SamplingParams
+from .rng import stream_i64
 
 
 class Sampler:
@@ -17,11 +18,23 @@ class Sampler:
         params.validate()
         self.params = params
 
-    def __call__(self, logits: torch.Tensor, keys: torch.Tensor, steps: torch.Tensor, out: torch.Tensor,
+    def streams(self, keys) -> list:
+        """The random stream ids (int64 values) of the sequences with these keys under the
+        sampler's seed: what `__call__` takes as `streams`."""
+        return [stream_i64(self.params.seed, int(k)) for k in keys]
+
+    @property
+    def structure(self):
+        """What of the options shapes the kernels that run (the seed does not: it is data)."""
+        from dataclasses import replace
+        return replace(self.params, seed=0)
+
+    def __call__(self, logits: torch.Tensor, streams: torch.Tensor, steps: torch.Tensor, out: torch.Tensor,
                  prev: Optional[torch.Tensor] = None, n_prev: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """logits float32 [rows][vocab]; keys int64 [rows] (one per sequence); steps int32 [rows]
-        (draws made so far); prev int32 [rows][window] and n_prev int32 [rows] hold each
-        sequence's recent tokens when penalties are on.  Writes token ids into `out` (int32)."""
+        """logits float32 [rows][vocab]; streams int64 [rows] (`streams(keys)`, one per sequence);
+        steps int32 [rows] (draws made so far); prev int32 [rows][window] and n_prev int32 [rows]
+        hold each sequence's recent tokens when penalties are on.  Writes token ids into `out`
+        (int32)."""
         p = self.params
         if p.has_penalties:
             if prev is None or n_prev is None:
@@ -31,11 +44,11 @@ class Sampler:
             ops.argmax(logits, out)
             return out
         if ops.sample_filtered_takes(logits.shape[-1], p.top_k, p.temp):
-            ops.sample_filtered(logits, p.top_k, p.top_p, p.temp, p.seed, keys, steps, out)
+            ops.sample_filtered(logits, p.top_k, p.top_p, p.temp, streams, steps, out)
             return out
         if p.top_k > 0:
             ops.top_k(logits, p.top_k)
         if 0.0 < p.top_p < 1.0:
             ops.top_p(logits, p.top_p)
-        ops.sample(logits, p.temp, p.seed, keys, steps, out)
+        ops.sample(logits, p.temp, streams, steps, out)
         return out

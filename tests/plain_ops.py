@@ -47,9 +47,10 @@ def convert(src, dst):
     dst.copy_(src.to(dst.dtype))
 
 
-def fill_normal(out, seed, std):
-    g = torch.Generator(device="cpu").manual_seed(seed & 0x7FFFFFFFFFFFFFFF)
-    out.copy_((torch.randn(out.shape, generator=g, dtype=torch.float32) * std).to(out.dtype))
+def fill_normal(out, seed, std, round_bf16=True):
+    """The library's own host fill: the numbers are defined by csrc/random_normal.h, on both sides."""
+    from minfer_amd.kernels import ops
+    ops.fill_normal_host(out, seed, std, round_bf16)
 
 
 def rope_table(n_pos, half, theta, freq_scale, device):
@@ -64,8 +65,11 @@ def rope_kvwrite(qkv, cos, sin, positions, seq_of_tok, page_table, q_out, kcache
     t = positions.numel()
     half = head_dim // 2
     x = qkv.double().view(t, n_heads + 2 * n_kv_heads, head_dim)
-    c = cos[positions.long()].double()[:, None, :]
-    s = sin[positions.long()].double()[:, None, :]
+    if cos is None:                      # nothing is rotated: q is rounded, k and v are stored
+        c, s = torch.ones(t, 1, half, dtype=torch.float64), torch.zeros(t, 1, half, dtype=torch.float64)
+    else:
+        c = cos[positions.long()].double()[:, None, :]
+        s = sin[positions.long()].double()[:, None, :]
 
     def rot(v):
         v0, v1 = v[..., :half], v[..., half:]
@@ -83,6 +87,16 @@ def rope_kvwrite(qkv, cos, sin, positions, seq_of_tok, page_table, q_out, kcache
         vcache[page, :, (pos % PAGE) // 32, :, pos % 32] = v
     else:
         vcache[page, :, pos % PAGE, :] = v
+
+
+def rope_inplace(qkv, cos, sin, positions, n_rot_heads, n_heads_total, head_dim):
+    t, half = positions.numel(), head_dim // 2
+    x = qkv.view(t, n_heads_total, head_dim)
+    c = cos[positions.long()].double()[:, None, :]
+    s = sin[positions.long()].double()[:, None, :]
+    v = x[:, :n_rot_heads].double()
+    v0, v1 = v[..., :half], v[..., half:]
+    x[:, :n_rot_heads] = torch.cat([v0 * c - v1 * s, v0 * s + v1 * c], dim=-1).float()
 
 
 def linear(x, weight, bias, out, accumulate=False, variant=0):
@@ -190,14 +204,20 @@ def argmax(logits, out):
         out[i] = pq.greedy(logits[i].numpy())
 
 
-def sample(logits, temp, seed, keys, steps, out, forced_r=None):
+def stream_uniform(stream_i64: int, step: int) -> float:
+    """The draw of a stream id (as an int64 tensor holds it) at a step: the device's uniform01."""
+    from minfer_amd.sampling.rng import mix64
+    h = mix64((stream_i64 & 0xFFFFFFFFFFFFFFFF) ^ (step & 0xFFFFFFFFFFFFFFFF))
+    return (h >> 40) / 16777216.0
+
+
+def sample(logits, temp, streams, steps, out, forced_r=None):
     import plain_qwen2 as pq
-    from minfer_amd.sampling.rng import uniform
     for i in range(logits.shape[0]):
         if temp < 1e-6:
             out[i] = pq.greedy(logits[i].numpy())
             continue
-        r = float(forced_r[i]) if forced_r is not None else uniform(seed, int(keys[i]), int(steps[i]))
+        r = float(forced_r[i]) if forced_r is not None else stream_uniform(int(streams[i]), int(steps[i]))
         out[i] = pq.sample_from_probs(pq.temperature_probs(logits[i].numpy(), temp), r)
 
 
@@ -224,12 +244,12 @@ def sample_filtered_takes(vocab, k, temp):
     return 1 <= k <= 48 and k < vocab <= 32 * 256 * 32 and temp >= 1e-6
 
 
-def sample_filtered(logits, k, p, temp, seed, keys, steps, out, forced_r=None):
+def sample_filtered(logits, k, p, temp, streams, steps, out, forced_r=None):
     work = logits.clone()
     top_k(work, k)
     if 0.0 < p < 1.0:
         top_p(work, p)
-    sample(work, temp, seed, keys, steps, out, forced_r)
+    sample(work, temp, streams, steps, out, forced_r)
 
 
 def advance(next_ids, sampled, positions, steps, prev=None, n_prev=None, cursor=None):
@@ -245,7 +265,7 @@ def advance(next_ids, sampled, positions, steps, prev=None, n_prev=None, cursor=
 
 
 NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", "rope_table",
-         "rope_kvwrite", "linear", "attn_tokens", "attn_prefill", "argmax", "sample", "penalties",
+         "rope_kvwrite", "rope_inplace", "linear", "attn_tokens", "attn_prefill", "argmax", "sample", "penalties",
          "top_k", "top_p", "sample_filtered", "sample_filtered_takes", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed", "attn_decode_rope"]
 
 

@@ -1,5 +1,6 @@
-"""Shared helpers of the replay tests: requests, the three ways of cutting them into
-steps, and the comparison with the plain implementation."""
+"""Shared helpers of the replay tests: requests, the ways of cutting them into steps (whole,
+the last tokens one by one, unequal batches, prompts in portions), and the comparison with the
+plain implementation."""
 from __future__ import annotations
 
 import numpy as np
@@ -15,6 +16,18 @@ from tiny import random_tokens
 BF16_RMS = 0.01
 BF16_MAX = 0.055
 F32_ABS = 1e-4
+# The tiny configurations (up to three layers) are all held to these figures.  At the 7B widths a
+# single layer already comes close to them, and every further layer adds roundings of its own,
+# independent of the others': the error's rms grows about with the root of the depth.  Measured at
+# those widths, worst row of five requests: the engine's own composition run on host stand-ins that
+# round at the same places and compute in 64 bits in between, so that nothing but the roundings
+# separates it from the plain implementation, differs from it by 0.81 % rms at one layer and
+# 1.40 % at four; the GPU engine by 0.83 % and 1.48 %.  A test of a deeper model at such widths
+# passes its depth and is held to the figures above times sqrt(layers).
+
+
+def bf16_depth_factor(layers: int) -> float:
+    return max(1.0, float(layers) ** 0.5)
 
 
 def requests_for(vocab: int, lengths, seed: int = 0):
@@ -73,6 +86,31 @@ def batch_steps(requests, batches, prompt_frac: float = 0.6):
     return steps
 
 
+def chunk_steps(requests, batches, sizes=(2, 50, 64, 1, 17)):
+    """Prompts fed in portions.  The requests of a batch go on together; at every step each one
+    still alive brings its next portion, whose sizes run through `sizes` with a different start
+    for each request, so portions begin and end on and off page edges, a portion of several
+    tokens meets a non-empty cache, and one request's single token shares a step with another's
+    fifty.  Every position's logits are asked for; a request ends when its tokens run out."""
+    steps = []
+    for batch in batches:
+        done = {rid: 0 for rid in batch}
+        turn = {rid: i for i, rid in enumerate(batch)}
+        live = list(batch)
+        while live:
+            entries, ends = [], []
+            for rid in live:
+                n = min(sizes[turn[rid] % len(sizes)], len(requests[rid]) - done[rid])
+                turn[rid] += 1
+                entries.append(dict(id=rid, tokens=requests[rid][done[rid]:done[rid] + n], want=list(range(n))))
+                done[rid] += n
+                if done[rid] == len(requests[rid]):
+                    ends.append(rid)
+            steps.append(dict(step=len(steps), entries=entries, end=ends))
+            live = [rid for rid in live if rid not in ends]
+    return steps
+
+
 def run_steps(engine, steps):
     """Drives Engine.step with trace steps; returns {(request, position): logits row}."""
     slots, pos, rows = {}, {}, {}
@@ -97,22 +135,24 @@ def run_steps(engine, steps):
     return rows
 
 
-def compare(rows, ref, dtype: str, what: str):
-    """Every produced row against the plain implementation's; names the first bad place."""
+def compare(rows, ref, dtype: str, what: str, layers: int = 1):
+    """Every produced row against the plain implementation's; names the first bad place.
+    `layers`: the model's depth (it scales the bfloat16 bound beyond three layers)."""
     assert rows, "nothing was produced"
     worst = 0.0
+    depth = bf16_depth_factor(layers)
     for (rid, p), got in sorted(rows.items()):
         want = ref[rid][p]
         diff = got.astype(np.float64) - want
         err = float(np.abs(diff).max())
-        tol = F32_ABS if dtype == "float32" else BF16_MAX * float(want.std())
+        tol = F32_ABS if dtype == "float32" else BF16_MAX * depth * float(want.std())
         assert np.isfinite(got).all(), f"{what}: non-finite logits at request {rid} position {p}"
         assert err <= tol, (f"{what} [{dtype}]: request {rid} position {p} (of {len(ref[rid])}): "
                             f"max abs err {err:.3e} > {tol:.3e}")
         if dtype != "float32":
             rms = float(np.sqrt(np.mean(diff * diff)))
-            assert rms <= BF16_RMS * float(want.std()), (
+            assert rms <= BF16_RMS * depth * float(want.std()), (
                 f"{what} [{dtype}]: request {rid} position {p}: rms err {rms:.3e} > "
-                f"{BF16_RMS * float(want.std()):.3e}")
+                f"{BF16_RMS * depth * float(want.std()):.3e}")
         worst = max(worst, err)
     return worst

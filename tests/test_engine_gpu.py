@@ -4,7 +4,8 @@ requests end earlier, one batch after another so that slots are used again."""
 import pytest
 
 from plain_qwen2 import PlainQwen2
-from replays import batch_steps, compare, plain_logits, requests_for, run_steps, tail_steps, whole_steps
+from replays import (batch_steps, chunk_steps, compare, plain_logits, requests_for, run_steps, tail_steps,
+                     whole_steps)
 from tiny import TINIES, write_tiny
 
 pytestmark = pytest.mark.gpu
@@ -40,6 +41,9 @@ def test_three_replays_agree_with_plain(folders, plains, name, dtype):
     compare(run_steps(eng, tail_steps(reqs)), ref, dtype, f"tiny {name} last 32 one by one")
     batches = [ids[:3], ids[3:]] if len(ids) > 3 else [ids]
     compare(run_steps(eng, batch_steps(reqs, batches)), ref, dtype, f"tiny {name} unequal batches")
+    compare(run_steps(eng, chunk_steps(reqs, batches)), ref, dtype, f"tiny {name} prompts in portions")
+    compare(run_steps(eng, chunk_steps(reqs, [[r] for r in ids], sizes=(17,))), ref, dtype,
+            f"tiny {name} prompts in portions of 17")
     assert not eng.cache.live_slots()
 
 
@@ -69,3 +73,93 @@ def test_other_storage_types_in_the_bfloat16_run(tmp_path, stored):
     ref = plain_logits(plain, reqs)
     compare(run_steps(eng, batch_steps(reqs, [list(reqs)])), ref, "bfloat16", f"stored {stored}")
     compare(run_steps(eng, tail_steps(reqs, tail=4)), ref, "bfloat16", f"stored {stored} one by one")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_truncate_then_feed_again_gives_the_same_rows(folders, plains, dtype):
+    """A sequence rolled back to a shorter length and fed other tokens, then rolled back again and
+    fed the first ones: the rows after each roll-back are those of a sequence that never held the
+    dropped tokens, across a page edge and with pages given back in between."""
+    import numpy as np
+    name = "B"
+    vocab = TINIES[name]["vocab_size"]
+    reqs = requests_for(vocab, (150, 150), seed=11)
+    a, b = reqs["r0"], reqs["r1"]
+    eng = engine_for(folders[name], dtype, max_tokens=64 * 4)
+    s = eng.new_sequence()
+    first = eng.step([s], [a], "all").cpu().numpy()
+    eng.truncate(s, 60)                                   # below the first page edge: two pages go back
+    assert eng.length(s) == 60 and eng.cache.free_tokens() == 64 * 3
+    mixed = a[:60] + b[60:140]
+    second = eng.step([s], [mixed[60:]], "all").cpu().numpy()
+    eng.truncate(s, 100)
+    third = eng.step([s], [mixed[100:]], "all").cpu().numpy()
+    eng.truncate(s, 60)
+    again = eng.step([s], [a[60:]], "all").cpu().numpy()
+    eng.end_sequence(s)
+    eng.cache.check_invariants()
+    ref_a, ref_m = plains[name].forward(a), plains[name].forward(mixed)
+    rows = {("a", p): first[p] for p in range(150)}
+    rows.update({("m", 60 + i): second[i] for i in range(80)})
+    rows.update({("m2", 100 + i): third[i] for i in range(40)})
+    rows.update({("a2", 60 + i): again[i] for i in range(90)})
+    compare(rows, {"a": ref_a, "m": ref_m, "m2": ref_m, "a2": ref_a}, dtype, "truncate")
+    if dtype == "float32":
+        assert np.abs(again - first[60:]).max() < 2e-5
+    with pytest.raises(Exception, match="truncate"):
+        s2 = eng.new_sequence()
+        eng.truncate(s2, 5)
+
+
+def test_random_model_on_the_device_is_the_written_folder(tmp_path):
+    """`write_random_model` + `load_model` and `random_model` give the same tensors for the same
+    configuration and seed, in both run types: one stream of random numbers, host and device."""
+    import torch
+    from minfer_amd import config_from_dict, load_model, random_model, write_random_model
+    for name, seed in (("A", 3), ("C", 12345678901)):
+        cfg = config_from_dict(TINIES[name])
+        folder = write_random_model(str(tmp_path / f"rw_{name}"), cfg, seed)
+        for dtype in ("bfloat16", "float32"):
+            loaded, made = load_model(folder, dtype=dtype), random_model(cfg, seed=seed, dtype=dtype)
+            pairs = [(loaded.embedding.weight, made.embedding.weight), (loaded.head.weight, made.head.weight),
+                     (loaded.final_norm.weight, made.final_norm.weight)]
+            for lb, mb in zip(loaded.blocks, made.blocks):
+                pairs += [(lb.mixer.qkv.weight, mb.mixer.qkv.weight), (lb.mixer.qkv.bias, mb.mixer.qkv.bias),
+                          (lb.mixer.o.weight, mb.mixer.o.weight), (lb.feed_forward.down.weight, mb.feed_forward.down.weight),
+                          (lb.mixer_norm.weight, mb.mixer_norm.weight)]
+                if lb.feed_forward.fused is not None:
+                    pairs.append((lb.feed_forward.fused, mb.feed_forward.fused))
+                else:
+                    pairs.append((lb.feed_forward.gate_up.weight, mb.feed_forward.gate_up.weight))
+            for x, y in pairs:
+                assert x.dtype == y.dtype and torch.equal(x, y)
+            assert loaded.embedding.weight.float().std().item() == pytest.approx(cfg.initializer_range, rel=0.05)
+    other = random_model(config_from_dict(TINIES["A"]), seed=4, dtype="bfloat16")
+    assert not torch.equal(other.embedding.weight, load_model(str(tmp_path / "rw_A"), dtype="bfloat16").embedding.weight)
+
+
+def test_sessions_and_memory_stay_flat_over_many_seeds(folders):
+    """Twenty calls with twenty seeds: the seed is data of the captured step, so the engine keeps
+    one decode session per batch size and the device memory in use does not grow."""
+    import torch
+    from minfer_amd import LLM
+    from minfer_amd.engine.engine import MAX_SESSIONS
+    llm = LLM(folders["A"], dtype="bfloat16", n_ctx=128, n_slots=2)
+    prompts = [[5, 6, 7], [9, 10]]
+    outs = set()
+    sizes = []
+    for seed in range(20):
+        res = llm.generate(prompts, max_new=8, temp=0.9, seed=seed, stop_tokens=[])
+        outs.add(tuple(map(tuple, res.tokens)))
+        torch.cuda.synchronize()
+        sizes.append((len(llm.engine._sessions), torch.cuda.memory_allocated()))
+    assert len(outs) > 10, "different seeds give different tokens"
+    assert sizes[-1][0] == sizes[2][0] <= 2, sizes
+    assert sizes[-1][1] <= sizes[2][1], "allocated memory grew with the number of seeds"
+    again = llm.generate(prompts, max_new=8, temp=0.9, seed=3, stop_tokens=[])
+    assert tuple(map(tuple, again.tokens)) in outs
+    # other options: other sessions, and never more than the bound
+    for k in range(MAX_SESSIONS + 3):
+        llm.generate(prompts, max_new=3, temp=0.5 + 0.01 * k, seed=1, stop_tokens=[])
+    assert len(llm.engine._sessions) <= MAX_SESSIONS
+    assert not llm.engine.cache.live_slots()

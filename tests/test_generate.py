@@ -219,3 +219,65 @@ def test_step_errors_leave_the_cache_alone(tmp_path):
         llm.step([t], [[1] * 100])
     assert llm.engine.length(t) == 0
     llm.engine.cache.check_invariants()
+
+
+def test_an_error_in_the_middle_of_a_batch_leaves_no_slot_taken(tmp_path):
+    """A step that raises, or an `on_token` that raises, ends the call; every slot the call had
+    taken is given back, so the engine is as free as before."""
+    class Failing(ScriptedEngine):
+        def step(self, slots, tokens, want="last"):
+            if len(self.calls) == 2:
+                raise RuntimeError("scripted failure in the third step")
+            return super().step(slots, tokens, want)
+    eng = Failing({10: [5, 6, 7, 8, 9], 20: [7, 8, 9, 11, 12], 30: [1, 2, 3]}, max_seqs=2)
+    with pytest.raises(RuntimeError, match="scripted failure"):
+        generate(eng, [[10, 1], [20, 3], [30]], GREEDY, max_new=5, stop_tokens=[], use_graph=False)
+    assert eng.end_bookkeeping() == {} and sorted(eng.free) == [0, 1]
+    eng2 = ScriptedEngine({10: [5, 6, 7, 8, 9], 20: [7, 8, 9, 11, 12]})
+
+    def boom(r, t):
+        if t == 8:
+            raise KeyError("callback")
+    with pytest.raises(KeyError):
+        generate(eng2, [[10, 1], [20, 3]], GREEDY, max_new=5, stop_tokens=[], use_graph=False, on_token=boom)
+    assert eng2.end_bookkeeping() == {} and len(eng2.free) == 8
+    # the real engine through the captured-step path of the loop (stand-in kernels on the host)
+    from minfer_amd import LLM
+    llm = LLM(write_tiny(tmp_path, "A", seed=2), dtype="float32", device="cpu", n_ctx=64, n_slots=2)
+    count = []
+
+    def third(r, t):
+        count.append(t)
+        if len(count) == 5:
+            raise ValueError("stop here")
+    with pytest.raises(ValueError, match="stop here"):
+        llm.generate([[1, 2, 3], [4, 5]], max_new=6, temp=0.0, stop_tokens=[], on_token=third)
+    assert not llm.engine.cache.live_slots()
+    llm.engine.cache.check_invariants()
+    assert llm.generate([[1, 2, 3], [4, 5]], max_new=3, temp=0.0, stop_tokens=[]).finish_reasons == ["length"] * 2
+
+
+def test_stop_tokens_come_from_config_and_generation_config(tmp_path):
+    """config.json's eos ids, joined by generation_config.json's (where a chat model lists its
+    end-of-turn token); an explicit list replaces both."""
+    import json
+    from minfer_amd import LLM
+    folder = write_tiny(tmp_path, "A", seed=2)                     # eos_token_id 7 in config.json
+    llm = LLM(folder, dtype="float32", device="cpu", n_ctx=64, n_slots=1)
+    assert llm.engine.stop_tokens() == (7,)
+    with open(folder + "/generation_config.json", "w") as f:
+        json.dump({"eos_token_id": [9, 7], "temperature": 0.7}, f)
+    llm = LLM(folder, dtype="float32", device="cpu", n_ctx=64, n_slots=1)
+    assert llm.engine.stop_tokens() == (7, 9)
+    free = llm.generate([[1, 2, 3]], max_new=8, temp=0.0, stop_tokens=[]).tokens[0]
+    with open(folder + "/generation_config.json", "w") as f:
+        json.dump({"eos_token_id": free[2]}, f)
+    llm = LLM(folder, dtype="float32", device="cpu", n_ctx=64, n_slots=1)
+    res = llm.generate([[1, 2, 3]], max_new=8, temp=0.0)
+    first = free.index(free[2])
+    assert res.tokens[0] == free[:first] and res.finish_reasons == ["stop"]
+    with open(folder + "/generation_config.json", "w") as f:
+        json.dump({"eos_token_id": 99999}, f)
+    from minfer_amd import ConfigError
+    with pytest.raises(ConfigError, match="eos_token_id"):
+        LLM(folder, dtype="float32", device="cpu", n_ctx=64, n_slots=1)

@@ -153,7 +153,16 @@ def test_command_line(folders, tmp_path):
     cfg.write_text(json.dumps(TINIES["B"]))
     r = subprocess.run(exe + ["--config", str(cfg), "--random-weights", "--prompt-tokens", "1,2,3", "--max-new", "4",
                               "--temp", "0.8", "--seed", "3"], capture_output=True, text=True, env=env, timeout=300)
-    assert r.returncode == 0 and len(r.stdout.strip().split(",")) <= 4, r.stderr
+    assert r.returncode == 0, r.stderr
+    # the same options through the Python entry point: the same random weights, the same draws
+    from minfer_amd import LLM
+    same = LLM.random(TINIES["B"], seed=0, dtype="bfloat16", n_ctx=4096, n_slots=1).generate(
+        [[1, 2, 3]], max_new=4, temp=0.8, seed=3)
+    assert [int(x) for x in r.stdout.strip().split(",") if x] == same.tokens[0] and 1 <= len(same.tokens[0]) <= 4
+    # ... and they are the weights of the folder that the same configuration and seed write
+    folder_b = write_tiny(tmp_path, "B", seed=0)
+    from_folder = LLM(folder_b, dtype="bfloat16", n_ctx=4096, n_slots=1).generate([[1, 2, 3]], max_new=4, temp=0.8, seed=3)
+    assert from_folder.tokens == same.tokens
     r = subprocess.run(exe + [folders["A"], "--bogus"], capture_output=True, text=True, env=env, timeout=60)
     assert r.returncode == 1 and "unknown option --bogus" in r.stderr and "USAGE" in r.stderr
     r = subprocess.run(exe + [folders["A"], "--prompt-tokens", "1", "--temp"], capture_output=True, text=True,

@@ -433,7 +433,7 @@ def prefill_case(nh, nk, hd, new, start, seed):
                            start_pos=torch.tensor(start, dtype=torch.int32, device=dev),
                            slot_ids=torch.zeros(len(new), dtype=torch.int32, device=dev), logit_rows=None,
                            page_tables={}, max_len=max(lengths), max_new=max(new), all_decode=False,
-                           host_slots=list(range(len(new))), host_new=list(new), host_start=list(start))
+                           host_new=list(new), host_start=list(start))
     return q, kc, stored_v(vc), table, ctx_on
 
 

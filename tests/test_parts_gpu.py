@@ -39,7 +39,7 @@ def context(cache, slots, new, start):
                        positions=pos.to(DEV), seq_of_tok=seq.to(DEV), cu_seqlens=cu.to(DEV),
                        start_pos=torch.tensor(start, dtype=torch.int32, device=DEV),
                        slot_ids=torch.tensor(slots, dtype=torch.int32, device=DEV), logit_rows=None, page_tables=tables,
-                       max_len=max_len, max_new=max(new), all_decode=all(n == 1 for n in new), host_slots=list(slots),
+                       max_len=max_len, max_new=max(new), all_decode=all(n == 1 for n in new),
                        host_new=list(new), host_start=list(start), new_lengths=new_len)
 
 
@@ -153,15 +153,18 @@ class ToyDecayMixer(Mixer):
         return StateRequest((self.hidden,), torch.float32)
 
     def forward(self, x, h, ctx, entry, writes_cache):
+        # the sequences' rows of the state are addressed by ctx.slot_ids, on the device: which
+        # slots they are is data, so a captured decode step works for any binding
         state = ctx.cache.state(entry)
+        ids = ctx.slot_ids.long()
+        s = state.index_select(0, ids)                    # [sequences][hidden]
         off = 0
-        for slot, n in zip(ctx.host_slots, ctx.host_new):
-            s = state[slot]
+        for b, n in enumerate(ctx.host_new):
             for t in range(off, off + n):
-                s = DECAY * s + x[t].float()
-                h[t] += self.w @ s
-            state[slot] = s
+                s[b] = DECAY * s[b] + x[t].float()
+                h[t] += self.w @ s[b]
             off += n
+        state.index_copy_(0, ids, s)
 
 
 class ToyConfig:
@@ -297,28 +300,16 @@ class ToyTop1Experts(FeedForward):
 
 @register_position("toy_position_bias")
 class ToyPositionBias(PositionEncoding):
-    """No rotation: position p adds p * slope to the first element of every q and k head."""
+    """No rotation: position p adds p * slope to the first element of every q and k head.  It
+    treats q and k and nothing else; where keys and values go is the cache's business."""
 
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
         self.head_dim, self.slope = int(spec.params["head_dim"]), float(spec.params["slope"])
 
-    def rotate_and_store(self, qkv, ctx, q_out, kcache, vcache, page_table, n_heads, n_kv_heads, write_kv):
-        t, hd = qkv.shape[0], self.head_dim
-        x = qkv.view(t, n_heads + 2 * n_kv_heads, hd).clone()
-        bump = ctx.positions.float() * self.slope
-        x[:, :n_heads + n_kv_heads, 0] += bump[:, None]
-        q_out.copy_(x[:, :n_heads].reshape(t, n_heads * hd).to(q_out.dtype))
-        if not write_kv:
-            return
-        pos = ctx.positions.long()
-        page = page_table.long()[ctx.seq_of_tok.long(), pos // 64]
-        k, v = x[:, n_heads:n_heads + n_kv_heads], x[:, n_heads + n_kv_heads:]
-        kcache[page, :, pos % 64, :] = k.to(kcache.dtype)
-        if vcache.dtype == torch.bfloat16:      # a bfloat16 page of V is [2][hd][32] (cache.paged.v_page_shape)
-            vcache[page, :, (pos % 64) // 32, :, pos % 32] = v.to(vcache.dtype)
-        else:
-            vcache[page, :, pos % 64, :] = v.to(vcache.dtype)
+    def encode(self, qkv, ctx, n_heads, n_kv_heads):
+        x = qkv.view(qkv.shape[0], n_heads + 2 * n_kv_heads, self.head_dim)
+        x[:, :n_heads + n_kv_heads, 0] += (ctx.positions.float() * self.slope)[:, None]
 
 
 @register_norm("toy_scale_norm")
@@ -418,3 +409,133 @@ def test_toy_routing_position_norm_and_block_parts(tmp_path):
     compare(run_steps(eng, whole_steps(requests)), ref, "float32", "routed whole")
     compare(run_steps(eng, tail_steps(requests, tail=8)), ref, "float32", "routed one by one")
     compare(run_steps(eng, batch_steps(requests, [ids[:3], ids[3:]])), ref, "float32", "routed batches")
+
+
+# ------------------------------------------------------------------ the toy state through the captured decode step
+@pytest.mark.parametrize("dtype", ["float32"])
+def test_toy_state_mixer_through_generate_with_a_captured_step(tmp_path, dtype):
+    """Two batches through `generate(use_graph=True)`: the second finds its sequences in other
+    slots than the ones the decode step was captured with.  Per-sequence state is addressed
+    through `ctx.slot_ids` only, so the replayed step reads and writes the right rows; greedy
+    tokens equal the plain model's."""
+    from minfer_amd import Engine, generate, load_model, register_architecture, write_random_model
+    from minfer_amd.sampling import SamplingParams
+    register_architecture("ToyStateLM", ToyConfig)
+    cfg = ToyConfig(dict(architectures=["ToyStateLM"], hidden_size=48, vocab_size=300))
+    folder = write_random_model(str(tmp_path / "toy"), cfg, seed=7)
+    eng = Engine(load_model(folder, dtype=dtype), max_tokens=64 * 8, max_seqs=5, poison_cache=True)
+    plain = PlainToy(folder)
+    prompts = [[int(t) for t in np.random.default_rng(40 + i).integers(0, 300, size=n)] for i, n in enumerate((4, 7, 5, 6))]
+
+    def expected(p, n):
+        seq, out = list(p), []
+        for _ in range(n):
+            out.append(pq.greedy(plain.forward(seq)[-1].astype(np.float32)))
+            seq.append(out[-1])
+        return out
+    want = [expected(p, 6) for p in prompts]
+    first = generate(eng, prompts[:2], SamplingParams.greedy(), max_new=6, stop_tokens=[], use_graph=True)
+    assert first.tokens == want[:2]
+    sessions = dict(eng._sessions)
+    assert len(sessions) == 1 and next(iter(sessions.values())).graph is not None
+    used = set(next(iter(sessions.values())).slots)
+    blockers = [eng.new_sequence() for _ in range(2)]              # take the slots that were just given back
+    second = generate(eng, prompts[2:], SamplingParams.greedy(), max_new=6, stop_tokens=[], use_graph=True)
+    session = next(iter(eng._sessions.values()))
+    assert dict(eng._sessions).keys() == sessions.keys(), "the same captured step served both batches"
+    assert set(session.slots) != used, "the second batch lives in other slots"
+    assert second.tokens == want[2:]
+    for s in blockers:
+        eng.end_sequence(s)
+    assert not eng.cache.live_slots()
+
+
+# ------------------------------------------------------------------ other ends of the model
+from minfer_amd.parts import Embedding, Head, register_embedding, register_head      # noqa: E402
+
+
+@register_embedding("toy_scaled_embedding")
+class ToyScaledEmbedding(Embedding):
+    """Rows of the table times a constant."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.vocab, self.hidden, self.scale = int(spec.params["vocab_size"]), int(spec.params["hidden_size"]), float(spec.params["scale"])
+
+    def tensor_specs(self):
+        return {"emb": TensorSpec((self.vocab, self.hidden))}
+
+    def load(self, get):
+        self.weight = get("emb").float()
+
+    def table(self):
+        return self.weight
+
+    def forward(self, token_ids, out):
+        out.copy_(self.weight[token_ids.long()] * self.scale)
+
+
+@register_head("toy_capped_head")
+class ToyCappedHead(Head):
+    """logits = cap * tanh((W x + b) / cap), W tied to the embedding table."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.vocab, self.cap = int(spec.params["vocab_size"]), float(spec.params["cap"])
+
+    def tensor_specs(self):
+        return {"head_bias": TensorSpec((self.vocab,))}
+
+    def load(self, get):
+        self.bias = get("head_bias").float()
+
+    def tie(self, embedding):
+        self.w = embedding.table()
+
+    def forward(self, x):
+        return (self.cap * torch.tanh((x.float() @ self.w.t() + self.bias) / self.cap)).contiguous()
+
+
+class ToyEndsConfig(ToyConfig):
+    def model_spec(self):
+        hid = self.hidden
+        norm = lambda n: PartSpec("rmsnorm", dict(size=hid, eps=1e-5, weight=n))
+        pos = PartSpec("rope_neox", dict(head_dim=16, theta=1e4, max_positions=256))
+        attn = PartSpec("gqa_attention", dict(hidden_size=hid, n_heads=2, n_kv_heads=2, head_dim=16, scale=0.25, window=None,
+                                              qkv_bias=False, out_bias=False, position=pos, q="a.q", k="a.k", v="a.v", o="a.o"))
+        ffn = PartSpec("swiglu", dict(hidden_size=hid, intermediate_size=40, gate="f.g", up="f.u", down="f.d"))
+        sizes = dict(vocab_size=self.vocab, hidden_size=hid)
+        return ModelSpec(hidden_size=hid, vocab_size=self.vocab, final_norm=norm("nf"),
+                         blocks=(BlockSpec("prenorm", "l0.", attn, ffn, norm("n1"), norm("n2")),),
+                         schedule=(RunEntry(0, 0),), max_positions=256,
+                         embedding=PartSpec("toy_scaled_embedding", dict(sizes, scale=3.0)),
+                         head=PartSpec("toy_capped_head", dict(sizes, cap=0.5)))
+
+
+def test_other_embedding_and_head_parts_without_touching_the_model(tmp_path):
+    """A scaled embedding and a capped, biased, tied head are registered parts; the model's step
+    is the same code."""
+    from minfer_amd import Engine, load_model, register_architecture, write_random_model
+    from safetensors.torch import load_file
+    register_architecture("ToyEndsLM", ToyEndsConfig)
+    cfg = ToyEndsConfig(dict(architectures=["ToyEndsLM"], hidden_size=32, vocab_size=150))
+    folder = write_random_model(str(tmp_path / "ends"), cfg, seed=9)
+    model = load_model(folder, dtype="float32")
+    assert set(model.expected_tensors()) >= {"emb", "head_bias", "nf"} and "lm_head.weight" not in model.expected_tensors()
+    w = {k: v.double().numpy() for k, v in load_file(folder + "/model.safetensors").items()}
+
+    def plain(tokens):
+        pos = np.arange(len(tokens))
+        h = w["emb"][tokens] * 3.0
+        x = pq.rms_norm(h, w["l0.n1"], 1e-5)
+        q = pq.rope_neox(pq.linear(x, w["l0.a.q.weight"]), pos, 2, 16, 1e4)
+        k = pq.rope_neox(pq.linear(x, w["l0.a.k.weight"]), pos, 2, 16, 1e4)
+        a = pq.gqa_attention(q, k, pq.linear(x, w["l0.a.v.weight"]), pos, pos, 2, 2, 16, 0.25)
+        h = h + pq.linear(a, w["l0.a.o.weight"])
+        h = h + pq.swiglu_ffn(pq.rms_norm(h, w["l0.n2"], 1e-5), w["l0.f.g.weight"], w["l0.f.u.weight"], w["l0.f.d.weight"])
+        return 0.5 * np.tanh((pq.rms_norm(h, w["nf"], 1e-5) @ w["emb"].T + w["head_bias"]) / 0.5)
+    eng = Engine(model, max_tokens=64 * 4, max_seqs=2, poison_cache=True)
+    requests = requests_for(150, (9, 70), seed=2)
+    ref = {r: plain(t) for r, t in requests.items()}
+    compare(run_steps(eng, whole_steps(requests)), ref, "float32", "toy ends whole")
+    compare(run_steps(eng, tail_steps(requests, tail=5)), ref, "float32", "toy ends one by one")

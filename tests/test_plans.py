@@ -70,3 +70,36 @@ def test_decode_split_plan_bounds():
         assert 1 <= n <= 32
         assert n == 1 or n * 256 <= max_len + 255
     assert ops.decode_split_plan(1, 4, 7, 32768) == 32 and ops.decode_split_plan(64, 4, 7, 32768) == 1
+
+
+def test_plan_linear_names_the_kernels_of_the_model_shapes():
+    """Which kernel a product takes, as the library decides it (nothing is launched): the decode
+    shapes of the 7B, 32B and 72B widths get the kernels the design describes, and widths off the
+    family's (896, 1024, 2560, 6144) a named path of their own."""
+    p = lambda *a, **k: ops.plan_linear(*a, n_cu=256, **k)["kernel"]
+    for h, inter, qkv in ((3584, 18944, 4608), (5120, 27648, 7168), (8192, 29568, 10240)):
+        for m in (1, 8, 16):
+            assert p(m, qkv, h, normed=True) == "stationary16_kernel(norm)"
+            assert p(m, 2 * inter, h, swiglu=True, normed=True) == "stationary16_kernel(norm)"
+            assert p(m, 152064, h, normed=True) == "stationary16_kernel(norm)"
+        assert p(8, h, h, accumulate=True) == ("stationary16_kernel" if h <= 5120 else "rolling16_kernel")
+        assert p(64, 2 * inter, h, swiglu=True) == "panel_kernel" and p(64, 152064, h) == "panel_kernel"
+        # the ring form needs K in whole chunks of 256 (29568 is 115.5 of them)
+        assert p(64, h, inter, accumulate=True) == ("skinny_ring_kernel" if inter % 256 == 0 else "skinny_kernel")
+        assert p(2048, 2 * inter, h, swiglu=True) == "tile_dma_kernel"
+        assert p(40, qkv, h, normed=True) == ""                       # no fold above 16 rows: norm, then product
+    assert p(8, 3584, 18944, accumulate=True) == "rolling16_kernel"
+    assert p(2048, 3584, 18944, accumulate=True) == "tile_dma_kernel(split K)"
+    assert p(200, 3584, 18944, accumulate=True) == "tile_kernel<128,128>(split K)"
+    # other widths: multiples of 256 that are instantiated take the register-resident kernel, the
+    # rest the rolling one; unaligned operands the guarded ones
+    for k in (1024, 2560, 3072, 6144, 7168):
+        assert p(4, 4096, k, normed=True) == "stationary16_kernel(norm)", k
+    assert p(4, 4096, 896, normed=True) == "" and p(4, 4096, 896) == "rolling16_kernel"
+    assert p(4, 4096, 1280) == "rolling16_kernel"                       # 5 x 256: not instantiated
+    assert p(4, 4096, 900, aligned=False) == "skinny16_kernel"
+    assert p(4, 100, 1024) == "rolling16_kernel"                        # too few weight rows to go round
+    assert p(30, 4096, 900, aligned=False) == "skinny_kernel"
+    for ns in ops.STATIONARY_NS:
+        assert ops.stationary_shape(4096, 256 * ns, True) and p(2, 4096, 256 * ns, normed=True) != ""
+    assert not ops.stationary_shape(4096, 256 * 5) and not ops.stationary_shape(4096, 256 * 33, True)

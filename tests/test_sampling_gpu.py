@@ -4,10 +4,15 @@ import pytest
 import torch
 
 import plain_qwen2 as pq
-from minfer_amd.sampling import Sampler, SamplingParams, uniform
+from minfer_amd.sampling import Sampler, SamplingParams, stream_i64, uniform
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
+
+
+def streams_of(seed, keys):
+    """Stream ids (seed and key folded on the host) as the int64 tensor the kernels read."""
+    return torch.tensor([stream_i64(seed, k) for k in keys], dtype=torch.int64, device=DEV)
 
 
 @pytest.fixture(scope="module")
@@ -93,7 +98,7 @@ def test_temperature_draw_matches_plain(ops, vocab, temp):
     out = torch.empty(rows, dtype=torch.int32, device=DEV)
     keys = torch.zeros(rows, dtype=torch.int64, device=DEV)
     steps = torch.zeros(rows, dtype=torch.int32, device=DEV)
-    ops.sample(l.to(DEV), temp, 0, keys, steps, out, torch.from_numpy(rs).to(DEV))
+    ops.sample(l.to(DEV), temp, keys, steps, out, torch.from_numpy(rs).to(DEV))
     for i in range(rows):
         probs = pq.temperature_probs(l[i].numpy(), temp)
         # the kernel keeps the running sum in double; so does the oracle for a large vocabulary
@@ -107,7 +112,7 @@ def test_temperature_draw_matches_plain(ops, vocab, temp):
     m = torch.full((1, 50), float("-inf"))
     m[0, 7] = m[0, 31] = 1.0
     for r, want in ((0.0, 7), (0.49, 7), (0.51, 31), (0.999, 31)):
-        ops.sample(m.to(DEV), 1.0, 0, keys[:1], steps[:1], out[:1], torch.tensor([r], device=DEV))
+        ops.sample(m.to(DEV), 1.0, keys[:1], steps[:1], out[:1], torch.tensor([r], device=DEV))
         assert out[0].item() == want
 
 
@@ -133,11 +138,11 @@ def test_sample_filtered_is_top_k_top_p_and_the_draw(ops, rows, vocab, k, p, tem
     want = torch.empty(rows, dtype=torch.int32, device=DEV)
     ops.top_k(chain, k)
     ops.top_p(chain, p)
-    ops.sample(chain, temp, 0, keys, steps, want, forced)
+    ops.sample(chain, temp, keys, steps, want, forced)
     d = l.to(DEV).clone()
     got = torch.empty(rows, dtype=torch.int32, device=DEV)
     assert ops.sample_filtered_takes(vocab, k, temp)
-    ops.sample_filtered(d, k, p, temp, 0, keys, steps, got, forced)
+    ops.sample_filtered(d, k, p, temp, keys, steps, got, forced)
     assert got.cpu().tolist() == want.cpu().tolist()
     untouched = [i for i in range(rows) if i != 3]
     assert torch.equal(d[untouched].cpu(), l[untouched])
@@ -149,23 +154,23 @@ def test_sample_filtered_is_top_k_top_p_and_the_draw(ops, rows, vocab, k, p, tem
         if i != 4:
             assert int(got[i]) == pq.sample(l[i].numpy(), temp, float(rs[i]), k, p, 1.0, 0.0, 0.0, [])
     # without forced draws: the generator's uniform, as `sample` takes it
-    keys = torch.arange(rows, dtype=torch.int64, device=DEV) + 5
+    keys = streams_of(77, range(5, rows + 5))
     steps = torch.arange(rows, dtype=torch.int32, device=DEV)
     chain = l.to(DEV).clone()
     ops.top_k(chain, k)
     ops.top_p(chain, p)
-    ops.sample(chain, temp, 77, keys, steps, want)
-    ops.sample_filtered(l.to(DEV).clone(), k, p, temp, 77, keys, steps, got)
+    ops.sample(chain, temp, keys, steps, want)
+    ops.sample_filtered(l.to(DEV).clone(), k, p, temp, keys, steps, got)
     assert got.cpu().tolist() == want.cpu().tolist()
 
 
 def test_device_uniform_is_the_host_uniform_and_draws_follow_softmax(ops):
     rows, vocab = 4000, 3
     small = torch.tensor([0.0, 1.0, 2.0]).repeat(rows, 1).to(DEV)
-    keys = torch.arange(rows, dtype=torch.int64, device=DEV)
+    keys = streams_of(42, range(rows))
     steps = (torch.arange(rows, dtype=torch.int32, device=DEV) % 7)
     out = torch.empty(rows, dtype=torch.int32, device=DEV)
-    ops.sample(small, 1.0, 42, keys, steps, out)
+    ops.sample(small, 1.0, keys, steps, out)
     probs = pq.temperature_probs(np.array([0, 1, 2], dtype=np.float32), 1.0)
     want = [pq.sample_from_probs(probs, uniform(42, i, i % 7)) for i in range(rows)]
     assert out.cpu().tolist() == want
@@ -191,7 +196,8 @@ def test_pipeline_order_and_greedy_with_penalty():
         w[0] = int(torch.argmax(base[i]))                  # penalise the favourite
         prev[i, :20] = torch.tensor(w)
     out = torch.empty(rows, dtype=torch.int32, device=DEV)
-    Sampler(params)(base.to(DEV).clone(), torch.arange(rows, dtype=torch.int64, device=DEV),
+    sampler = Sampler(params)
+    sampler(base.to(DEV).clone(), torch.tensor(sampler.streams(range(rows)), dtype=torch.int64, device=DEV),
                     torch.full((rows,), 3, dtype=torch.int32, device=DEV), out, prev.to(DEV),
                     torch.full((rows,), 20, dtype=torch.int32, device=DEV))
     want = [pq.sample(base[i].numpy(), 0.7, uniform(9, i, 3), 40, 0.9, 1.3, 0.2, 0.1, windows[i]) for i in range(rows)]

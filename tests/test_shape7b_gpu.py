@@ -1,20 +1,41 @@
-"""One layer at the widths of Qwen2.5-7B (hidden 3584, 28 heads over 4 kv heads of 128,
-feed-forward 18944, vocabulary 152064) with random weights: 32-bit logits against the plain
-implementation under the three ways of cutting, and bfloat16 within its tolerance.  The
-sums here are as long as in the full model (18944 terms in the down product)."""
+"""The widths of Qwen2.5-7B (hidden 3584, 28 heads over 4 kv heads of 128, feed-forward 18944,
+vocabulary 152064) with random weights against the plain implementation in 64 bits:
+
+* four layers with an untied head (of the model's 28: the plain implementation's time and the
+  4 GB folder bound the depth), 32-bit logits within 1e-4 and bfloat16 within the suite's bound
+  under all the ways of cutting requests into steps;
+* one layer with a tied head, the same, and a batch of twenty;
+* a context of 2,150 tokens whose last tokens are decoded one by one through the captured decode
+  step (key splits and their merge in bfloat16), with weights made so that the one key that
+  matters lies 1,400 positions back;
+* one layer at the 72B widths in 32 bits.
+"""
 import numpy as np
 import pytest
 
 from plain_qwen2 import PlainQwen2
-from replays import batch_steps, compare, plain_logits, requests_for, run_steps, tail_steps, whole_steps
+from replays import (batch_steps, chunk_steps, compare, plain_logits, requests_for, run_steps, tail_steps,
+                     whole_steps)
 
 pytestmark = pytest.mark.gpu
 
-SHAPE_7B_ONE_LAYER = dict(
+WIDTHS_7B = dict(
     architectures=["Qwen2ForCausalLM"], model_type="qwen2", hidden_act="silu",
-    num_hidden_layers=1, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+    hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
     intermediate_size=18944, vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-6,
-    max_position_embeddings=32768, tie_word_embeddings=True, use_sliding_window=False)
+    max_position_embeddings=32768, use_sliding_window=False)
+SHAPE_7B_ONE_LAYER = dict(WIDTHS_7B, num_hidden_layers=1, tie_word_embeddings=True)
+SHAPE_7B_FOUR_LAYERS = dict(WIDTHS_7B, num_hidden_layers=4, tie_word_embeddings=False)
+
+
+def all_replays(eng, reqs, ref, dtype, what, layers, tail=8):
+    ids = list(reqs)
+    halves = [ids[:3], ids[3:]]
+    return max(compare(run_steps(eng, whole_steps(reqs)), ref, dtype, f"{what} whole", layers),
+               compare(run_steps(eng, tail_steps(reqs, tail=tail)), ref, dtype, f"{what} one by one", layers),
+               compare(run_steps(eng, batch_steps(reqs, halves)), ref, dtype, f"{what} batches", layers),
+               compare(run_steps(eng, chunk_steps(reqs, halves, sizes=(2, 17, 1, 5))), ref, dtype,
+                       f"{what} portions", layers))
 
 
 @pytest.fixture(scope="module")
@@ -34,11 +55,8 @@ def reference(folder):
 def test_one_layer_at_7b_widths(folder, reference, dtype):
     from minfer_amd import Engine, load_model
     reqs, ref = reference
-    ids = list(reqs)
     eng = Engine(load_model(folder, dtype=dtype), max_tokens=64 * 4, poison_cache=True)
-    worst = max(compare(run_steps(eng, whole_steps(reqs)), ref, dtype, "7B widths whole"),
-                compare(run_steps(eng, tail_steps(reqs, tail=8)), ref, dtype, "7B widths one by one"),
-                compare(run_steps(eng, batch_steps(reqs, [ids[:3], ids[3:]])), ref, dtype, "7B widths batches"))
+    worst = all_replays(eng, reqs, ref, dtype, "7B widths", layers=1)
     print(f"{dtype}: worst abs err {worst:.3e}")
 
 
@@ -57,6 +75,113 @@ def test_batch_of_twenty_at_7b_widths(folder):
     print(f"worst abs err {worst:.3e}")
 
 
+# ------------------------------------------------------------------ four layers, untied head
+@pytest.fixture(scope="module")
+def folder4(tmp_path_factory):
+    from minfer_amd import config_from_dict, write_random_model
+    return write_random_model(str(tmp_path_factory.mktemp("shape7b4") / "m"), config_from_dict(SHAPE_7B_FOUR_LAYERS),
+                              seed=15)
+
+
+@pytest.fixture(scope="module")
+def reference4(folder4):
+    plain = PlainQwen2.from_folder(folder4, dtype=np.float64)
+    reqs = requests_for(152064, (3, 20, 9, 33, 6), seed=16)
+    ref = plain_logits(plain, reqs)
+    del plain
+    return reqs, ref
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_four_layers_untied_head_at_7b_widths(folder4, reference4, dtype):
+    """4 of the model's 28 layers, every width and the vocabulary as in the model, lm_head a
+    tensor of its own: 32-bit logits within 1e-4 of the plain implementation, bfloat16 within the
+    bound for this depth, whole, one by one, in unequal batches and with prompts in portions."""
+    from minfer_amd import Engine, load_model
+    reqs, ref = reference4
+    model = load_model(folder4, dtype=dtype)
+    assert model.head.weight.data_ptr() != model.embedding.weight.data_ptr() and len(model.blocks) == 4
+    eng = Engine(model, max_tokens=64 * 4, poison_cache=True)
+    worst = all_replays(eng, reqs, ref, dtype, "7B widths, 4 layers, untied", layers=4)
+    print(f"{dtype}: worst abs err {worst:.3e} (logit std {float(ref['r1'].std()):.3f})")
+
+
+# ------------------------------------------------------------------ a long context through the captured decode step
+NEEDLE_KEY, NEEDLE_QUERY, NEEDLE_AT, CONTEXT, TAIL = 4242, 9797, 700, 2150, 8
+
+
+@pytest.fixture(scope="module")
+def needle(tmp_path_factory):
+    """One layer at the 7B widths whose q and k matrices are given a strong response, in the head
+    dimensions that rotate slowest, to the embeddings of two tokens: a query made from token
+    NEEDLE_QUERY scores about 20 against the key of token NEEDLE_KEY wherever it lies, against
+    about 1 for any other key.  The request holds NEEDLE_KEY once, at position 700, and ends in
+    NEEDLE_QUERY tokens: what attention returns for them is the value row stored 1,400 positions
+    earlier, in the second of the eight key splits of the bfloat16 decode kernel."""
+    import torch
+    from safetensors.torch import load_file, save_file
+    from minfer_amd import config_from_dict, write_random_model
+    folder = write_random_model(str(tmp_path_factory.mktemp("needle") / "m"), config_from_dict(SHAPE_7B_ONE_LAYER), seed=25)
+    path = folder + "/model.safetensors"
+    t = load_file(path)
+    emb = t["model.embed_tokens.weight"].float()
+    unit = lambda tok: emb[tok] / emb[tok].norm()
+    hd, alpha = 128, 0.25
+    slow = [h * hd + i for h in range(28) for i in (hd // 2 - 1, hd - 1)]          # the slowest pair of every q head
+    slow_k = [h * hd + i for h in range(4) for i in (hd // 2 - 1, hd - 1)]
+    q = t["model.layers.0.self_attn.q_proj.weight"].float()
+    k = t["model.layers.0.self_attn.k_proj.weight"].float()
+    q[slow] += alpha * unit(NEEDLE_QUERY)
+    k[slow_k] += alpha * unit(NEEDLE_KEY)
+    t["model.layers.0.self_attn.q_proj.weight"] = q.to(torch.bfloat16)
+    t["model.layers.0.self_attn.k_proj.weight"] = k.to(torch.bfloat16)
+    save_file(t, path)
+    rng = np.random.default_rng(31)
+    tokens = [int(x) for x in rng.integers(0, 152064, size=CONTEXT)]
+    tokens = [x if x not in (NEEDLE_KEY, NEEDLE_QUERY) else 11 for x in tokens]
+    tokens[NEEDLE_AT] = NEEDLE_KEY
+    for p in range(CONTEXT - TAIL - 1, CONTEXT):
+        tokens[p] = NEEDLE_QUERY if (p % 3) else tokens[p]              # most of the tail asks for the needle
+    plain = PlainQwen2.from_folder(folder, dtype=np.float64)
+    hidden = plain.hidden(tokens)
+    ref = plain.head(hidden[CONTEXT - TAIL:])
+    # the plain model itself confirms the construction: without the needle's key the rows differ widely
+    other = list(tokens)
+    other[NEEDLE_AT] = 12
+    moved = plain.head(plain.hidden(other)[CONTEXT - TAIL:])
+    assert np.abs(moved - ref).max() > 20 * 0.055 * ref.std(), "the far key does not matter enough for this test"
+    return folder, tokens, ref
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_context_through_the_captured_decode_step(needle, dtype):
+    """2,142 tokens in one step, then the last 8 one by one through `DecodeSession` (eager once,
+    captured once, then replayed), each step's logits against the plain implementation."""
+    import torch
+    from minfer_amd import Engine, load_model
+    from minfer_amd.kernels import ops
+    from minfer_amd.sampling import Sampler, SamplingParams
+    folder, tokens, ref = needle
+    eng = Engine(load_model(folder, dtype=dtype), max_tokens=64 * 40, max_seqs=2, poison_cache=True)
+    if dtype == "bfloat16":
+        assert ops.decode_split_plan(1, 4, 7, 2304) >= 8, "the decode attention splits the keys here"
+    slot = eng.new_sequence()
+    head = CONTEXT - TAIL
+    eng.step([slot], [tokens[:head]], [[]])
+    session = eng.decode_session(1, CONTEXT + 8, Sampler(SamplingParams.greedy()), use_graph=True)
+    session.bind([slot], [tokens[head]], [0], [0])
+    rows = {}
+    for i in range(TAIL):
+        if i:
+            session.token_ids.copy_(torch.tensor([tokens[head + i]], dtype=torch.int32))    # the given token, not the sampled one
+        session.step()
+        rows[("needle", i)] = session.last_logits[0].cpu().numpy().copy()
+    assert session.graph is not None and eng.length(slot) == CONTEXT
+    eng.end_sequence(slot)
+    worst = compare(rows, {"needle": ref}, dtype, "long context, captured decode step")
+    print(f"{dtype}: worst abs err {worst:.3e}")
+
+
 SHAPE_72B_ONE_LAYER = dict(
     architectures=["Qwen2ForCausalLM"], model_type="qwen2", hidden_act="silu",
     num_hidden_layers=1, hidden_size=8192, num_attention_heads=64, num_key_value_heads=8,
@@ -66,7 +191,7 @@ SHAPE_72B_ONE_LAYER = dict(
 
 def test_one_layer_at_72b_widths_in_32_bits(tmp_path_factory):
     """Hidden 8192 and feed-forward 29568 (a small vocabulary keeps the folder small) in the
-    32-bit path: sums of up to 29568 terms, 64 heads over 8 kv heads, under the three ways of
+    32-bit path: sums of up to 29568 terms, 64 heads over 8 kv heads, under the ways of
     cutting.  (The bfloat16 kernels for K of 5120 and 8192 are checked one by one in
     test_kernels_gpu.py against references with the same rounded inputs; a bfloat16 run at
     these widths differs from the 64-bit plain implementation by about 1 % of the logits'
@@ -80,9 +205,6 @@ def test_one_layer_at_72b_widths_in_32_bits(tmp_path_factory):
     plain = PlainQwen2.from_folder(folder, dtype=np.float64)
     reqs = requests_for(3000, (3, 20, 9, 37), seed=9)
     ref = plain_logits(plain, reqs)
-    ids = list(reqs)
     eng = Engine(load_model(folder, dtype=dtype), max_tokens=64 * 4, poison_cache=True)
-    worst = max(compare(run_steps(eng, whole_steps(reqs)), ref, dtype, "72B widths whole"),
-                compare(run_steps(eng, tail_steps(reqs, tail=8)), ref, dtype, "72B widths one by one"),
-                compare(run_steps(eng, batch_steps(reqs, [ids[:3], ids[3:]])), ref, dtype, "72B widths batches"))
+    worst = all_replays(eng, reqs, ref, dtype, "72B widths", layers=1)
     print(f"{dtype}: worst abs err {worst:.3e}")
