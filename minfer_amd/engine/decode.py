@@ -11,6 +11,8 @@ and it may start the next step before it has read them (`launch` / `collect`).
 """
 from __future__ import annotations
 
+import gc
+import weakref
 from typing import Dict, List, Optional, Sequence
 
 import torch
@@ -30,7 +32,11 @@ class DecodeSession:
     sampling options other than the seed."""
 
     def __init__(self, engine, n_seqs: int, max_len: int, sampler, use_graph: bool = True):
-        self.engine, self.n, self.sampler = engine, n_seqs, sampler
+        # the engine owns its sessions; the way back is a weak reference, so that an engine that
+        # goes out of use is freed at once, with its graphs, and not whenever the collector of
+        # reference cycles happens to run (which may be in the middle of another capture)
+        self._engine = weakref.ref(engine)
+        self.n, self.sampler = n_seqs, sampler
         self.max_len = max_len
         self.n_cols = (max_len + PAGE - 1) // PAGE
         self.use_graph = use_graph and engine.device.type == "cuda" and not tuning.DEBUG_SYNC
@@ -63,6 +69,13 @@ class DecodeSession:
         self.slots: List[int] = []
         self._host_tables: Dict[int, List[List[int]]] = {}
         engine.model.prepare(max_len)
+
+    @property
+    def engine(self):
+        engine = self._engine()
+        if engine is None:
+            raise RuntimeError("the engine of this decode session is gone")
+        return engine
 
     # ------------------------------------------------------------ binding
     def abandon(self) -> None:
@@ -164,8 +177,14 @@ class DecodeSession:
             self.warm = True
         else:
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                self._run()
+            collecting = gc.isenabled()
+            gc.disable()                     # nothing may be freed on the device while the stream is captured
+            try:
+                with torch.cuda.graph(graph):
+                    self._run()
+            finally:
+                if collecting:
+                    gc.enable()
             self.graph = graph
             self._graph_generation = ops.workspace_generation()
             graph.replay()
