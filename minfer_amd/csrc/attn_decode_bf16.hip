@@ -28,6 +28,7 @@
 // length, so every split has work.  With several splits each block writes an unnormalised
 // partial (acc, max, sum) and attn_combine_kernel merges them in a fixed order.
 #include "attn_tokens_impl.h"
+#include "noalloc.h"
 
 namespace {
 
@@ -403,4 +404,53 @@ MF_API int mf_attn_decode_rope_bf16(const float* qkv, const float* cs, const flo
   const RopeArgs rope{qkv, cs, sn, write_kv};
   return dispatch(nullptr, kc, vt, page_table, pt_stride, positions, seq_of_tok, out, part, n_tok, nh, nk, hd,
                   scale, window, n_splits, &rope, stream);
+}
+
+// ------------------------------------------------------------------ the entry point that allocates nothing
+// (see noalloc.h)
+namespace {
+
+// The partials of the key splits.  In host code this name is only a handle for the runtime: the
+// memory's address on a device comes from hipGetSymbolAddress, once per device, below.
+static __device__ __align__(256) float scratch[MF_NOALLOC_SCRATCH_FLOATS];
+
+constexpr int MAX_DEVICES = 64;
+float* scratch_on_device[MAX_DEVICES] = {};      // each GPU holds its own copy of the array, at its own address
+
+// the array's address on the current device; nullptr and `rc` set on failure
+float* scratch_address(int* rc) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { *rc = (int)e; return nullptr; }
+  if (dev < 0 || dev >= MAX_DEVICES) { *rc = (int)hipErrorInvalidDevice; return nullptr; }
+  float* p = __atomic_load_n(&scratch_on_device[dev], __ATOMIC_ACQUIRE);
+  if (p) return p;
+  void* addr = nullptr;
+  e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !addr) { *rc = e != hipSuccess ? (int)e : (int)hipErrorUnknown; return nullptr; }
+  p = (float*)addr;
+  __atomic_store_n(&scratch_on_device[dev], p, __ATOMIC_RELEASE);    // two first calls at once store the same address
+  return p;
+}
+
+}  // namespace
+
+MF_API size_t mf_attn_decode_bf16_noalloc_capacity(void) { return MF_NOALLOC_SCRATCH_FLOATS; }
+
+MF_API int mf_attn_decode_bf16_noalloc(const void* q, const void* kc, const void* vt, const int* page_table,
+                                       int pt_stride, const int* positions, const int* seq_of_tok, void* out,
+                                       int n_tok, int nh, int nk, int hd, float scale, int window, int n_splits,
+                                       hipStream_t stream) {
+  if (n_tok <= 0) return 0;
+  if (n_splits < 1 || n_splits > 64 || nh <= 0 || hd <= 0) return (int)hipErrorInvalidValue;
+  float* part = nullptr;
+  if (n_splits > 1) {
+    const size_t need = (size_t)n_tok * (size_t)nh * (size_t)n_splits * (size_t)(hd + 2);
+    if (need > MF_NOALLOC_SCRATCH_FLOATS) return MF_NOALLOC_TOO_LARGE;
+    int rc = 0;
+    part = scratch_address(&rc);
+    if (!part) return rc;
+  }
+  return dispatch(q, const_cast<void*>(kc), const_cast<void*>(vt), page_table, pt_stride, positions, seq_of_tok,
+                  out, part, n_tok, nh, nk, hd, scale, window, n_splits, nullptr, stream);
 }

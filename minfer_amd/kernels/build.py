@@ -35,7 +35,7 @@ LIBRARIES: Dict[str, str] = {
 HEADERS = {"host_random": ["random_normal.h"],
            "elementwise": ["common.h", "random_normal.h"],
            "attn_tokens_f32": ["common.h", "attn_tokens_impl.h"],
-           "attn_decode_bf16": ["common.h", "attn_tokens_impl.h"]}
+           "attn_decode_bf16": ["common.h", "attn_tokens_impl.h", "noalloc.h"]}
 
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-shared", "-std=c++17",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
