@@ -1,0 +1,74 @@
+// Two measuring kernels for the benchmark: what this GPU gives a plain streaming read, and what its
+// matrix cores give a loop of bfloat16 products that never leaves the registers.  They price the
+// roofline fractions that the benchmark reports next to the published peaks.  Neither is on the
+// path of a model's step.
+#include "common.h"
+
+namespace {
+
+// Every lane reads 16 bytes at a time, a block walks contiguous kilobytes, the grid strides over
+// the buffer; the loaded values are folded into one word per block so that the loads stay.
+__global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict__ src, size_t n16,
+                                                         unsigned* __restrict__ sink) {
+  unsigned acc = 0;
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+    acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+  }
+  for (; i < n16; i += stride) {
+    const uint4 a = src[i];
+    acc ^= a.x ^ a.y ^ a.z ^ a.w;
+  }
+  if (acc == 0x9E3779B9u) sink[blockIdx.x] = acc;      // (practically never: the store keeps the loads alive)
+}
+
+// 8 waves a block, each 2 x 4 independent 32x32x16 products per round from operands held in
+// registers (128 accumulator registers a wave): no memory traffic at all.
+__global__ __launch_bounds__(512) void probe_mfma_kernel(int rounds, float* __restrict__ sink) {
+  bf16x8 a[2], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    a[i & 1] = bf16x8{(bf16)(threadIdx.x * 0.001f + i), 1, 2, 3, 4, 5, 6, 7};
+    b[i] = bf16x8{(bf16)(blockIdx.x * 0.002f + i), 7, 6, 5, 4, 3, 2, 1};
+  }
+  floatx16 acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  for (int it = 0; it < rounds; ++it) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s += acc[i][j][r];
+  if (s == 123.456f) sink[blockIdx.x] = s;
+}
+
+}  // namespace
+
+// Reads `bytes` (a multiple of 16) from src once with `blocks` blocks; sink holds `blocks` words.
+MF_API int mf_probe_read(const void* src, size_t bytes, void* sink, int blocks, hipStream_t stream) {
+  if (bytes < 16 || blocks <= 0 || (uintptr_t)src % 16 != 0) return (int)hipErrorInvalidValue;
+  probe_read_kernel<<<blocks, 256, 0, stream>>>((const uint4*)src, bytes / 16, (unsigned*)sink);
+  return mf_launch_status();
+}
+
+// `blocks` blocks of 8 waves run `rounds` rounds of 8 products of 32 x 32 x 16 each:
+// blocks * 8 * rounds * 8 * 2 * 32 * 32 * 16 floating-point operations.
+MF_API int mf_probe_mfma(int rounds, void* sink, int blocks, hipStream_t stream) {
+  if (rounds <= 0 || blocks <= 0) return (int)hipErrorInvalidValue;
+  probe_mfma_kernel<<<blocks, 512, 0, stream>>>(rounds, (float*)sink);
+  return mf_launch_status();
+}

@@ -31,6 +31,7 @@ LIBRARIES: Dict[str, str] = {
     "attn_decode_bf16": "attn_decode_bf16.hip",
     "attn_prefill_bf16": "attn_prefill_bf16.hip",
     "sampling": "sampling.hip",
+    "probe": "probe.hip",
 }
 HEADERS = {"host_random": ["random_normal.h"],
            "elementwise": ["common.h", "random_normal.h"],

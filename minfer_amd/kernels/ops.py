@@ -39,6 +39,10 @@ _PROTOTYPES = {
         "mf_rope_inplace": [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
         "mf_fill_normal": [_P, c_int, c_size_t, c_uint64, c_float, c_int, _P],
     },
+    "probe": {
+        "mf_probe_read": [_P, c_size_t, _P, c_int, _P],
+        "mf_probe_mfma": [c_int, _P, c_int, _P],
+    },
     "host_random": {
         "mf_fill_normal_host": [_P, c_int, c_size_t, c_uint64, c_float, c_int, c_int],
     },
@@ -103,6 +107,10 @@ def _check(rc: int, what: str) -> None:
     if rc != 0:
         raise KernelError(f"{what}: HIP error {rc}"
                           + (" (invalid argument: a size the kernel does not take)" if rc == 1 else ""))
+    if _trace is not None:
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        _trace.append((what, ev))
     if tuning.DEBUG_SYNC and not torch.cuda.is_current_stream_capturing():
         try:
             torch.cuda.current_stream().synchronize()
@@ -113,6 +121,30 @@ def _check(rc: int, what: str) -> None:
 
 def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
     return c_void_p(0 if t is None else t.data_ptr())
+
+
+# ------------------------------------------------------------------ per-launch timing
+_trace: Optional[list] = None
+
+
+def start_trace() -> None:
+    """From here on every launch is followed by an event on the stream; `stop_trace` turns them
+    into (launch name, microseconds) pairs.  The time of a launch is the time between the event
+    behind the launch before it and its own, so the GPU must not run dry in between: queue
+    enough work first (`probe_mfma`) that the host stays ahead."""
+    global _trace
+    first = torch.cuda.Event(enable_timing=True)
+    first.record()
+    _trace = [("", first)]
+
+
+def stop_trace():
+    global _trace
+    events, _trace = _trace or [], None
+    if len(events) < 2:
+        return []
+    events[-1][1].synchronize()
+    return [(name, events[i - 1][1].elapsed_time(ev) * 1e3) for i, (name, ev) in enumerate(events) if i]
 
 
 def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
@@ -435,7 +467,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
     if x.dtype == torch.float32:
         _need(out, "linear.out", torch.float32)
         _check(_fn("gemm_f32", "mf_gemm_f32")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n, m,
-                                               n, k, 1 if accumulate else 0, _stream()), "gemm_f32")
+                                               n, k, 1 if accumulate else 0, _stream()), f"gemm_f32 {m}x{n}x{k}")
         return
     if accumulate and out.dtype != torch.float32:
         raise KernelError("linear: accumulation needs a float32 output")
@@ -446,7 +478,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
         part = workspace("skinny", splits * m * n, x.device) if splits > 1 else None
         _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(bias),
                                                         _ptr(out), n, _ptr(part), m, n, k, splits, per,
-                                                        epi, _stream()), "gemm_bf16_skinny")
+                                                        epi, _stream()), f"gemm_bf16_skinny {m}x{n}x{k}")
         return
     if variant == 0:
         splits, per, big = _k_split(m, n, k, False, aligned)
@@ -454,10 +486,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
             part = workspace("skinny", splits * m * n, x.device)
             _check(_fn("gemm_bf16", "mf_gemm_bf16_splitk")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n,
                                                             _ptr(part), m, n, k, splits, per, epi, 1 if big else 0,
-                                                            _stream()), "gemm_bf16_splitk")
+                                                            _stream()), f"gemm_bf16_splitk {m}x{n}x{k}")
             return
     _check(_fn("gemm_bf16", "mf_gemm_bf16")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n, m,
-                                             n, k, epi, variant, _stream()), "gemm_bf16")
+                                             n, k, epi, variant, _stream()), f"gemm_bf16 {m}x{n}x{k}")
 
 
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
@@ -491,7 +523,7 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, vari
         part = workspace("skinny", splits * m * n, x.device) if m > 16 or splits > 1 else None
         _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
                                                         _ptr(part), m, n, k, splits, per, EPI_SWIGLU, _stream()),
-               "gemm_bf16_skinny(swiglu)")
+               f"gemm_bf16_skinny(swiglu) {m}x{n}x{k}")
         return
     if variant == 0:
         splits, per, big = _k_split(m, n, k, True, aligned)
@@ -499,10 +531,10 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, vari
             part = workspace("skinny", splits * m * n, x.device)
             _check(_fn("gemm_bf16", "mf_gemm_bf16_splitk")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
                                                             _ptr(part), m, n, k, splits, per, EPI_SWIGLU, 0,
-                                                            _stream()), "gemm_bf16_splitk(swiglu)")
+                                                            _stream()), f"gemm_bf16_splitk(swiglu) {m}x{n}x{k}")
             return
     _check(_fn("gemm_bf16", "mf_gemm_bf16")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf, m, n, k,
-                                             EPI_SWIGLU, variant, _stream()), "gemm_bf16(swiglu)")
+                                             EPI_SWIGLU, variant, _stream()), f"gemm_bf16(swiglu) {m}x{n}x{k}")
 
 
 NOT_BUILT = -2      # an entry point's answer for a shape it has no kernel for; nothing was launched
@@ -549,7 +581,7 @@ def linear_normed(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, row_id
                                                  _stream())
     if rc == NOT_BUILT:
         return False
-    _check(rc, "gemm_bf16_normed")
+    _check(rc, f"gemm_bf16_normed{'(swiglu)' if swiglu else ''} {m}x{n}x{k}")
     return True
 
 
@@ -794,3 +826,23 @@ def advance(next_ids: torch.Tensor, sampled: torch.Tensor, positions: torch.Tens
     _check(_fn("sampling", "mf_advance")(_ptr(next_ids), _ptr(sampled), _ptr(positions), _ptr(steps), n,
                                           _ptr(prev), max_prev, _ptr(n_prev if prev is not None else None),
                                           _ptr(cursor if prev is not None else None), _stream()), "advance")
+
+
+# ------------------------------------------------------------------ measuring kernels
+def probe_read(buffer: torch.Tensor, blocks: Optional[int] = None) -> None:
+    """Launches one plain streaming read of the whole buffer (for the benchmark's measured
+    memory bandwidth; time it from outside)."""
+    _need(buffer, "probe_read.buffer")
+    nbytes = buffer.numel() * buffer.element_size() // 16 * 16
+    blocks = blocks or cu_count() * 8
+    sink = workspace("probe", blocks, buffer.device)
+    _check(_fn("probe", "mf_probe_read")(_ptr(buffer), nbytes, _ptr(sink), blocks, _stream()), "probe_read")
+
+
+def probe_mfma(rounds: int, blocks: Optional[int] = None, device="cuda") -> float:
+    """Launches a register-resident loop of bfloat16 matrix-core products and returns the number
+    of floating-point operations it performs (time it from outside)."""
+    blocks = blocks or cu_count()
+    sink = workspace("probe", blocks, device)
+    _check(_fn("probe", "mf_probe_mfma")(int(rounds), _ptr(sink), blocks, _stream()), "probe_mfma")
+    return float(blocks) * 8 * rounds * 8 * 2 * 32 * 32 * 16

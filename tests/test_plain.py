@@ -278,3 +278,70 @@ def test_uniform_stream():
     assert all(0.0 <= x < 1.0 for x in u) and abs(np.mean(u) - 0.5) < 0.03 and len(set(u)) > 1990
     assert uniform(42, 0, 5) == uniform(42, 0, 5) != uniform(42, 1, 5) != uniform(43, 0, 5)
     assert all(float(np.float32(x)) == x for x in u[:50])            # exact in float32
+
+
+# ------------------------------------------------------------------ how the parts are put together
+def with_random_gains(m, seed):
+    """The same model with norm gains that are not one, so that where a norm stands shows."""
+    w = dict(m.w)
+    for n in w:
+        if n.endswith("layernorm.weight") or n == "model.norm.weight":
+            w[n] = 1.0 + 0.5 * rnd(*w[n].shape, seed=seed + len(n))
+    return pq.PlainQwen2(m.c, w)
+
+
+@pytest.mark.parametrize("name", list(TINIES))
+def test_whole_model_equals_a_composition_of_library_routines(models, name):
+    """The model once more, put together from torch's own routines (rms_norm, linear,
+    scaled_dot_product_attention with its default scale 1/sqrt(head size) and its grouped-query
+    mode, silu); only the rotation is the plain implementation's (pinned above).  Placement of
+    the norms (gains are not one here), which products carry a bias (q, k, v; not o, not the
+    feed-forward), the scale (TINY_C's head size is not width / heads), the head mapping and the
+    tied head all have to agree.  src/models/qwen2/graph.rs:59-182."""
+    F = torch.nn.functional
+    m = with_random_gains(models[name], seed=31)
+    c = m.c
+    nh, nk = c["num_attention_heads"], c["num_key_value_heads"]
+    hd = c.get("head_dim") or c["hidden_size"] // nh
+    eps, theta = c["rms_norm_eps"], c["rope_theta"]
+    toks = random_tokens(c["vocab_size"], 11, 7)
+    t = {k: torch.tensor(v) for k, v in m.w.items()}
+    n = len(toks)
+    pos = np.arange(n)
+    h = t["model.embed_tokens.weight"][toks]
+    for i in range(c["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        x = F.rms_norm(h, (h.shape[-1],), t[p + "input_layernorm.weight"], eps)
+        q = F.linear(x, t[p + "self_attn.q_proj.weight"], t[p + "self_attn.q_proj.bias"])
+        k = F.linear(x, t[p + "self_attn.k_proj.weight"], t[p + "self_attn.k_proj.bias"])
+        v = F.linear(x, t[p + "self_attn.v_proj.weight"], t[p + "self_attn.v_proj.bias"])
+        q = torch.tensor(pq.rope_neox(q.numpy(), pos, nh, hd, theta)).view(n, nh, hd).transpose(0, 1)
+        k = torch.tensor(pq.rope_neox(k.numpy(), pos, nk, hd, theta)).view(n, nk, hd).transpose(0, 1)
+        v = v.view(n, nk, hd).transpose(0, 1)
+        a = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)      # scale: 1/sqrt(hd)
+        h = h + F.linear(a.transpose(0, 1).reshape(n, nh * hd), t[p + "self_attn.o_proj.weight"])
+        x = F.rms_norm(h, (h.shape[-1],), t[p + "post_attention_layernorm.weight"], eps)
+        h = h + F.linear(F.silu(F.linear(x, t[p + "mlp.gate_proj.weight"])) * F.linear(x, t[p + "mlp.up_proj.weight"]),
+                         t[p + "mlp.down_proj.weight"])
+    x = F.rms_norm(h, (h.shape[-1],), t["model.norm.weight"], eps)
+    out = F.linear(x, t["model.embed_tokens.weight"] if c.get("tie_word_embeddings") else t["lm_head.weight"])
+    assert f"model.layers.0.self_attn.o_proj.bias" not in m.w and "model.layers.0.mlp.down_proj.bias" not in m.w
+    assert np.abs(m.forward(toks) - out.numpy()).max() < 1e-10
+
+
+def test_each_branch_reads_the_normed_stream_and_adds_to_the_raw_one(models):
+    """Pre-norm: a branch sees norm(h) and its output is added to h itself.  With the other
+    branch switched off (its output matrix zero), layer(c h) - c h is the same for every c > 0,
+    because norm(c h) = norm(h) (eps aside); a norm after the addition, or a branch fed h itself,
+    would not give that."""
+    m = with_random_gains(models["B"], seed=41)
+    h = rnd(6, 128, seed=42) * 3.0
+    pos = np.arange(6)
+    for off, what in (("mlp.down_proj.weight", "attention"), ("self_attn.o_proj.weight", "feed-forward")):
+        w = dict(m.w)
+        w["model.layers.0." + off] = np.zeros_like(w["model.layers.0." + off])
+        z = pq.PlainQwen2(m.c, w)
+        base = z.layer(0, h, pos) - h
+        assert np.abs(base).max() > 1e-3, what
+        for c in (0.5, 7.0):
+            assert np.allclose(z.layer(0, c * h, pos) - c * h, base, rtol=1e-4, atol=1e-7), what
