@@ -15,10 +15,9 @@
 //   O^T[col][head] += V^T P^T   A = V^T rows straight from the cache, B = P^T
 // The cache keeps V transposed inside a page in bfloat16, in two halves of 32 keys
 // ([2][head_dim][32 keys]), so V^T rows are contiguous over the keys of a step like K rows are
-// over head_dim, the 16 rows a load takes are one contiguous kilobyte (whole 128-byte lines: with
-// rows of 64 keys a step asked for half of each line, and what a CU can have in flight is counted
-// in lines: 64 sequences of up to 2,048 keys took 41 us that way and take 30 now), and neither
-// operand passes through LDS.  In both results a lane owns one head (lane % 16): the softmax statistics are
+// over head_dim, the 16 rows a load takes are one contiguous kilobyte (whole 128-byte lines: what
+// a CU can have in flight is counted in lines, and rows of 64 keys would ask for half of each),
+// and neither operand passes through LDS.  In both results a lane owns one head (lane % 16): the softmax statistics are
 // per-lane scalars, and the scores a lane holds (8 consecutive keys, by the choice of which
 // key each K row of a tile is) are exactly the 8 k-slots of its B operand in the second
 // product, so P never leaves its registers.
@@ -187,9 +186,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int n_steps = j_begin < j_end ? (j_end - 1) / STEP - step0 + 1 : 0;
   bf16x8 kn[2][KS], vn[CT];
   // The page of a step is looked up a whole step before its keys are asked for, so that the
-  // look-up's latency does not stand in front of every step's loads.  (Two steps in flight per
-  // wave instead of one measured the same, 30 us for 64 sequences of up to 2,048 keys and 4.7
-  // TB/s at 30,000, at twice the registers: the waves are not what the memory waits for.)
+  // look-up's latency does not stand in front of every step's loads.  One step in flight per wave
+  // is enough: with two, at twice the registers, nothing was faster.
   auto page_of = [&](int i) { return pt[(step0 + i) * STEP / MF_PAGE]; };
   auto issue = [&](int i, int page) {
     const int jb = (step0 + i) * STEP;

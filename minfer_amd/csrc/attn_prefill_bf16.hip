@@ -25,9 +25,9 @@ constexpr int BQ = 128;             // query tokens per block
 constexpr int KT = MF_PAGE;         // keys per step: one page
 constexpr int VT_LD = KT + 4;       // LDS row stride of V^T in elements: 34 words, conflict-free 8-byte reads
 
-// Two blocks per CU up to head size 128: left to itself the compiler takes 348 registers there
-// (one wave per SIMD) and shuffles the accumulators between the two register files; held to 256
-// it needs no scratch and the kernel takes 82 us instead of 144 (28 heads, 2,048 tokens).
+// Two blocks per CU up to head size 128: left to itself the compiler takes more than 256 registers
+// there (one wave per SIMD) and shuffles the accumulators between the two register files; held to
+// 256 it needs no scratch and runs nearly twice as fast.
 template <int NKS>                  // head_dim / 16
 __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,

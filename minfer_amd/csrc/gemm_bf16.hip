@@ -249,10 +249,9 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const 
 // without passing registers (global_load_lds_dwordx4: lane i's 16 bytes land at the wave's LDS
 // base + 16 i), two stages of 64 KB, and the 32 staging registers are gone.
 //
-// A row of a k tile is one 128-byte line, fetched by 8 adjacent lanes: a CU keeps only about 64
-// requests to L2 in flight (measured: 64-byte requests, which k tiles of 32 make, drew 28 GB/s
-// a CU at L2's 300 cycles and left the waves waiting for their tiles 40% of the time), so every
-// request has to be a whole line.
+// A row of a k tile is one 128-byte line, fetched by 8 adjacent lanes: what a CU can have in
+// flight towards L2 is counted in requests, so every request should be a whole line (k tiles of
+// 32, half lines, drew markedly less).
 //
 // There is no room for padding in such a copy, so a row's eight 16-byte chunks are stored
 // permuted: chunk c of row r sits at position c ^ ((r >> 1) & 7), which spreads the 16 rows
@@ -263,27 +262,9 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const 
 // kernel does, with vmcnt counts it keeps itself (8 loads per wave and tile, in order) and
 // one barrier per tile: behind it, tile kt + 1 has landed for every wave, and the stage of tile
 // kt, which every wave holds in registers by then, is free to take tile kt + 2.
-// Needs 16-byte aligned rows and K a multiple of 64.
-// Measured on the 2048 x 37888 x 3584 product (0.95 PFLOP/s): without the copies 1.1, without
-// copies and fragment reads 1.3 (the matrix cores alone, with the epilogue's 310 MB of output),
-// at a clock of 2.0 GHz under this load; asking for a tile in four parts spread over a tile's
-// products, or leaving the barrier out, changed nothing, and neither did three stages for the W
-// tiles (which come from HBM) beside two for the A tiles, five times 32 KB, so that a W tile has
-// two tile times to arrive: it is not the copies' latency that the matrix cores wait for.
-// Counters on that product: the matrix cores busy 53% of the cycles at 1.93 GHz, LDS 16%, no bank
-// conflicts, waves 1.6% of their time waiting for LDS.  Nor is it that the two waves of a SIMD
-// run in step: a variant whose waves took turns in two groups (one multiplies a whole k tile from
-// registers, 32 products in a row, while the other reads its fragments and issues the copies; a
-// barrier per half tile) gave the same 1.0 PFLOP/s to the percent.
-// What the loop is made of, each measured alone on 256 blocks of 8 waves (the same 32 products
-// per k tile from the same registers): products only 2.4 PFLOP/s with constant operands and 1.9
-// with this kernel's; with the 24 fragment reads and a barrier per tile still 1.9; with the
-// copies as well, two stages, 1.55 when every copy is an L2 hit, 1.24 when the A tiles are
-// shared by all blocks and a W tile by 8 blocks on different XCDs, 0.79 when every block streams
-// its own data from HBM (6.2 TB/s).  So the distance from 1.9 is the copies: where their lines
-// come from, not how they are issued.  Touching the lines of the tile four ahead with one dword
-// each (to have them in L2 when the copies ask) made it 10% slower: the touches go through the
-// same queue and the same L1.
+// Needs 16-byte aligned rows and K a multiple of 64.  What keeps this kernel from the matrix
+// cores' own rate is where the copies' lines come from (HBM and other dies' share of the data),
+// not how the copies are issued; the figures are in the design notes.
 constexpr int DMA_BM = 256, DMA_BN = 256, DMA_BK = 64, DMA_STAGES = 2;
 constexpr int DMA_STAGE_BYTES = (DMA_BM + DMA_BN) * DMA_BK * 2;
 
