@@ -834,7 +834,7 @@ def probe_read(buffer: torch.Tensor, blocks: Optional[int] = None) -> None:
     memory bandwidth; time it from outside)."""
     _need(buffer, "probe_read.buffer")
     nbytes = buffer.numel() * buffer.element_size() // 16 * 16
-    blocks = blocks or cu_count() * 8
+    blocks = blocks or cu_count()
     sink = workspace("probe", blocks, buffer.device)
     _check(_fn("probe", "mf_probe_read")(_ptr(buffer), nbytes, _ptr(sink), blocks, _stream()), "probe_read")
 
