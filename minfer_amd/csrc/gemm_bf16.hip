@@ -6,8 +6,9 @@
 // The kernels:
 //  * `tile_kernel`: many rows (prompts).  A BM x BN block tile per 4 or 8 waves, K walked in
 //    steps of BK through double-buffered LDS, 32x32x16 MFMA, each wave a WM x WN tile.
-//  * `tile_dma_kernel`: the 256 x 256 tile with its k tiles copied straight into LDS; the
-//    choice for large aligned products.
+//  * `tile_dma_kernel`: tiles of 256 x 256, 256 x 192 or 256 x 128 with their k tiles copied
+//    straight into LDS; the choice for large aligned products (the width by how the tiles fill
+//    the chip's rounds).
 //  * `stationary16_kernel`: at most 16 rows and K of 1536, 2048, 3584, 4096, 5120 or 8192 (decode):
 //    one block per CU keeps the activations in registers and walks over weight tiles.
 //  * `rolling16_kernel`, `skinny16_kernel`: at most 16 rows, any K (decode).  The time is the
@@ -18,8 +19,6 @@
 //    weight rows and reads them from HBM straight into MFMA operands, the activation rows are
 //    staged in LDS and shared by the block, K may be split over blocks with a fixed-order
 //    reduction afterwards.
-// For measurements the environment can take a kernel out of the choice: MF_NO_STATIONARY,
-// MF_NO_PANEL, MF_NO_SKINNY_RING, and MF_NO_XCD_REMAP (the tile kernels' block order).
 // Both operands have K contiguous, which is exactly the MFMA operand layout (8 consecutive
 // k per lane), so nothing is transposed.
 //
@@ -245,9 +244,14 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const 
 }
 
 // ------------------------------------------------------------------ tiled kernel, loads straight into LDS
-// The same 256 x 256 tile on 8 waves (each 128 x 64), but k tiles of 64 travel global -> LDS
+// A tile of 256 rows by BN weight rows on 8 waves, but k tiles of 64 travel global -> LDS
 // without passing registers (global_load_lds_dwordx4: lane i's 16 bytes land at the wave's LDS
-// base + 16 i), two stages of 64 KB, and the 32 staging registers are gone.
+// base + 16 i), in two or three stages of (256 + BN) * 128 bytes, and the staging registers are
+// gone.  The widths: 256 (waves of 128 x 64, two stages of 64 KB) has the most products per
+// byte copied and is the fastest where its tiles fill the chip's rounds; 192 (waves of 64 x 96)
+// and 128 (waves of 64 x 64, three stages) make more, smaller tiles for products whose 256-wide
+// tiles would leave a round half empty (q|k|v and o of a prompt of 2,048 tokens: 144 and 112
+// such tiles for 256 CUs).
 //
 // A row of a k tile is one 128-byte line, fetched by 8 adjacent lanes: what a CU can have in
 // flight towards L2 is counted in requests, so every request should be a whole line (k tiles of
@@ -259,14 +263,14 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const 
 // is free (its global address), so the permutation costs nothing on the way in.
 //
 // The compiler does not know that these loads write LDS and so does not wait for them; the
-// kernel does, with vmcnt counts it keeps itself (8 loads per wave and tile, in order) and
-// one barrier per tile: behind it, tile kt + 1 has landed for every wave, and the stage of tile
-// kt, which every wave holds in registers by then, is free to take tile kt + 2.
+// kernel does, with vmcnt counts it keeps itself (4 + BN / 64 loads per wave and tile, in order)
+// and one barrier per tile: behind it, tile kt + 1 has landed for every wave, and the stage of
+// tile kt, which every wave holds in registers by then, is free to take tile kt + STAGES.
 // Needs 16-byte aligned rows and K a multiple of 64.  What keeps this kernel from the matrix
 // cores' own rate is where the copies' lines come from (HBM and other dies' share of the data),
-// not how the copies are issued; the figures are in the design notes.
-constexpr int DMA_BM = 256, DMA_BN = 256, DMA_BK = 64, DMA_STAGES = 2;
-constexpr int DMA_STAGE_BYTES = (DMA_BM + DMA_BN) * DMA_BK * 2;
+// not how the copies are issued: blocks that run side by side on an XCD must walk K in step, so
+// that a line one of them fetches is in that XCD's L2 for the others.
+constexpr int DMA_BM = 256, DMA_BK = 64;
 
 // 16 bytes per lane from base + off (a wave-uniform base and a 32-bit byte offset per lane: one
 // register where a 64-bit address takes two, and no address arithmetic per copy)
@@ -275,13 +279,30 @@ __device__ __forceinline__ void dma16(const bf16* base, unsigned off, unsigned l
                : "memory", "m0");
 }
 
+// waits until at most `tiles` of the youngest k tiles' copies (LOADS a wave and tile) are in flight
+template <int LOADS>
+__device__ __forceinline__ void dma_wait(int tiles) {
+  if (tiles <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  else if (tiles == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS) : "memory");
+  else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LOADS) : "memory");
+}
+
+// BN: the tile's width (256 or 128); WAVES_M x (8 / WAVES_M): the grid of the 8 waves over the
+// tile; STAGES: k tiles of a tile in LDS (2 or 3), (256 + BN) * 128 bytes each.
+template <int BN, int WAVES_M, int STAGES>
 __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ A, int lda,
                                                        const bf16* __restrict__ W, int ldw,
                                                        const float* __restrict__ bias, void* __restrict__ C,
                                                        int ldc, int M, int N, int K, int epi, int tiles_m,
                                                        int xcd_remap, int k_per_split) {
-  constexpr int TM = 4, TN = 2;
+  constexpr int WAVES_N = 8 / WAVES_M;
+  constexpr int WM = DMA_BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int ROW = DMA_BK * 2;              // bytes of a row in LDS
+  constexpr int STAGE_BYTES = (DMA_BM + BN) * ROW;
+  constexpr int WB = BN / 64;                  // 1 KB blocks of the W tile that a wave copies
+  constexpr int LOADS = 4 + WB;                // copies per wave and k tile
+  static_assert(STAGES == 2 || STAGES == 3, "the waits count one or two tiles in flight");
   if (k_per_split > 0) {
     // K split over blockIdx.y (k_per_split a multiple of 64): this block multiplies its part of K
     // and stores 32-bit sums into its own [M][N] slab of C; another kernel adds the slabs
@@ -299,10 +320,10 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
     tile = x * per + min(x, rem) + qq;
   }
   const int bm = tile % tiles_m, bn = tile / tiles_m;
-  const int m0 = bm * DMA_BM, n0 = bn * DMA_BN;
+  const int m0 = bm * DMA_BM, n0 = bn * BN;
   const int lane = threadIdx.x & 63;
   const int wid = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wm = (wid & 1) * 128, wn = (wid >> 1) * 64;
+  const int wm = (wid % WAVES_M) * WM, wn = (wid / WAVES_M) * WN;
   const int fr = lane & 31, fk = lane >> 5;
 
   floatx16 acc[TM][TN];
@@ -313,28 +334,27 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // this lane's share of a tile's copy: wave `wid` moves the 1 KB blocks wid, 8 + wid, 16 + wid
-  // and 24 + wid (8 rows each) of the A tile and of the W tile; the lane fetches row
-  // 8 b + lane / 8, the chunk that belongs at position lane % 8
+  // this lane's share of a tile's copy: wave `wid` moves the 1 KB blocks wid, 8 + wid, ... (8 rows
+  // each) of the A tile and of the W tile; the lane fetches row 8 b + lane / 8, the chunk that
+  // belongs at position lane % 8
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
-  unsigned ga[4], gw[4];                       // byte offsets from A and W (the host checks that they fit)
+  unsigned ga[4], gw[WB];                      // byte offsets from A and W (the host checks that they fit)
 #pragma unroll
   for (int jj = 0; jj < 4; ++jj) {
     const int r = 8 * (jj * 8 + wid) + (lane >> 3);
     const int chunk = (lane & 7) ^ ((r >> 1) & 7);
     ga[jj] = ((unsigned)min(m0 + r, M - 1) * (unsigned)lda + chunk * 8) * 2u;
-    gw[jj] = ((unsigned)min(n0 + r, N - 1) * (unsigned)ldw + chunk * 8) * 2u;
+    if (jj < WB) gw[jj] = ((unsigned)min(n0 + r, N - 1) * (unsigned)ldw + chunk * 8) * 2u;
   }
-  // copy q of a wave's eight for tile kt: four blocks of the A tile, then four of the W tile
-  auto issue_one = [&](int kt, int q) {
-    const unsigned st = lds0 + (unsigned)(kt % DMA_STAGES) * DMA_STAGE_BYTES + wid * 1024;
+  // the copies of a wave for tile kt into stage st: four blocks of the A tile, then WB of the W tile
+  auto issue = [&](int kt, int st) {
+    const unsigned base = lds0 + (unsigned)st * STAGE_BYTES + wid * 1024;
     const int k = kt * DMA_BK;
-    if (q < 4) dma16(A + k, ga[q], __builtin_amdgcn_readfirstlane(st + q * 8192));
-    else dma16(W + k, gw[q - 4], __builtin_amdgcn_readfirstlane(st + DMA_BM * ROW + (q - 4) * 8192));
-  };
-  auto issue = [&](int kt) {
 #pragma unroll
-    for (int q = 0; q < 8; ++q) issue_one(kt, q);
+    for (int q = 0; q < 4; ++q) dma16(A + k, ga[q], __builtin_amdgcn_readfirstlane(base + q * 8192));
+#pragma unroll
+    for (int q = 0; q < WB; ++q)
+      dma16(W + k, gw[q], __builtin_amdgcn_readfirstlane(base + DMA_BM * ROW + q * 8192));
   };
   // fragment reads: row R of a tile, chunk 4 half + 2 ks + fk of its 8, at position chunk ^ ((R >> 1) & 7)
   const int sw = (fr >> 1) & 7;
@@ -351,7 +371,7 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
   bf16x8 fa[2][2][TM], fw[2][2][TN];          // [set][k-step][tile]
   auto read_frags = [&](int stage, auto HALF) {
     constexpr int half = decltype(HALF)::value;          // which is also the register set
-    const unsigned char* st = smem + stage * DMA_STAGE_BYTES;
+    const unsigned char* st = smem + stage * STAGE_BYTES;
     const int pos0 = ((half * 4 + fk) ^ sw) * 16, pos1 = ((half * 4 + 2 + fk) ^ sw) * 16;
 #pragma unroll
     for (int i = 0; i < TM; ++i) fa[half][0][i] = *reinterpret_cast<const bf16x8*>(st + offa[i] + pos0);
@@ -372,12 +392,11 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
   };
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
-  issue(0);
-  int issued = 0;
-  if (nkt > 1) { issue(1); issued = 1; }
-  // the loads of tile 0 (of this wave) have landed when at most tile 1's eight are in flight
-  if (issued == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // tiles 0 .. STAGES - 1 set out at once; tile 0 has landed (for this wave) when only the ones
+  // after it are in flight
+  int issued = 0;                              // tiles set out so far
+  for (; issued < STAGES && issued < nkt; ++issued) issue(issued, issued);
+  dma_wait<LOADS>(issued - 1);
   __syncthreads();
   read_frags(0, S0{});
   int stage = 0;                               // of tile kt
@@ -397,11 +416,10 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
     // this tile's stage free
     multiply(0, S1{});
     __builtin_amdgcn_sched_barrier(0);
-    if (issued > kt + 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    dma_wait<LOADS>(issued - kt - 2);          // tile kt + 1 has landed when only the later ones are in flight
     __syncthreads();
-    if (issued + 1 < nkt) { issue(issued + 1); ++issued; }      // into the stage of tile kt
-    stage ^= 1;
+    if (issued < nkt) { issue(issued, stage); ++issued; }         // into the stage of tile kt
+    stage = stage + 1 == STAGES ? 0 : stage + 1;
     read_frags(stage, S0{});
     __builtin_amdgcn_sched_barrier(0);
     multiply(1, S1{});
@@ -417,19 +435,21 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
   tile_epilogue<TM, TN>(acc, bias, C, ldc, M, N, epi, m0, wm, n0, wn, lane);
 }
 
+template <int BN, int WAVES_M, int STAGES>
 int launch_tile_dma(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc, int M,
                     int N, int K, int epi, hipStream_t stream, int splits = 1, int k_per_split = 0) {
-  constexpr int smem = DMA_STAGES * DMA_STAGE_BYTES;
+  constexpr int smem = STAGES * (DMA_BM + BN) * DMA_BK * 2;
   static bool configured = false;
+  auto kern = tile_dma_kernel<BN, WAVES_M, STAGES>;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(tile_dma_kernel),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     configured = true;
   }
-  const int tiles_m = (M + DMA_BM - 1) / DMA_BM, tiles_n = (N + DMA_BN - 1) / DMA_BN;
-  tile_dma_kernel<<<dim3(tiles_m * tiles_n, splits), 512, smem, stream>>>(
-      A, lda, W, ldw, bias, C, ldc, M, N, K, epi, tiles_m, tiles_m * tiles_n >= 16, k_per_split);
+  const int tiles_m = (M + DMA_BM - 1) / DMA_BM, tiles_n = (N + BN - 1) / BN;
+  kern<<<dim3(tiles_m * tiles_n, splits), 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, tiles_m,
+                                                               tiles_m * tiles_n >= 16, k_per_split);
   return mf_launch_status();
 }
 
@@ -1495,22 +1515,69 @@ int launch_panel(const bf16* A, int lda, const bf16* W, int ldw, const float* bi
   return MF_NOT_BUILT;
 }
 
-// The tile kernel of a product with many rows: 256 x 256 tiles run one block per CU (faster
-// through the direct-to-LDS pipeline than through registers), 128 x 128 tiles two blocks per CU at a
-// somewhat lower rate each; the number of rounds the tiles take over the CUs decides.  Tiny
-// problems take 64 x 64.
-int tile_variant(int M, int N, bool dma_ok, int epi, int n_cu) {
-  const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-  const long t128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-  const long slots = n_cu > 0 ? n_cu : 1;
-  const double cost256 = (double)((t256 + slots - 1) / slots) * (256. * 256.) / (dma_ok ? 0.95 : 0.88);
-  const double cost128 = (t128 <= slots ? 1. : 2. * (double)((t128 + 2 * slots - 1) / (2 * slots))) *
-                         (128. * 128.) / 0.80;
-  int variant;
-  if (cost256 < cost128) variant = dma_ok ? 12 : 9;
-  else variant = (t128 >= 64 || M > 64) ? 2 : 3;
-  if (epi == EPI_SWIGLU && variant == 3) variant = 2;
-  return variant;
+// ---- which tile kernel a product of many rows takes
+// Variants: 2: 128 x 128 tiles through registers (two blocks a CU), 3: 64 x 64, 9: 256 x 256 through
+// registers, and the direct-to-LDS kernel (aligned operands, K in 64s) with tiles of 256 x 256
+// (12), 256 x 192 (15, no SwiGLU) and 256 x 128 in three stages (13).  With `splits` > 1 the K
+// dimension is cut over blocks (variants 12 and 2) and skinny_reduce_kernel adds the parts.
+struct TilePlan { int variant, splits, k_per_split; double us; };
+
+// The estimate behind the choice: a kernel's tiles go over its slots (blocks that fit the chip at
+// once) in rounds; a round takes the product's k tiles of 64 times the variant's time per k tile
+// (measured at the 7B widths with every CU busy), a last round that is not full somewhat less
+// (fewer blocks pull on the fabric); a start, the epilogue's traffic, and for a K split the
+// parts' way to memory and back come on top.
+double rounds_us(long blocks, long slots, double step_us, long nkt) {
+  const long full = blocks / slots;
+  const double fill = (double)(blocks % slots) / (double)slots;
+  return (double)nkt * step_us * ((double)full + (fill > 0. ? 0.7 + 0.3 * fill : 0.));
+}
+
+TilePlan plan_tiles(int M, int N, int K, bool dma_ok, int epi, int n_cu) {
+  const long cu = n_cu > 0 ? n_cu : 1;
+  const long nkt = (K + 63) / 64, chunks = (K + 255) / 256;
+  const double mn = (double)M * (double)N;
+  const double epi_us = (epi == EPI_ACC_F32 ? 8. : epi == EPI_F32 ? 4. : epi == EPI_BF16 ? 2. : 1.) * mn / 4e6;
+  const double start_us = 12.;
+  auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+  auto cut = [&](long parts, int& splits, int& per) {          // K in `parts` runs of whole chunks of 256
+    const long c = (chunks + parts - 1) / parts;
+    splits = (int)((chunks + c - 1) / c);
+    per = (int)(c * 256);
+  };
+  auto parts_us = [&](int splits) { return (double)(splits + 2) * mn * 4. / 3.5e6 + 5.; };
+  TilePlan best{0, 1, K, 1e30};
+  auto offer = [&](int variant, int splits, int per, double us) {
+    if (us < best.us) best = TilePlan{variant, splits, per, us};
+  };
+  if (dma_ok) {
+    offer(12, 1, K, rounds_us(tiles(256, 256), cu, 1.75, nkt) + start_us + epi_us);
+    offer(13, 1, K, rounds_us(tiles(256, 128), cu, 1.00, nkt) + start_us + epi_us);
+    if (epi != EPI_SWIGLU) offer(15, 1, K, rounds_us(tiles(256, 192), cu, 1.35, nkt) + start_us + epi_us);
+    // many rows against few weight rows and a long K (the down product of a prompt): K cut over
+    // the big tiles, each part at least 2,048 of K
+    if (epi != EPI_SWIGLU && M >= 768)
+      for (long parts = 2; parts <= std::min<long>(8, K / 2048); ++parts) {
+        int splits, per;
+        cut(parts, splits, per);
+        if (splits < 2) continue;
+        offer(12, splits, per, rounds_us(tiles(256, 256) * splits, cu, 1.75, per / 64) + start_us + parts_us(splits));
+      }
+  } else {
+    offer(9, 1, K, rounds_us(tiles(256, 256), cu, 2.1, nkt) + start_us + epi_us);
+  }
+  const long t128 = tiles(128, 128);
+  offer(M <= 64 && t128 < 64 && epi != EPI_SWIGLU ? 3 : 2, 1, K,
+        rounds_us(t128, 2 * cu, 1.45, nkt) + start_us + epi_us);
+  // a few hundred rows against a few thousand weight rows (some 50 tiles of 128 x 128, bound by
+  // the weight stream): K over about two blocks per CU, each with at least 512 of K
+  const long parts = std::min(chunks / 2, (2 * cu) / std::max(1L, t128));
+  if (t128 < cu && parts >= 2) {
+    int splits, per;
+    cut(parts, splits, per);
+    if (splits >= 2) offer(2, splits, per, rounds_us(t128 * splits, 2 * cu, 1.45, per / 64) + start_us + parts_us(splits));
+  }
+  return best;
 }
 
 // Which kernel a product of at most 64 rows takes.
@@ -1540,9 +1607,9 @@ SkinnyChoice skinny_choice(int M, int N, int K, bool aligned, int epi, int split
 
 }  // namespace
 
-// `variant`: 0 picks by shape; 1: 256x256 tile with 4 waves, 2: 128x128, 3: 64x64, 6: 256x128
-// with 8 waves, 9: 256x256 with 8 waves, 12: 256x256 through the direct-to-LDS pipeline, K in 64s (tests
-// name them).
+// `variant`: 0 picks by shape among the whole-K kernels; 1: 256x256 tile with 4 waves, 2: 128x128,
+// 3: 64x64, 6: 256x128 with 8 waves, 9: 256x256 with 8 waves; through the direct-to-LDS pipeline, K in
+// 64s: 12: 256x256, 13: 256x128 in three stages, 15: 256x192 (tests name them).
 MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
                         int ldc, int M, int N, int K, int epi, int variant, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -1555,7 +1622,11 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
   const bf16* w = (const bf16*)W;
   // the direct-to-LDS kernel addresses its operands with 32-bit byte offsets
   const bool dma_ok = vec_ok && K % DMA_BK == 0 && (size_t)M * lda * 2 < (1ull << 32) && (size_t)N * ldw * 2 < (1ull << 32);
-  if (variant == 0) variant = tile_variant(M, N, dma_ok, epi, cu_count());
+  if (variant == 0) {
+    const TilePlan plan = plan_tiles(M, N, K, dma_ok, epi, cu_count());
+    if (plan.splits > 1) return (int)hipErrorInvalidValue;       // a K split needs the caller's workspace
+    variant = plan.variant;
+  }
   if (epi == EPI_SWIGLU && variant == 3) variant = 2;      // needs two 32-column tiles per wave
   switch (variant) {
     case 1: return launch_tile<256, 256, 128, 128>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
@@ -1565,7 +1636,13 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
     case 9: return launch_tile<256, 256, 128, 64, 64>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case 12:
       if (!dma_ok) return (int)hipErrorInvalidValue;
-      return launch_tile_dma(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+      return launch_tile_dma<256, 2, 2>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+    case 13:
+      if (!dma_ok) return (int)hipErrorInvalidValue;
+      return launch_tile_dma<128, 4, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+    case 15:
+      if (!dma_ok || epi == EPI_SWIGLU) return (int)hipErrorInvalidValue;
+      return launch_tile_dma<192, 4, 2>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
   }
   return (int)hipErrorInvalidValue;
 }
@@ -1576,7 +1653,7 @@ MF_API int mf_gemm_bf16(const void* A, int lda, const void* W, int ldw, const fl
 // k_per_split is a multiple of 64.
 MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
                                int ldc, float* part, int M, int N, int K, int splits, int k_per_split,
-                               int epi, int big_tiles, hipStream_t stream) {
+                               int epi, int variant, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || lda < K || ldw < K || epi < 0 || epi > 3 || splits < 2 || !part || k_per_split % 64 != 0 ||
       (long)splits * k_per_split < K || (long)(splits - 1) * k_per_split >= K)
@@ -1585,12 +1662,14 @@ MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, c
     return (int)hipErrorInvalidValue;
   const int vec_ok = (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) &&
                      ((uintptr_t)W % 16 == 0) && (K % 8 == 0);
-  // big_tiles: 256 x 256 tiles through the direct-to-LDS pipeline (many rows against few weight
-  // rows and a long K: the down product of a prompt); else 128 x 128 (few rows)
+  // variant 12: 256 x 256 tiles through the direct-to-LDS pipeline (many rows against few weight
+  // rows and a long K: the down product of a prompt); 2: 128 x 128 (few rows)
+  if (variant != 12 && variant != 2) return (int)hipErrorInvalidValue;
+  const bool big_tiles = variant == 12;
   if (big_tiles && (!vec_ok || K % DMA_BK != 0 || (size_t)M * lda * 2 >= (1ull << 32) ||
                     (size_t)N * ldw * 2 >= (1ull << 32)))
     return (int)hipErrorInvalidValue;
-  int rc = big_tiles ? launch_tile_dma((const bf16*)A, lda, (const bf16*)W, ldw, nullptr, part, N, M, N, K,
+  int rc = big_tiles ? launch_tile_dma<256, 2, 2>((const bf16*)A, lda, (const bf16*)W, ldw, nullptr, part, N, M, N, K,
                                        EPI_F32, stream, splits, k_per_split)
                      : launch_tile<128, 128, 64, 64>((const bf16*)A, lda, (const bf16*)W, ldw, nullptr, part, N, M,
                                                      N, K, EPI_F32, vec_ok, stream, splits, k_per_split);
@@ -1670,13 +1749,26 @@ MF_API int mf_gemm_bf16_normed(const float* x, int ldx, const int* row_idx, cons
   return stationary16(x, ldx, (const bf16*)W, ldw, bias, C, ldc, M, N, K, epi, &norm, stream);
 }
 
+// How a product of more than 64 rows is run: out[0] the variant for mf_gemm_bf16, or with out[1] > 1
+// for mf_gemm_bf16_splitk with out[1] splits of out[2] of K each.  `aligned`: 16-byte aligned
+// operands with row strides and K in multiples of 8.
+MF_API int mf_gemm_bf16_tile_plan(int M, int N, int K, int aligned, int epi, int n_cu, int* out) {
+  if (!out || M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 3 || n_cu <= 0) return (int)hipErrorInvalidValue;
+  const bool dma_ok = aligned && K % DMA_BK == 0 && (size_t)M * K * 2 < (1ull << 32) && (size_t)N * K * 2 < (1ull << 32);
+  const TilePlan plan = plan_tiles(M, N, K, dma_ok, epi, n_cu);
+  out[0] = plan.variant;
+  out[1] = plan.splits;
+  out[2] = plan.k_per_split;
+  return 0;
+}
+
 // The name of the kernel that a product of this shape takes, without launching anything: `rows`
 // activation rows against `N` weight rows of length `K`; `aligned`: 16-byte aligned operands with
-// row strides and K in multiples of 8; `splits`, `k_per_split`, `big_tiles`: the caller's K split
-// (1, K, 0 for none); `normed`: the RMS norm is to be folded in (an empty name then means "no such
-// kernel": norm and product run one after the other); `n_cu`: compute units of the device.
+// row strides and K in multiples of 8; for at most 64 rows `splits`, `k_per_split`: the caller's K
+// split (1, K for none); `normed`: the RMS norm is to be folded in (an empty name then means "no
+// such kernel": norm and product run one after the other); `n_cu`: compute units of the device.
 MF_API int mf_gemm_bf16_plan(int M, int N, int K, int aligned, int epi, int splits, int k_per_split,
-                             int big_tiles, int normed, int n_cu, char* name, int cap) {
+                             int normed, int n_cu, char* name, int cap) {
   if (!name || cap < 48 || M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 3 || n_cu <= 0) return (int)hipErrorInvalidValue;
   const char* what = "";
   if (normed) {
@@ -1690,14 +1782,15 @@ MF_API int mf_gemm_bf16_plan(int M, int N, int K, int aligned, int epi, int spli
       case SK_RING: what = "skinny_ring_kernel"; break;
       case SK_STAGED: what = "skinny_kernel"; break;
     }
-  } else if (splits > 1) {
-    what = big_tiles ? "tile_dma_kernel(split K)" : "tile_kernel<128,128>(split K)";
   } else {
     const bool dma_ok = aligned && K % DMA_BK == 0 && (size_t)M * K * 2 < (1ull << 32) && (size_t)N * K * 2 < (1ull << 32);
-    switch (tile_variant(M, N, dma_ok, epi, n_cu)) {
-      case 12: what = "tile_dma_kernel"; break;
+    const TilePlan plan = plan_tiles(M, N, K, dma_ok, epi, n_cu);
+    switch (plan.variant) {
+      case 12: what = plan.splits > 1 ? "tile_dma_kernel<256>(split K)" : "tile_dma_kernel<256>"; break;
+      case 13: what = "tile_dma_kernel<128>"; break;
+      case 15: what = "tile_dma_kernel<192>"; break;
       case 9: what = "tile_kernel<256,256>"; break;
-      case 2: what = "tile_kernel<128,128>"; break;
+      case 2: what = plan.splits > 1 ? "tile_kernel<128,128>(split K)" : "tile_kernel<128,128>"; break;
       default: what = "tile_kernel<64,64>"; break;
     }
   }

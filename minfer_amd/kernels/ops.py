@@ -57,7 +57,8 @@ _PROTOTYPES = {
                                 c_int, c_int, _P],
         "mf_gemm_bf16_normed": [_P, c_int, _P, _P, c_float, _P, c_int, _P, _P, c_int, c_int, c_int, c_int,
                                 c_int, _P],
-        "mf_gemm_bf16_plan": [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_char_p, c_int],
+        "mf_gemm_bf16_plan": [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_char_p, c_int],
+        "mf_gemm_bf16_tile_plan": [c_int, c_int, c_int, c_int, c_int, c_int, _P],
     },
     "attn_tokens_f32": {
         "mf_attn_tokens_f32": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
@@ -377,52 +378,21 @@ def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None,
     return (chunks + per - 1) // per, per * 256
 
 
-def tile_split_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None) -> Tuple[int, int, bool]:
-    """(splits, k_per_split, big) of the tile product; (1, k, False) where its tiles alone fill the
-    chip.  Two cases split K over blocks, with a second kernel that adds the parts:
-
-    * many rows whose 256 x 256 tiles leave CUs idle or a last round nearly empty (the down product
-      of a prompt of 2,048 tokens at a width of 3584: 112 such tiles for 256 CUs): the big tiles
-      (`big`) with K cut in s parts, s chosen by an estimate of the rounds it takes (cost per unit
-      of K of a round of big and of 128 x 128 tiles, and of adding the parts), each part at least
-      2,048 of K;
-    * a prompt of a few hundred tokens against a few thousand weight rows (some 50 tiles of
-      128 x 128, bound by the weight stream): those tiles with about two blocks per CU, each with
-      at least 512 of K."""
-    cu = target_blocks if target_blocks is not None else cu_count()
-    chunks = (k + 255) // 256
-
-    def cut(splits):
-        per = (chunks + splits - 1) // splits
-        return (chunks + per - 1) // per, per * 256
-
-    t256 = ((m + 255) // 256) * ((n + 255) // 256)
-    tiles = ((m + 127) // 128) * ((n + 127) // 128)
-    if m >= 768 and k % 64 == 0 and not tuning.NO_BIG_SPLIT:
-        rounds = lambda blocks, slots: (blocks + slots - 1) // slots
-        whole = min(rounds(t256, cu) * 28.5e-9 * k, rounds(tiles, 2 * cu) * 18.2e-9 * k)
-        best, best_s = whole, 1
-        for parts in range(2, min(8, k // 2048) + 1):
-            t = rounds(t256 * parts, cu) * 28.5e-9 * k / parts + (parts + 2) * m * n * 4 / 3.5e12
-            if t < 0.92 * best:
-                best, best_s = t, parts
-        if best_s > 1:
-            return cut(best_s) + (True,)
-    splits = min(chunks // 2, (2 * cu) // max(1, tiles))
-    if tiles >= cu or splits < 2:
-        return 1, k, False
-    return cut(splits) + (False,)
+def tile_plan(m: int, n: int, k: int, epi: int, aligned: bool = True, n_cu: Optional[int] = None) -> Tuple[int, int, int]:
+    """(variant, splits, k_per_split) of a bfloat16 product of more than 64 rows, as the library
+    chooses among its tile kernels (an estimate of the rounds their tiles take over the CUs); with
+    splits > 1, K is cut over blocks and a second kernel adds the parts."""
+    out = (c_int * 3)()
+    rc = _fn("gemm_bf16", "mf_gemm_bf16_tile_plan")(m, n, k, 1 if aligned else 0, epi, n_cu or cu_count(), out)
+    if rc != 0:
+        raise KernelError(f"tile_plan: error {rc} for m {m}, n {n}, k {k}")
+    return out[0], out[1], out[2]
 
 
-def _k_split(m: int, n: int, k: int, swiglu: bool, aligned: bool, n_cu: Optional[int] = None) -> Tuple[int, int, bool]:
-    """(splits, k_per_split, big tiles) as `linear` and `linear_swiglu` cut a bfloat16 product."""
-    if m <= 64:
-        target = tuning.SKINNY_TARGET or n_cu
-        return skinny_plan(m, n, k, target_blocks=target, swiglu=swiglu) + (False,)
-    splits, per, big = tile_split_plan(m, n, k, target_blocks=n_cu)
-    if big and (swiglu or not aligned or k % 8):
-        return 1, k, False                     # the big tiles take aligned operands and no SwiGLU epilogue
-    return splits, per, big
+def _k_split(m: int, n: int, k: int, swiglu: bool, aligned: bool, n_cu: Optional[int] = None) -> Tuple[int, int]:
+    """(splits, k_per_split) as `linear` and `linear_swiglu` cut a bfloat16 product of at most 64 rows."""
+    target = tuning.SKINNY_TARGET or n_cu
+    return skinny_plan(m, n, k, target_blocks=target, swiglu=swiglu)
 
 
 def plan_linear(m: int, n: int, k: int, swiglu: bool = False, normed: bool = False, aligned: bool = True,
@@ -434,14 +404,16 @@ def plan_linear(m: int, n: int, k: int, swiglu: bool = False, normed: bool = Fal
     the other).  `n` counts the interleaved gate|up rows for `swiglu`."""
     n_cu = n_cu or cu_count()
     epi = EPI_SWIGLU if swiglu else (EPI_BF16 if out_bf16 else (EPI_ACC_F32 if accumulate else EPI_F32))
-    splits, per, big = 1, k, False
+    splits, per = 1, k
     if normed:
         if m > 16 or tuning.NO_FOLD:
             return dict(kernel="", splits=1, k_per_split=k)
+    elif m <= 64:
+        splits, per = _k_split(m, n, k, swiglu, aligned, n_cu)
     else:
-        splits, per, big = _k_split(m, n, k, swiglu, aligned, n_cu)
+        _, splits, per = tile_plan(m, n, k, epi, aligned, n_cu)
     name = ctypes.create_string_buffer(64)
-    rc = _fn("gemm_bf16", "mf_gemm_bf16_plan")(m, n, k, 1 if aligned else 0, epi, splits, per, 1 if big else 0,
+    rc = _fn("gemm_bf16", "mf_gemm_bf16_plan")(m, n, k, 1 if aligned else 0, epi, splits, per,
                                                1 if normed else 0, n_cu, name, 64)
     if rc != 0:
         raise KernelError(f"plan_linear: error {rc} for m {m}, n {n}, k {k}")
@@ -474,18 +446,18 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
     epi = EPI_BF16 if out.dtype == torch.bfloat16 else (EPI_ACC_F32 if accumulate else EPI_F32)
     aligned = not (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8)
     if m <= 64 and variant == 0:
-        splits, per, _ = _k_split(m, n, k, False, aligned)
+        splits, per = _k_split(m, n, k, False, aligned)
         part = workspace("skinny", splits * m * n, x.device) if splits > 1 else None
         _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(bias),
                                                         _ptr(out), n, _ptr(part), m, n, k, splits, per,
                                                         epi, _stream()), f"gemm_bf16_skinny {m}x{n}x{k}")
         return
     if variant == 0:
-        splits, per, big = _k_split(m, n, k, False, aligned)
+        variant, splits, per = tile_plan(m, n, k, epi, aligned)
         if splits > 1:
             part = workspace("skinny", splits * m * n, x.device)
             _check(_fn("gemm_bf16", "mf_gemm_bf16_splitk")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n,
-                                                            _ptr(part), m, n, k, splits, per, epi, 1 if big else 0,
+                                                            _ptr(part), m, n, k, splits, per, epi, variant,
                                                             _stream()), f"gemm_bf16_splitk {m}x{n}x{k}")
             return
     _check(_fn("gemm_bf16", "mf_gemm_bf16")(_ptr(x), k, _ptr(weight), k, _ptr(bias), _ptr(out), n, m,
@@ -519,18 +491,18 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, vari
         return
     aligned = not (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8)
     if m <= 64 and variant == 0:
-        splits, per, _ = _k_split(m, n, k, True, aligned)
+        splits, per = _k_split(m, n, k, True, aligned)
         part = workspace("skinny", splits * m * n, x.device) if m > 16 or splits > 1 else None
         _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
                                                         _ptr(part), m, n, k, splits, per, EPI_SWIGLU, _stream()),
                f"gemm_bf16_skinny(swiglu) {m}x{n}x{k}")
         return
     if variant == 0:
-        splits, per, big = _k_split(m, n, k, True, aligned)
+        variant, splits, per = tile_plan(m, n, k, EPI_SWIGLU, aligned)
         if splits > 1:
             part = workspace("skinny", splits * m * n, x.device)
             _check(_fn("gemm_bf16", "mf_gemm_bf16_splitk")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
-                                                            _ptr(part), m, n, k, splits, per, EPI_SWIGLU, 0,
+                                                            _ptr(part), m, n, k, splits, per, EPI_SWIGLU, variant,
                                                             _stream()), f"gemm_bf16_splitk(swiglu) {m}x{n}x{k}")
             return
     _check(_fn("gemm_bf16", "mf_gemm_bf16")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf, m, n, k,

@@ -17,7 +17,6 @@ Kernel choice, for measurements (each overrides what `ops` would pick by shape):
 * MF_SKINNY_TARGET=n    blocks the K-split decode product aims at (default: one per CU)
 * MF_NO_FOLD=1          the RMS norm is a kernel of its own instead of being folded into the
                         product that follows it
-* MF_NO_BIG_SPLIT=1     prompt products never cut K over the 256 x 256 tiles
 """
 from __future__ import annotations
 
@@ -40,4 +39,3 @@ TIMING = _flag("MF_TIMING")
 ATTN_SPLITS = _int("MF_ATTN_SPLITS")
 SKINNY_TARGET = _int("MF_SKINNY_TARGET")
 NO_FOLD = _flag("MF_NO_FOLD")
-NO_BIG_SPLIT = _flag("MF_NO_BIG_SPLIT")

@@ -210,7 +210,7 @@ def test_gemm_f32(ops, m, n, k):
     close(acc, ref - b.double() + base.double(), 1e-5 * math.sqrt(k) / 8, 1e-5)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 6, 9, 12])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 6, 9, 12, 13, 15])
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES + [(2048, 512, 256), (1, 152064, 64), (64, 3584, 3584),
                                                  # at most 16 rows with K of 1536..4096: activations in registers
                                                  (1, 2100, 1536), (5, 2050, 2048), (8, 4001, 3584), (16, 2048, 4096),
@@ -223,11 +223,13 @@ def test_gemm_f32(ops, m, n, k):
                                                  # more than 64 rows but few tiles: K split over blocks
                                                  (200, 3584, 18944), (65, 1000, 1100), (512, 777, 2048),
                                                  # many rows, few big tiles, a long K: K split over 256 x 256 tiles
-                                                 (800, 300, 4096), (1030, 777, 6144)])
+                                                 (800, 300, 4096), (1030, 777, 6144),
+                                                 # tiles of 256 x 192 and 256 x 128 where the 256-wide ones leave CUs idle
+                                                 (2048, 4608, 512), (1100, 3584, 1024), (8192, 1000, 192)])
 def test_gemm_bf16(ops, variant, m, n, k):
     if variant and (m * n * k > 3e9):
         pytest.skip("large shape is covered by the default variant")
-    if variant == 12 and k % 64:
+    if variant >= 12 and k % 64:
         pytest.skip("the direct-to-LDS kernel takes K in multiples of 64")
     x, w, b = rnd((m, k), torch.bfloat16, 8), rnd((n, k), torch.bfloat16, 9, 0.05), rnd((n,), seed=10)
     ref = x.double() @ w.double().t() + b.double()
@@ -511,7 +513,7 @@ def test_gemm_bf16_wide_few_rows(ops, m, n, k):
     close(ob, ref, tol + 1e-3, 1e-2)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 9, 12])
+@pytest.mark.parametrize("variant", [0, 1, 2, 9, 12, 13])
 @pytest.mark.parametrize("m,nf,k", [(1, 176, 64), (8, 344, 128), (16, 32, 200), (17, 176, 64), (64, 1000, 344),
                                     (65, 232, 200), (300, 18944, 256), (130, 31, 72),
                                     (8, 1100, 1536), (3, 2100, 3584), (16, 1030, 4096), (1, 1024, 2048),
@@ -521,7 +523,7 @@ def test_gemm_bf16_wide_few_rows(ops, m, n, k):
                                     # more than 64 rows but few tiles: K split over blocks
                                     (100, 1000, 1024), (200, 512, 3584)])
 def test_gemm_bf16_swiglu(ops, variant, m, nf, k):
-    if variant == 12 and k % 64:
+    if variant >= 12 and k % 64:
         pytest.skip("the direct-to-LDS pipeline takes k in steps of 64")
     x = rnd((m, k), torch.bfloat16, 30)
     wg, wu = rnd((nf, k), torch.bfloat16, 31, 0.3), rnd((nf, k), torch.bfloat16, 32, 0.3)

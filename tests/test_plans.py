@@ -32,26 +32,30 @@ def test_skinny_plan_choices_at_the_model_shapes():
     assert ops.skinny_plan(12, 300, 8192, target_blocks=256, swiglu=True)[0] > 1      # too few weight rows for it
 
 
-def test_tile_split_plan():
-    for m, n, k in itertools.product((65, 128, 200, 512, 1024, 2048, 8192), (96, 3584, 4608, 37888),
-                                     (64, 256, 3584, 18944)):
-        splits, per, big = ops.tile_split_plan(m, n, k, target_blocks=256)
-        if splits == 1:
-            assert per == k and not big
+def test_tile_plan():
+    """The tile product's plan for every shape is one the kernels take: a K split only for the
+    variants that have one, in whole chunks of 256 with no empty part, the direct-to-LDS kernel only
+    for K in 64s, no SwiGLU epilogue on the 192-wide tile."""
+    for m, n, k, epi, aligned in itertools.product((65, 128, 200, 512, 1024, 2048, 5977, 8192), (96, 3584, 4608, 37888),
+                                                   (64, 200, 256, 3584, 18944), (ops.EPI_F32, ops.EPI_SWIGLU),
+                                                   (True, False)):
+        if epi == ops.EPI_SWIGLU and n % 64:
             continue
-        assert per % 256 == 0 and per >= 512
+        variant, splits, per = ops.tile_plan(m, n, k, epi, aligned and k % 8 == 0, n_cu=256)
+        assert variant in (2, 9, 12, 13, 15)
+        if variant in (12, 13, 15):
+            assert aligned and k % 64 == 0
+        assert variant != 15 or epi != ops.EPI_SWIGLU
+        if splits == 1:
+            assert per == k
+            continue
+        assert variant in (2, 12) and per % 256 == 0 and per >= 512
         assert splits * per >= k and (splits - 1) * per < k
-        if big:
-            t256 = ((m + 255) // 256) * ((n + 255) // 256)
-            assert m >= 768 and k % 64 == 0 and per >= 2048 and splits <= 8
+        if variant == 12:
+            assert m >= 768 and per >= 2048 and splits <= 8 and epi != ops.EPI_SWIGLU
         else:
             tiles = ((m + 127) // 128) * ((n + 127) // 128)
             assert tiles < 256 and splits * tiles <= 512
-    assert ops.tile_split_plan(2048, 3584, 18944, target_blocks=256) == (2, 9472, True)   # 112 big tiles, twice
-    assert ops.tile_split_plan(2048, 3584, 3584, target_blocks=256) == (1, 3584, False)   # K too short to split
-    assert ops.tile_split_plan(2048, 37888, 3584, target_blocks=256) == (1, 3584, False)
-    assert ops.tile_split_plan(200, 3584, 18944, target_blocks=256)[0::2] == (9, False)
-    assert ops.tile_split_plan(2048, 5120, 27648, target_blocks=256)[0::2] == (3, True)   # 160 big tiles: 480 blocks, two rounds
 
 
 def test_split_plan_of_the_32_bit_attention():
@@ -86,10 +90,18 @@ def test_plan_linear_names_the_kernels_of_the_model_shapes():
         assert p(64, 2 * inter, h, swiglu=True) == "panel_kernel" and p(64, 152064, h) == "panel_kernel"
         # the ring form needs K in whole chunks of 256 (29568 is 115.5 of them)
         assert p(64, h, inter, accumulate=True) == ("skinny_ring_kernel" if inter % 256 == 0 else "skinny_kernel")
-        assert p(2048, 2 * inter, h, swiglu=True) == "tile_dma_kernel"
+        assert p(2048, 2 * inter, h, swiglu=True) == "tile_dma_kernel<256>"
         assert p(40, qkv, h, normed=True) == ""                       # no fold above 16 rows: norm, then product
     assert p(8, 3584, 18944, accumulate=True) == "rolling16_kernel"
-    assert p(2048, 3584, 18944, accumulate=True) == "tile_dma_kernel(split K)"
+    # a prompt of 2,048 tokens at the 7B widths: 256-wide tiles of q|k|v (144) and o (112) would leave
+    # half of the 256 CUs idle, so 192 tiles of 256 x 192 and 224 of 256 x 128; down has K to split
+    assert p(2048, 4608, 3584, out_bf16=True) == "tile_dma_kernel<192>"
+    assert p(2048, 3584, 3584, accumulate=True) == "tile_dma_kernel<128>"
+    assert p(2048, 3584, 18944, accumulate=True) == "tile_dma_kernel<256>(split K)"
+    assert p(8192, 4608, 3584, out_bf16=True) == "tile_dma_kernel<192>"       # 768 tiles: three whole rounds
+    assert p(4096, 3584, 3584, accumulate=True) == "tile_dma_kernel<256>"     # 224 tiles: one round nearly full
+    assert p(4096, 37888, 3584, swiglu=True) == "tile_dma_kernel<256>"
+    assert p(2048, 3584, 3584 + 8, accumulate=True) == "tile_kernel<128,128>"      # K not in 64s
     assert p(200, 3584, 18944, accumulate=True) == "tile_kernel<128,128>(split K)"
     # other widths: multiples of 256 that are instantiated take the register-resident kernel, the
     # rest the rolling one; unaligned operands the guarded ones
