@@ -14,6 +14,7 @@ before, to a plain streaming read and to a register-resident loop of matrix-core
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import statistics
 import sys
@@ -257,10 +258,21 @@ def main() -> int:
     breakdown = kernel_breakdown(eng, cfg, a.batch, a.prompt_max) if a.breakdown else None
     if points_on:
         points["prefill_512"] = round(512 / run_prefill(eng, cfg, 512, repeats=3), 1)
-        # long contexts run in a cache of their own on the same weights
-        long_eng = Engine(llm.model, max_tokens=8 * 32768, max_seqs=8)
+        # long contexts: 8 sequences of up to 32,768 tokens, in the same cache where it holds them,
+        # else in one of their own on the same weights (the first one is given back before)
+        need = 8 * 32768
+        long_eng = eng
+        if eng.capacity_tokens() < need:
+            from minfer_amd.engine.engine import tokens_that_fit
+            llm.engine = eng = None
+            gc.collect()
+            torch.cuda.empty_cache()
+            long_eng = Engine(llm.model, max_tokens=min(need, tokens_that_fit(llm.model)), max_seqs=8)
         points["prefill_16384"] = round(16384 / run_prefill(long_eng, cfg, 16384, repeats=2), 1)
         for ctx_max, tag in ((16384, "16k"), (30000, "30k")):
+            if long_eng.capacity_tokens() < 8 * (ctx_max + 64 + half[0] + half[1]):
+                points[f"decode_b8_ctx{tag}"] = None         # the memory left by the weights does not hold it
+                continue
             r = run_decode(long_eng, cfg, 8, ctx_max, half[0], half[1], not a.no_graph, elem, seed=3)
             points[f"decode_b8_ctx{tag}"] = round(r["tok_s"], 1)
     flops = prefill_flops(cfg, a.prefill_tokens)
