@@ -115,6 +115,19 @@ __device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[TM][TN], const flo
     }
 }
 
+// Tile number -> (row of tiles, column of tiles).  The tiles are numbered in bands of 8 rows of
+// tiles, down a band's rows first: 32 neighbouring numbers (what an XCD has in flight, see the
+// kernels) are then 8 x 4 tiles, which share 12 operand panels between them (a whole column of
+// 32 tile rows would share 33).
+__device__ __forceinline__ void tile_position(int tile, int tiles_m, int tiles_n, int& bm, int& bn) {
+  constexpr int BAND = 8;
+  const int band = tile / (BAND * tiles_n), first = band * BAND;
+  const int rows = min(tiles_m - first, BAND);
+  const int in_band = tile - band * BAND * tiles_n;
+  bm = first + in_band % rows;
+  bn = in_band / rows;
+}
+
 // ------------------------------------------------------------------ tiled kernel
 // LDS row stride is BK + 8 elements (144 bytes for BK 64, 80 for BK 32): conflict-free b128 reads
 template <int BM, int BN, int WM, int WN, int BK, bool VEC>
@@ -143,15 +156,16 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void tile_kernel(const 
   bf16* Ws = As + 2 * BM * LDS_LD;                        // [2][BN][LDS_LD]
 
   // Workgroups go to the 8 XCDs in turn, each with an L2 of its own: give every XCD one
-  // contiguous eighth of the tiles, walking down M first, so that a W tile is fetched by one
-  // L2 only and the tiles an XCD has in flight share their W rows.
+  // contiguous eighth of the tile numbers, so that the tiles an XCD has in flight are neighbours
+  // and share their operands' rows in its L2.
   int tile = blockIdx.x;
   if (xcd_remap) {
     const int n_tiles = gridDim.x, per = n_tiles / 8, rem = n_tiles % 8;
     const int x = blockIdx.x % 8, qq = blockIdx.x / 8;
     tile = x * per + min(x, rem) + qq;
   }
-  const int bm = tile % tiles_m, bn = tile / tiles_m;
+  int bm, bn;
+  tile_position(tile, tiles_m, gridDim.x / tiles_m, bm, bn);
   const int m0 = bm * BM, n0 = bn * BN;
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int wm = (wid % (BM / WM)) * WM, wn = (wid / (BM / WM)) * WN;
@@ -319,7 +333,8 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
     const int x = blockIdx.x % 8, qq = blockIdx.x / 8;
     tile = x * per + min(x, rem) + qq;
   }
-  const int bm = tile % tiles_m, bn = tile / tiles_m;
+  int bm, bn;
+  tile_position(tile, tiles_m, gridDim.x / tiles_m, bm, bn);
   const int m0 = bm * DMA_BM, n0 = bn * BN;
   const int lane = threadIdx.x & 63;
   const int wid = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
