@@ -9,7 +9,12 @@
 // 32-bit, probabilities are rounded to bfloat16 for the second product.
 //
 // A block (4 waves) owns 128 consecutive query tokens of one sequence and one query head;
-// each wave 32 of them.  Per cache page (64 keys): K goes to LDS as stored and V^T as rows of 64
+// each wave 32 of them.  The time of a prompt's attention is that of its last tile, whose block
+// walks every page of the sequence one after the other, so the host may give a tile to several
+// blocks, which take its pages in turn (block s of n the pages first + s, first + s + n, ...):
+// each leaves its maxima, sums and output in `parts`, counts itself in, and the one that comes
+// last adds all of them up, in the order of s, and writes the result.
+// Per cache page (64 keys): K goes to LDS as stored and V^T as rows of 64
 // keys (the cache keeps a page of V transposed in two halves, [2][head_dim][32 keys], which the
 // copy puts side by side), into one of two buffers.
 //   S^T[key][q] = K Q^T      32x32x16 MFMA, A = K rows from LDS, B = Q held in registers
@@ -33,8 +38,9 @@ __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ page_table, int pt_stride, const int* __restrict__ cu_seqlens,
     const int* __restrict__ start_pos, const int* __restrict__ tile_seq,
-    const int* __restrict__ tile_q0, bf16* __restrict__ out, int n_tiles, int nh, int nk, float scale, int window,
-    int pair_slots) {
+    const int* __restrict__ tile_q0, const int* __restrict__ tile_share, float* __restrict__ parts,
+    int* __restrict__ arrived, int max_shares, bf16* __restrict__ out, int n_tiles, int nh, int nk, float scale,
+    int window, int pair_slots) {
   constexpr int HD = NKS * 16;
   constexpr int NDT = (NKS + 1) / 2;          // 32-wide output tiles over head_dim
   constexpr int HDP = NDT * 32;
@@ -56,6 +62,10 @@ __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
   const int tile = item / nh;
   const int b = tile_seq[tile], q0 = tile_q0[tile];
   const int h = item % nh, hk = h / (nh / nk);
+  // tile_share[tile]: which of how many blocks of these queries this one is, and the number of the
+  // queries' slot in `parts` and `arrived`: share + 256 * shares + 65536 * slot (0 shares: alone)
+  const int share_word = tile_share ? tile_share[tile] : 0;
+  const int share = share_word & 255, n_shares = max(1, (share_word >> 8) & 255), share_slot = share_word >> 16;
   const int tok0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - tok0, start = start_pos[b];
   const int* pt = page_table + (size_t)b * pt_stride;
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
@@ -149,16 +159,18 @@ __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
   };
   // Two buffers, one barrier a page: while page i is multiplied from one buffer, page i + 1
   // (fetched a step ago) goes from registers into the other and page i + 2 sets out from memory.
-  const int page_first = key_lo / KT, page_last = blk_p_hi / KT;
-  fetch(page_first);
-  stage(0);
-  if (page_first < page_last) fetch(page_first + 1);
+  const int page_first = key_lo / KT + share, page_last = blk_p_hi / KT;
+  if (page_first <= page_last) {
+    fetch(page_first);
+    stage(0);
+    if (page_first + n_shares <= page_last) fetch(page_first + n_shares);
+  }
   __syncthreads();
   int buf = 0;
-  for (int page_i = page_first; page_i <= page_last; ++page_i, buf ^= 1) {
-    if (page_i < page_last) {
+  for (int page_i = page_first; page_i <= page_last; page_i += n_shares, buf ^= 1) {
+    if (page_i + n_shares <= page_last) {
       stage(buf ^ 1);             // every wave is past the barrier behind its last read of that buffer
-      if (page_i + 1 < page_last) fetch(page_i + 2);
+      if (page_i + 2 * n_shares <= page_last) fetch(page_i + 2 * n_shares);
     }
     const bf16* Ks = kv + buf * BUF;
     const bf16* Vt = Ks + KT * K_LD;
@@ -241,6 +253,55 @@ __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
     __syncthreads();
   }
 
+  if (n_shares > 1) {
+    // This block's part goes to memory (lane-major: value v of thread t at v * 256 + t), written
+    // through and read past the caches, since the blocks of a tile may sit behind different L2s.
+    constexpr int XW = NDT * 16 + 2;
+    float* slot0 = parts + ((size_t)share_slot * nh + h) * max_shares * XW * 256 + tid;
+    float* mine = slot0 + (size_t)share * XW * 256;
+    __hip_atomic_store(mine, m_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(mine + 256, l_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        __hip_atomic_store(mine + (2 + dt * 16 + r) * 256, oacc[dt][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __builtin_amdgcn_s_waitcnt(0);                       // this wave's stores have reached memory
+    __syncthreads();
+    int* last = reinterpret_cast<int*>(smem);            // (the page buffers are free behind the loop's last barrier)
+    if (tid == 0) {
+      int* count = arrived + share_slot * nh + h;
+      const int before = __hip_atomic_fetch_add(count, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      if (before == n_shares - 1) __hip_atomic_store(count, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);   // as it was found
+      *last = before == n_shares - 1;
+    }
+    __syncthreads();
+    const bool is_last = *last != 0;
+    __syncthreads();                                     // the word is in the output staging's place
+    if (!is_last) return;
+    m_run = -INFINITY;
+    l_run = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+    for (int s = 0; s < n_shares; ++s) {                 // every part, this block's own too, in the order of s
+      const float* theirs = slot0 + (size_t)s * XW * 256;
+      const float m_o = __hip_atomic_load(theirs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      const float l_o = __hip_atomic_load(theirs + 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      const float m_new = fmaxf(m_run, m_o);
+      const float c_mine = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
+      const float c_theirs = (m_o == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_o - m_new);
+      l_run = l_run * c_mine + l_o * c_theirs;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          oacc[dt][r] = oacc[dt][r] * c_mine +
+                        __hip_atomic_load(theirs + (2 + dt * 16 + r) * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) * c_theirs;
+      m_run = m_new;
+    }
+  }
   // normalise; O^T regs: d = 32 dt + 8 (r / 4) + 4 hf + r % 4 for this lane's query
   const float l_tot = l_run + __shfl_xor(l_run, 32, MF_WAVE);
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
@@ -270,8 +331,9 @@ __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
 
 template <int NKS>
 int launch(const bf16* q, const bf16* kc, const bf16* vc, const int* page_table, int pt_stride,
-           const int* cu_seqlens, const int* start_pos, const int* tile_seq, const int* tile_q0, bf16* out,
-           int n_tiles, int nh, int nk, float scale, int window, hipStream_t stream) {
+           const int* cu_seqlens, const int* start_pos, const int* tile_seq, const int* tile_q0,
+           const int* tile_share, float* parts, int* arrived, int max_shares, bf16* out, int n_tiles, int nh, int nk,
+           float scale, int window, hipStream_t stream) {
   constexpr int HD = NKS * 16, HDP = ((NKS + 1) / 2) * 32, K_LD = HD + 8;
   static int n_cu = 0;                 // compute units of the device (asked once)
   if (n_cu == 0) {
@@ -293,24 +355,34 @@ int launch(const bf16* q, const bf16* kc, const bf16* vc, const int* page_table,
     configured = true;
   }
   kern<<<n_tiles * nh, 256, smem, stream>>>(q, kc, vc, page_table, pt_stride, cu_seqlens, start_pos, tile_seq,
-                                            tile_q0, out, n_tiles, nh, nk, scale, window, pair_slots);
+                                            tile_q0, tile_share, parts, arrived, max_shares, out, n_tiles, nh, nk, scale,
+                                            window, tile_share ? 0 : pair_slots);
   return mf_launch_status();
 }
 
 }  // namespace
 
 // tile_seq[i], tile_q0[i]: sequence (index in the step's batch) and first new token of the
-// i-th block of 128 query tokens; the host lists them.
+// i-th block of 128 query tokens; the host lists them, longest first.  tile_share (or null: every
+// block has its queries to itself): entry i is share + 256 * shares + 65536 * slot, block `share`
+// of `shares` (at most max_shares, which is at most 255) that take the pages of these queries in
+// turn; their parts meet in parts[slot][head][max_shares][mf_attn_prefill_part_floats(hd)] and
+// arrived[slot][head], which is zero before the call and after it.  Calls that use the same parts and arrived run on one stream.
+MF_API int mf_attn_prefill_part_floats(int hd) { return (((hd / 16 + 1) / 2) * 16 + 2) * 256; }
+
 MF_API int mf_attn_prefill_bf16(const void* q, const void* kc, const void* vc, const int* page_table,
                                 int pt_stride, const int* cu_seqlens, const int* start_pos,
-                                const int* tile_seq, const int* tile_q0, void* out, int n_tiles, int nh,
-                                int nk, int hd, float scale, int window, hipStream_t stream) {
+                                const int* tile_seq, const int* tile_q0, const int* tile_share, float* parts,
+                                int* arrived, int max_shares, void* out, int n_tiles, int nh, int nk, int hd,
+                                float scale, int window, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (hd % 16 != 0 || hd < 16 || hd > 256 || nk <= 0 || nh % nk != 0) return (int)hipErrorInvalidValue;
+  if (tile_share && (!parts || !arrived || max_shares < 1 || max_shares > 255)) return (int)hipErrorInvalidValue;
 #define MF_CASE(E)                                                                                        \
   case E:                                                                                                 \
     return launch<E>((const bf16*)q, (const bf16*)kc, (const bf16*)vc, page_table, pt_stride, cu_seqlens, \
-                     start_pos, tile_seq, tile_q0, (bf16*)out, n_tiles, nh, nk, scale, window, stream);
+                     start_pos, tile_seq, tile_q0, tile_share, parts, arrived, max_shares, (bf16*)out, n_tiles, nh, \
+                     nk, scale, window, stream);
   switch (hd / 16) {
     MF_CASE(1) MF_CASE(2) MF_CASE(3) MF_CASE(4) MF_CASE(5) MF_CASE(6) MF_CASE(7) MF_CASE(8)
     MF_CASE(9) MF_CASE(10) MF_CASE(11) MF_CASE(12) MF_CASE(13) MF_CASE(14) MF_CASE(15) MF_CASE(16)

@@ -56,3 +56,38 @@ class StepContext:
             both = torch.tensor([seqs, starts], dtype=torch.int32).to(self.token_ids.device)
             self._memo[key] = (both[0], both[1])
         return self._memo[key]
+
+    def shared_query_tiles(self, block: int, page: int, window: int, load_of, max_shares: int):
+        """(tile_seq, tile_q0, tile_share, n_slots): as `query_tiles`, but a block of queries with
+        many pages of keys is listed several times, once for each of the workgroups that are to
+        take its pages in turn.  `load_of(total_pages)` gives the number of pages one workgroup
+        should get at most; entry i of tile_share is share + 256 * shares + 65536 * slot (0 for a
+        block listed once), slots numbering the blocks that are shared.  None where no block needs
+        sharing."""
+        key = ("shared_query_tiles", block, page, window, max_shares)
+        if key not in self._memo:
+            tiles = []
+            for b, n in enumerate(self.host_new):
+                first = self.host_start[b] if self.host_start else 0
+                for q0 in range(0, n, block):
+                    last_key = first + min(q0 + block, n) - 1
+                    first_key = max(0, first + q0 - window + 1) if window > 0 else 0
+                    tiles.append((last_key // page - first_key // page + 1, b, q0))
+            target = max(1, int(load_of(sum(t[0] for t in tiles))))
+            entries, n_slots = [], 0
+            for pages, b, q0 in tiles:
+                shares = min(max_shares, (pages + target - 1) // target)
+                if shares <= 1:
+                    entries.append((pages, b, q0, 0))
+                    continue
+                for s in range(shares):
+                    entries.append(((pages - s + shares - 1) // shares, b, q0, s + 256 * shares + 65536 * n_slots))
+                n_slots += 1
+            if n_slots == 0:
+                self._memo[key] = None
+            else:
+                entries.sort(key=lambda e: -e[0])                         # longest first
+                cols = torch.tensor([[e[1] for e in entries], [e[2] for e in entries], [e[3] for e in entries]],
+                                    dtype=torch.int32).to(self.token_ids.device)
+                self._memo[key] = (cols[0], cols[1], cols[2], n_slots)
+        return self._memo[key]

@@ -18,6 +18,8 @@ from ..cache.paged import v_page_shape
 PAGE = 64          # tokens per cache page (MF_PAGE in csrc/common.h)
 HAVE_PREFILL_ATTENTION = True
 PREFILL_BLOCK = 128     # query tokens per workgroup of the prompt attention kernel
+PREFILL_MAX_SHARES = 8  # workgroups that may take the pages of one such block of queries in turn
+PREFILL_MIN_PAGES = 4   # ... each with at least this many pages
 EPI_F32, EPI_ACC_F32, EPI_BF16, EPI_SWIGLU = 0, 1, 2, 3
 
 
@@ -71,8 +73,9 @@ _PROTOTYPES = {
                                      c_int, c_float, c_int, c_int, c_int, _P],
     },
     "attn_prefill_bf16": {
-        "mf_attn_prefill_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int,
+        "mf_attn_prefill_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, c_int,
                                  c_int, c_float, c_int, _P],
+        "mf_attn_prefill_part_floats": [c_int],
     },
     "sampling": {
         "mf_argmax": [_P, c_int, c_int, c_int, _P, _P, c_int, _P],
@@ -187,6 +190,25 @@ def workspace(tag: str, n_floats: int, device) -> torch.Tensor:
         w = torch.empty(max(n_floats, 1 << 16), dtype=torch.float32, device=device)
         _workspaces[key] = w
     return w
+
+
+_counters: Dict[Tuple[str, int], torch.Tensor] = {}
+
+
+def _zeroed_counters(tag: str, n: int, device) -> torch.Tensor:
+    """int32 counters for kernels whose workgroups count themselves in and leave the counters at
+    zero again: zero when made, kept per (tag, device), made anew (and the generation moved on)
+    when more are needed."""
+    global _workspace_generation
+    dev = torch.device(device)
+    key = (tag, dev.index if dev.index is not None else torch.cuda.current_device())
+    c = _counters.get(key)
+    if c is None or c.numel() < n:
+        if c is not None:
+            _workspace_generation += 1
+        c = torch.zeros(max(n, 1024), dtype=torch.int32, device=dev)
+        _counters[key] = c
+    return c
 
 
 def workspace_generation() -> int:
@@ -684,11 +706,27 @@ def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pa
     if ctx.max_len > page_table.shape[1] * PAGE or page_table.shape[0] != ctx.n_seqs:
         raise KernelError(f"attention: page table {tuple(page_table.shape)} does not cover "
                           f"{ctx.n_seqs} sequences of up to {ctx.max_len} positions")
-    tile_seq, tile_q0 = ctx.query_tiles(PREFILL_BLOCK)
+    # The kernel's time is that of the block with the most pages (the last queries of the longest
+    # prompt): blocks of queries with more pages than a workgroup's even share of all of them (two
+    # workgroups fit a CU) are given to several workgroups, which take the pages in turn.
+    window = int(window or 0)
+    slots = 2 * cu_count()
+    shared = None if tuning.NO_SHARED_PAGES else ctx.shared_query_tiles(
+        PREFILL_BLOCK, PAGE, window, lambda pages: max(PREFILL_MIN_PAGES, -(-pages * n_heads // slots)),
+        PREFILL_MAX_SHARES)
+    if shared is None:
+        tile_seq, tile_q0 = ctx.query_tiles(PREFILL_BLOCK)
+        tile_share = parts = arrived = None
+    else:
+        tile_seq, tile_q0, tile_share, n_slots = shared
+        part = _fn("attn_prefill_bf16", "mf_attn_prefill_part_floats")(head_dim)
+        parts = workspace("prefill_parts", n_slots * n_heads * PREFILL_MAX_SHARES * part, q.device)
+        arrived = _zeroed_counters("prefill_arrived", n_slots * n_heads, q.device)
     _check(_fn("attn_prefill_bf16", "mf_attn_prefill_bf16")(
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(ctx.cu_seqlens),
-        _ptr(ctx.start_pos), _ptr(tile_seq), _ptr(tile_q0), _ptr(out), tile_seq.numel(), n_heads,
-        n_kv_heads, head_dim, float(scale), int(window or 0), _stream()), "attn_prefill_bf16")
+        _ptr(ctx.start_pos), _ptr(tile_seq), _ptr(tile_q0), _ptr(tile_share), _ptr(parts), _ptr(arrived),
+        PREFILL_MAX_SHARES, _ptr(out), tile_seq.numel(), n_heads, n_kv_heads, head_dim, float(scale), window,
+        _stream()), "attn_prefill_bf16")
 
 
 # ------------------------------------------------------------------ sampling

@@ -465,6 +465,37 @@ def test_attn_prefill(ops, nh, nk, hd, window):
     close(out, tok.double(), 2e-2, 2e-2)
 
 
+@pytest.mark.parametrize("nh,nk,hd,window", [(4, 2, 128, 0), (3, 1, 64, 0), (2, 2, 256, 0), (4, 1, 128, 900), (5, 5, 80, 0)])
+def test_attn_prefill_shared_pages(ops, nh, nk, hd, window):
+    """Long sequences with few heads: a block of queries has far more pages than a workgroup's
+    share of all of them, so its pages go to up to eight workgroups in turn whose parts the last
+    one adds up (one sequence continues from 600 cached tokens; the short one stays whole)."""
+    new, start = [1500, 260, 40], [600, 0, 0]
+    q, kc, vc, table, ctx_on = prefill_case(nh, nk, hd, new, start, 23)
+    shared = ctx_on("cpu").shared_query_tiles(ops.PREFILL_BLOCK, ops.PAGE, window,
+                                              lambda pages: max(ops.PREFILL_MIN_PAGES, -(-pages * nh // 512)),
+                                              ops.PREFILL_MAX_SHARES)
+    assert shared is not None
+    words = shared[2].tolist()
+    assert max((w >> 8) & 255 for w in words) == (8 if window == 0 else 5)     # 33 pages, or the window's 16
+    by_slot = {}
+    for w in words:
+        if w:
+            by_slot.setdefault(w >> 16, []).append((w & 255, (w >> 8) & 255))
+    assert sorted(by_slot) == list(range(shared[3]))
+    for got in by_slot.values():                                  # every share of a slot once
+        assert sorted(s for s, _ in got) == list(range(got[0][1])) and len({n for _, n in got}) == 1
+    scale = 1.0 / math.sqrt(hd)
+    ref = torch.empty(q.shape, dtype=torch.float64)
+    plain_ops.attn_prefill(q, kc, vc, table, ctx_on("cpu"), ref, nh, nk, hd, scale, window)
+    out = torch.empty(q.shape, dtype=torch.bfloat16, device=DEV)
+    ops.attn_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), ctx_on(DEV), out, nh, nk, hd, scale, window)
+    close(out, ref, 1.5e-2, 1.5e-2)
+    again = torch.empty(q.shape, dtype=torch.bfloat16, device=DEV)
+    ops.attn_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), ctx_on(DEV), again, nh, nk, hd, scale, window)
+    assert torch.equal(out, again), "two runs differ"
+
+
 def test_attn_prefill_far_key_and_window_edge(ops):
     """One key's score is made to stand out for one query: the output is that key's V row
     when the key is visible (anywhere in a long prompt, across pages), and is not when the
