@@ -58,7 +58,7 @@ class StepContext:
         return self._memo[key]
 
     def shared_query_tiles(self, block: int, page: int, window: int, load_of, max_shares: int):
-        """(tile_seq, tile_q0, tile_share, n_slots): as `query_tiles`, but a block of queries with
+        """(tile_seq, tile_q0, tile_share, n_slots, most shares): as `query_tiles`, but a block of queries with
         many pages of keys is listed several times, once for each of the workgroups that are to
         take its pages in turn.  `load_of(total_pages)` gives the number of pages one workgroup
         should get at most; entry i of tile_share is share + 256 * shares + 65536 * slot (0 for a
@@ -74,9 +74,10 @@ class StepContext:
                     first_key = max(0, first + q0 - window + 1) if window > 0 else 0
                     tiles.append((last_key // page - first_key // page + 1, b, q0))
             target = max(1, int(load_of(sum(t[0] for t in tiles))))
-            entries, n_slots = [], 0
+            entries, n_slots, most = [], 0, 1
             for pages, b, q0 in tiles:
                 shares = min(max_shares, (pages + target - 1) // target)
+                most = max(most, shares)
                 if shares <= 1:
                     entries.append((pages, b, q0, 0))
                     continue
@@ -89,5 +90,5 @@ class StepContext:
                 entries.sort(key=lambda e: -e[0])                         # longest first
                 cols = torch.tensor([[e[1] for e in entries], [e[2] for e in entries], [e[3] for e in entries]],
                                     dtype=torch.int32).to(self.token_ids.device)
-                self._memo[key] = (cols[0], cols[1], cols[2], n_slots)
+                self._memo[key] = (cols[0], cols[1], cols[2], n_slots, most)
         return self._memo[key]

@@ -718,14 +718,14 @@ def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pa
         tile_seq, tile_q0 = ctx.query_tiles(PREFILL_BLOCK)
         tile_share = parts = arrived = None
     else:
-        tile_seq, tile_q0, tile_share, n_slots = shared
+        tile_seq, tile_q0, tile_share, n_slots, most_shares = shared
         part = _fn("attn_prefill_bf16", "mf_attn_prefill_part_floats")(head_dim)
-        parts = workspace("prefill_parts", n_slots * n_heads * PREFILL_MAX_SHARES * part, q.device)
+        parts = workspace("prefill_parts", n_slots * n_heads * most_shares * part, q.device)
         arrived = _zeroed_counters("prefill_arrived", n_slots * n_heads, q.device)
     _check(_fn("attn_prefill_bf16", "mf_attn_prefill_bf16")(
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(ctx.cu_seqlens),
         _ptr(ctx.start_pos), _ptr(tile_seq), _ptr(tile_q0), _ptr(tile_share), _ptr(parts), _ptr(arrived),
-        PREFILL_MAX_SHARES, _ptr(out), tile_seq.numel(), n_heads, n_kv_heads, head_dim, float(scale), window,
+        most_shares if shared is not None else 1, _ptr(out), tile_seq.numel(), n_heads, n_kv_heads, head_dim, float(scale), window,
         _stream()), "attn_prefill_bf16")
 
 

@@ -482,7 +482,7 @@ def test_attn_prefill_shared_pages(ops, nh, nk, hd, window):
     for w in words:
         if w:
             by_slot.setdefault(w >> 16, []).append((w & 255, (w >> 8) & 255))
-    assert sorted(by_slot) == list(range(shared[3]))
+    assert sorted(by_slot) == list(range(shared[3])) and shared[4] == max((w >> 8) & 255 for w in words)
     for got in by_slot.values():                                  # every share of a slot once
         assert sorted(s for s, _ in got) == list(range(got[0][1])) and len({n for _, n in got}) == 1
     scale = 1.0 / math.sqrt(hd)
