@@ -11,7 +11,7 @@ command line (`GenParams`, src/main.rs:42-70 of yusiwen/minfer).
 """
 from __future__ import annotations
 
-from typing import Any, Dict, List, Optional, Sequence, Union
+from typing import Any, Dict, Optional, Sequence, Union
 
 from .cache.paged import PAGE
 from .engine import Engine, GenerationResult, generate, load_model, random_model

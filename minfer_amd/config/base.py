@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import json
 import os
-from typing import Any, Callable, Dict, Optional
+from typing import Any, Dict, Optional
 
 
 class ConfigError(ValueError):

@@ -11,7 +11,7 @@ sequence index as data.  There is no padding: only the tokens given are run.
 from __future__ import annotations
 
 from collections import OrderedDict
-from typing import Dict, List, Optional, Sequence, Union
+from typing import Dict, Optional, Sequence, Union
 
 import numpy as np
 import torch

@@ -8,12 +8,12 @@ graph.rs:126-138) -> float32 logits.
 """
 from __future__ import annotations
 
-from typing import Callable, Dict, List, Optional
+from typing import Callable, Dict
 
 import torch
 
 from ..kernels import ops
-from ..parts.base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, Normed, Runtime, make_part,
+from ..parts.base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, Runtime, make_part,
                           normed_input)
 from ..parts.spec import BlockSpec, ModelSpec
 from ..weights.loader import TensorSpec

@@ -13,7 +13,7 @@ the run type and *add* their result into `h` in 32-bit.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, Optional
+from typing import Callable, Dict, Optional
 
 import torch
 

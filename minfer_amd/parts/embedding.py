@@ -9,7 +9,7 @@ import torch
 
 from ..kernels import ops
 from ..weights.loader import TensorSpec
-from .base import Embedding, Head, Normed, register_embedding, register_head
+from .base import Embedding, Head, register_embedding, register_head
 from .linear import Linear
 
 

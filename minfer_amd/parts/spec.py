@@ -13,7 +13,7 @@ src/graph/builder.rs:79-286 of yusiwen/minfer) inside one loop over layers
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional, Tuple
+from typing import Any, Dict, Optional, Tuple
 
 
 @dataclass(frozen=True)
