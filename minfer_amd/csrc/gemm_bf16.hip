@@ -1567,8 +1567,10 @@ TilePlan plan_tiles(int M, int N, int K, bool dma_ok, int epi, int n_cu) {
   };
   if (dma_ok) {
     offer(12, 1, K, rounds_us(tiles(256, 256), cu, 1.75, nkt) + start_us + epi_us);
-    offer(13, 1, K, rounds_us(tiles(256, 128), cu, 1.00, nkt) + start_us + epi_us);
-    if (epi != EPI_SWIGLU) offer(15, 1, K, rounds_us(tiles(256, 192), cu, 1.35, nkt) + start_us + epi_us);
+    // (the narrower tiles must promise 4 % to be taken: where the estimates are that close, the
+    // 256-wide tile has measured the faster)
+    offer(13, 1, K, 1.04 * (rounds_us(tiles(256, 128), cu, 1.00, nkt) + start_us + epi_us));
+    if (epi != EPI_SWIGLU) offer(15, 1, K, 1.04 * (rounds_us(tiles(256, 192), cu, 1.35, nkt) + start_us + epi_us));
     // many rows against few weight rows and a long K (the down product of a prompt): K cut over
     // the big tiles, each part at least 2,048 of K
     if (epi != EPI_SWIGLU && M >= 768)
