@@ -115,3 +115,43 @@ def test_plan_linear_names_the_kernels_of_the_model_shapes():
     for ns in ops.STATIONARY_NS:
         assert ops.stationary_shape(4096, 256 * ns, True) and p(2, 4096, 256 * ns, normed=True) != ""
     assert not ops.stationary_shape(4096, 256 * 5) and not ops.stationary_shape(4096, 256 * 33, True)
+
+
+def test_shared_query_tiles_cover_every_page_once():
+    """The host's list of workgroups for the prompt attention: every block of 128 queries appears
+    with all its shares or alone, a share's pages are at most the load asked for (unless the cap on
+    shares binds), the longest entries come first, and without long blocks there is no list."""
+    import torch
+    from minfer_amd.engine.batch import StepContext
+
+    def ctx(new, start):
+        n = sum(new)
+        return StepContext(cache=None, n_tokens=n, n_seqs=len(new), token_ids=torch.zeros(n, dtype=torch.int32),
+                           positions=None, seq_of_tok=None, cu_seqlens=None, start_pos=None, slot_ids=None,
+                           logit_rows=None, page_tables={}, max_len=0, max_new=max(new), all_decode=False,
+                           host_new=list(new), host_start=list(start))
+
+    for new, start, window, load, cap in (([1500, 260, 40], [600, 0, 0], 0, 4, 8), ([64], [30000], 0, 26, 8),
+                                          ([2048], [0], 0, 15, 8), ([300, 17], [900, 5000], 700, 4, 3)):
+        got = ctx(new, start).shared_query_tiles(128, 64, window, lambda pages: load, cap)
+        assert got is not None
+        seqs, q0s, words, n_slots, most = (x.tolist() if hasattr(x, "tolist") else x for x in got)
+        tiles = {}
+        for b, q0, w in zip(seqs, q0s, words):
+            tiles.setdefault((b, q0), []).append(w)
+        assert sorted(tiles) == sorted((b, q0) for b, n in enumerate(new) for q0 in range(0, n, 128))
+        slots = set()
+        for (b, q0), ws in tiles.items():
+            last_key = start[b] + min(q0 + 128, new[b]) - 1
+            first_key = max(0, start[b] + q0 - window + 1) if window else 0
+            pages = last_key // 64 - first_key // 64 + 1
+            if ws == [0]:
+                assert pages <= load
+                continue
+            n = (ws[0] >> 8) & 255
+            assert sorted(w & 255 for w in ws) == list(range(n)) and {(w >> 8) & 255 for w in ws} == {n}
+            assert len({w >> 16 for w in ws}) == 1 and 2 <= n <= min(cap, most)
+            assert n == cap or -(-pages // n) <= load
+            slots.add(ws[0] >> 16)
+        assert slots == set(range(n_slots))
+    assert ctx([100, 30], [0, 0]).shared_query_tiles(128, 64, 0, lambda pages: 4, 8) is None
