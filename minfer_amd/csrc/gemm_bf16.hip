@@ -1056,7 +1056,10 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
   bf16x8 w[NT][RING];
   const bf16* wrow[NT];          // this lane's rows in the next item
   const bf16* wcur[NT];          // and in the current one (used when RING < NS)
-  const int item = 0;
+  // The first item's loads are asked for without a condition (every block has an item: the grid is
+  // no larger than the units to share): a load behind a branch makes the compiler count, for every
+  // wait after it, with the path that has fewer loads in flight, and the prologue would wait for
+  // the activations until most of the first weights have arrived as well.
   auto first_loads = [&](int j) {
     wcur[j] = Wp + (size_t)lane_wrow(c_begin, j) * ldw + k0;
 #pragma unroll
@@ -1101,7 +1104,7 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
         x[s][1] = *reinterpret_cast<const float4*>(xrow + s * 32 + 4);
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (item < n_items) first_loads(0);
+      first_loads(0);
       __builtin_amdgcn_sched_barrier(0);
       *reinterpret_cast<float4*>(&gs[ge0]) = gt0;
       *reinterpret_cast<float4*>(&gs[ge1]) = gt1;
@@ -1140,7 +1143,7 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
         __builtin_amdgcn_sched_barrier(0);
       }
       asm volatile("" : "+s"(Wp), "+v"(afr[NS - 1]));     // no weights before the activations are in place
-      if (item < n_items) first_loads(0);
+      first_loads(0);
     }
     ss += __shfl_xor(ss, 16);
     ss += __shfl_xor(ss, 32);
@@ -1150,12 +1153,10 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
     const bf16* arow = (const bf16*)Av + (size_t)min(r16, M - 1) * lda + k0;
 #pragma unroll
     for (int s = 0; s < NS; ++s) afr[s] = *reinterpret_cast<const bf16x8*>(arow + s * 32);
-    if (item < n_items) first_loads(0);
+    first_loads(0);
   }
-  if (item < n_items) {
 #pragma unroll
-    for (int j = 1; j < NT; ++j) first_loads(j);
-  }
+  for (int j = 1; j < NT; ++j) first_loads(j);
   for (int it = 0; it < n_items; ++it) {
     // The loop body has no branch, so that the compiler can count the loads in flight and wait
     // for the oldest one only: behind the last item the loads go to the head of the matrix,
