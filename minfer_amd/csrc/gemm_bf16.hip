@@ -879,6 +879,18 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
   floatx4 acc[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // The epilogue's place of this lane: wave w adds up the sums of activation rows
+  // [w 64 / COLS, (w + 1) 64 / COLS), every wave one pass at the same time.  Where the product is
+  // added to what the output holds, the old value is asked for here, in front of the whole stream:
+  // behind it, its way from memory would be the kernel's tail, once per pass.
+  constexpr int ROWS_PER_PASS = 64 / COLS;
+  static_assert(NW * ROWS_PER_PASS >= 16, "a pass for every activation row");
+  const int e_c = lane % COLS;
+  const int e_n = tile_row(e_c >> 4) + (e_c & 15);
+  const int e_m = wid * ROWS_PER_PASS + lane / COLS;
+  const bool e_mine = e_m < M && e_n < N && (PAIR || e_c < rpb);
+  float c_old = 0.f;
+  if (epi == EPI_ACC_F32 && e_mine) c_old = ((const float*)C)[(size_t)e_m * ldc + e_n];
   const int R = T / S, rem = T % S;
   if (R == 0) {       // a slice shorter than the registers hold: step by step
     for (int s = 0; s < T; ++s) {
@@ -935,31 +947,25 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wid][(lane >> 4) * 4 + r][j * 16 + r16] = acc[j][r];
   __syncthreads();
-  if (wid != 0) return;
   if (epi == EPI_SWIGLU) {
     if constexpr (PAIR && NT == 2) {
       const int col = blockIdx.x * 16 + r16;
-      if (col < ldc) {
-        for (int m = lane >> 4; m < M; m += 4) {
-          float g = 0.f, u = 0.f;
+      const int m = wid * 4 + (lane >> 4);
+      if (col < ldc && m < M) {
+        float g = 0.f, u = 0.f;
 #pragma unroll
-          for (int ww = 0; ww < NW; ++ww) { g += red[ww][m][r16]; u += red[ww][m][16 + r16]; }
-          ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(g, u);
-        }
+        for (int ww = 0; ww < NW; ++ww) { g += red[ww][m][r16]; u += red[ww][m][16 + r16]; }
+        ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(g, u);
       }
     }
     return;
   }
-  const int c = lane % COLS;
-  const int n = tile_row(c >> 4) + (c & 15);
-  if (n >= N || (!PAIR && c >= rpb)) return;
-  const float b = bias ? bias[n] : 0.f;
-  for (int m = lane / COLS; m < M; m += 64 / COLS) {
-    float v = 0.f;
+  if (!e_mine) return;
+  float v = bias ? bias[e_n] : 0.f;
 #pragma unroll
-    for (int ww = 0; ww < NW; ++ww) v += red[ww][m][c];
-    store_out(C, ldc, m, n, v + b, epi);
-  }
+  for (int ww = 0; ww < NW; ++ww) v += red[ww][e_m][e_c];
+  if (epi == EPI_ACC_F32) ((float*)C)[(size_t)e_m * ldc + e_n] = c_old + v;
+  else store_out(C, ldc, e_m, e_n, v, epi);
 }
 
 template <int NW, int NT, int S, bool PAIR = false>
@@ -1024,7 +1030,8 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
                                                            const bf16* __restrict__ W, int ldw,
                                                            const float* __restrict__ bias,
                                                            void* __restrict__ C, int ldc, int M, int N,
-                                                           int cols_total, int unit, int epi, NormArgs norm) {
+                                                           int cols_total, int unit, int share, int extra, int epi,
+                                                           NormArgs norm) {
   constexpr int NW = 8;
   constexpr int COLS = 16 * NT;            // weight rows (output columns) of an item
   constexpr int RS = COLS + 4;             // row stride of the sums in LDS: conflict-free writes
@@ -1032,6 +1039,7 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
   __shared__ float ssq[NW][16];            // NORM: sum of x^2 over a wave's slice, per activation row
   extern __shared__ __attribute__((aligned(16))) float gs[];   // NORM: the norm's weight, K floats
   static_assert(NS % RING == 0, "the ring divides a slice");
+  static_assert(NW * (64 / COLS) >= 16, "an epilogue pass for every activation row");
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int r16 = lane & 15;
   const int k0 = wid * NS * 32 + (lane >> 4) * 8;         // this lane's k in step 0 of its slice
@@ -1040,10 +1048,12 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
   // whole items per block would leave some with a fifth more than others).  PAIR: a column is
   // a gate row and the up row 32 further on, in groups of 64 weight rows.  An item is CH
   // columns; lanes past c_end read the share's last row again, from the CU's own cache.
+  // (`share` units a block and one more for the first `extra` blocks: the host has divided, so
+  // that a block's first loads do not wait behind a division in software)
   constexpr int CH = PAIR ? 16 : COLS;
-  const int units = (cols_total + unit - 1) / unit;
-  const int c_begin = (int)((long)blockIdx.x * units / gridDim.x) * unit;
-  const int c_end = min((int)((long)(blockIdx.x + 1) * units / gridDim.x) * unit, cols_total);
+  const int b = blockIdx.x;
+  const int c_begin = (b * share + min(b, extra)) * unit;
+  const int c_end = min(((b + 1) * share + min(b + 1, extra)) * unit, cols_total);
   const int n_items = (c_end - c_begin + CH - 1) / CH;
   auto lane_wrow = [&](int c0, int j) {      // weight row of this lane in tile j of the item at c0
     if (PAIR) {
@@ -1169,6 +1179,22 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
     floatx4 acc[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    // The epilogue's place of this lane in this item: wave w adds up the sums of activation rows
+    // [w 64 / COLS, (w + 1) 64 / COLS), all waves at once.  What the epilogue needs from memory (the
+    // bias, and the output's old value where the product is added to it) is asked for here, in
+    // front of the item's refills and without a condition (a lane with no place, or no such
+    // operand, reads the head of the weights and drops it): behind the barrier it would make
+    // the wave wait for every load it has in flight, and the kernel's last item for memory.
+    const int e_c = lane % COLS;
+    const int e_n = c0 + e_c;
+    const int e_m = wid * (64 / COLS) + lane / COLS;
+    const bool e_mine = !PAIR && e_n < c_end && e_m < M;
+    float c_old = 0.f, e_bias = 0.f;
+    if constexpr (!PAIR) {
+      const float* dummy = reinterpret_cast<const float*>(W);
+      c_old = *((e_mine && epi == EPI_ACC_F32) ? (const float*)C + (size_t)e_m * ldc + e_n : dummy);
+      e_bias = *((e_mine && bias) ? bias + e_n : dummy);
+    }
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
 #pragma unroll
@@ -1184,6 +1210,8 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
                                        : *reinterpret_cast<const bf16x8*>(wrow[j] + (s + RING - NS) * 32);
         __builtin_amdgcn_sched_barrier(0);      // keep "use a register, then refill it" in this order
       }
+      // (held here, or the compiler moves the two loads to where they are used)
+      if (s == 0) asm volatile("" : "+v"(c_old), "+v"(e_bias));
     }
 #pragma unroll
     for (int j = 0; j < NT; ++j) wcur[j] = wrow[j];
@@ -1196,43 +1224,37 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
     __syncthreads();
     // The buffer is written again two items on, behind the next barrier, which this wave
     // reaches only after it has read its sums here.
-    if (wid != (it & (NW - 1))) continue;
     auto row_scale = [&](int m) {          // NORM: 1 / sqrt(mean(x^2) + eps) of activation row m
       float t = 0.f;
 #pragma unroll
       for (int ww = 0; ww < NW; ++ww) t += ssq[ww][m];
       return 1.0f / sqrtf(t / (float)(NW * NS * 32) + norm.eps);
     };
-    if (epi == EPI_SWIGLU) {
-      if constexpr (PAIR && NT == 2) {
-        const int col = c0 + r16;
-        if (col < c_end && col < ldc) {
-          for (int m = lane >> 4; m < M; m += 4) {
-            float g = 0.f, u = 0.f;
+    if constexpr (PAIR) {
+      static_assert(NT == 2, "a gate tile and an up tile");
+      const int col = c0 + r16;
+      const int m = wid * 4 + (lane >> 4);
+      if (epi == EPI_SWIGLU && col < c_end && col < ldc && m < M) {
+        float g = 0.f, u = 0.f;
 #pragma unroll
-            for (int ww = 0; ww < NW; ++ww) { g += red[buf][ww][m][r16]; u += red[buf][ww][m][16 + r16]; }
-            if constexpr (NORM) {
-              const float sc = row_scale(m);
-              g *= sc;
-              u *= sc;
-            }
-            ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(g, u);
-          }
+        for (int ww = 0; ww < NW; ++ww) { g += red[buf][ww][m][r16]; u += red[buf][ww][m][16 + r16]; }
+        if constexpr (NORM) {
+          const float sc = row_scale(m);
+          g *= sc;
+          u *= sc;
         }
+        ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(g, u);
       }
-      continue;
-    }
-    // a pass of the wave covers 64 / COLS activation rows of COLS adjacent outputs each
-    const int c = lane % COLS;
-    const int n = c0 + c;
-    if (n >= c_end) continue;
-    const float b = bias ? bias[n] : 0.f;
-    for (int m = lane / COLS; m < M; m += 64 / COLS) {
-      float v = 0.f;
+    } else {
+      if (e_mine) {
+        float v = 0.f;
 #pragma unroll
-      for (int ww = 0; ww < NW; ++ww) v += red[buf][ww][m][c];
-      if constexpr (NORM) v *= row_scale(m);
-      store_out(C, ldc, m, n, v + b, epi);
+        for (int ww = 0; ww < NW; ++ww) v += red[buf][ww][e_m][e_c];
+        if constexpr (NORM) v *= row_scale(e_m);
+        v += (bias ? e_bias : 0.f);
+        if (epi == EPI_ACC_F32) ((float*)C)[(size_t)e_m * ldc + e_n] = c_old + v;
+        else store_out(C, ldc, e_m, e_n, v, epi);
+      }
     }
   }
 }
@@ -1263,10 +1285,12 @@ int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const fl
       if (e != hipSuccess) return (int)e;
       configured = true;
     }
-    kern<<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, cols_total, unit, epi, *norm);
+    kern<<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, cols_total, unit, units / grid, units % grid,
+                                      epi, *norm);
   } else {
     stationary16_kernel<NS, RING, NT, PAIR, false><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
-                                                                             cols_total, unit, epi,
+                                                                             cols_total, unit, units / grid,
+                                                                             units % grid, epi,
                                                                              NormArgs{nullptr, nullptr, 0.f});
   }
   return mf_launch_status();
