@@ -840,6 +840,19 @@ bool ring_takes(bool aligned, int K, int splits, int k_per_split) {
   return aligned && K % 256 == 0 && (long)(splits - 1) * k_per_split < K;
 }
 
+// The tiled copy of a weight matrix (K a multiple of 32, rows padded to a multiple of 16):
+// [rows / 16][K / 32][16 rows][32 k], 1 KB a tile.  A wave's load of an MFMA operand (lane ->
+// row lane % 16, eight k at 8 (lane / 16)) is one tile: a contiguous kilobyte of whole 128-byte
+// lines, where the row-major matrix gives it sixteen halves of lines K elements apart, and a
+// wave that walks along K reads tile after tile.  The kernels for at most 64 rows, which take their
+// weights straight from memory into MFMA operands, read this copy where the caller has one (the
+// down product at 8 rows: 26.7 us from 34.1).  WSTEP: elements from one step of 32 k to the next.
+template <bool TILED>
+__device__ __forceinline__ const bf16* w_operand(const bf16* W, int ldw, int K, int row, int k) {
+  if constexpr (TILED) return W + ((size_t)(row >> 4) * (K >> 5) + (k >> 5)) * 512 + (row & 15) * 32 + (k & 31);
+  else return W + (size_t)row * ldw + k;
+}
+
 // The same split of the work as skinny16_kernel (a block owns 16 NT weight rows, its waves split
 // K), for aligned operands and K a multiple of 32, with the loads rolling: a wave holds S steps
 // of weights and activations in registers, and the refill of a register is issued right behind
@@ -847,7 +860,7 @@ bool ring_takes(bool aligned, int K, int splits, int k_per_split) {
 // registers of the two-buffer scheme above.  With K of many thousands and few weight rows
 // (the down projection) the chip is filled by loads in flight, not by blocks, and this is
 // what the time depends on.
-template <int NW, int NT, int S, bool PAIR>
+template <int NW, int NT, int S, bool PAIR, bool TILED>
 __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restrict__ A, int lda,
                                                             const bf16* __restrict__ W, int ldw,
                                                             const float* __restrict__ bias,
@@ -855,6 +868,7 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
                                                             int K, int steps_per_wave, int epi, int rpb) {
   constexpr int COLS = 16 * NT;
   constexpr int RS = COLS + 4;
+  constexpr int WSTEP = TILED ? 512 : 32;
   __shared__ float red[NW][16][RS];
   const int lane = threadIdx.x & 63;
   const int wid = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // the same in the whole wave
@@ -875,7 +889,7 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
   const bf16* arow = A + (size_t)min(r16, M - 1) * lda + kq;
   const bf16* wrow[NT];
 #pragma unroll
-  for (int j = 0; j < NT; ++j) wrow[j] = W + (size_t)min(lane_row(j), N - 1) * ldw + kq;
+  for (int j = 0; j < NT; ++j) wrow[j] = w_operand<TILED>(W, ldw, K, min(lane_row(j), N - 1), kq);
   floatx4 acc[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -898,7 +912,7 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
 #pragma unroll
       for (int j = 0; j < NT; ++j)
         acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            a1, *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32), acc[j], 0, 0, 0);
+            a1, *reinterpret_cast<const bf16x8*>(wrow[j] + s * WSTEP), acc[j], 0, 0, 0);
     }
   } else {
     bf16x8 a[S], w[NT][S];
@@ -906,7 +920,7 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
     for (int s = 0; s < S; ++s) {
       a[s] = *reinterpret_cast<const bf16x8*>(arow + s * 32);
 #pragma unroll
-      for (int j = 0; j < NT; ++j) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * 32);
+      for (int j = 0; j < NT; ++j) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + s * WSTEP);
     }
     // rounds whose refills all exist: no branch in the body
     int base = 0;
@@ -916,7 +930,7 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
           acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s], w[j][s], acc[j], 0, 0, 0);
-          w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + (base + S + s) * 32);
+          w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + (base + S + s) * WSTEP);
         }
         a[s] = *reinterpret_cast<const bf16x8*>(arow + (base + S + s) * 32);
         __builtin_amdgcn_sched_barrier(0);
@@ -930,7 +944,7 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
       if (s < rem) {
         a[s] = *reinterpret_cast<const bf16x8*>(arow + (base + S + s) * 32);
 #pragma unroll
-        for (int j = 0; j < NT; ++j) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + (base + S + s) * 32);
+        for (int j = 0; j < NT; ++j) w[j][s] = *reinterpret_cast<const bf16x8*>(wrow[j] + (base + S + s) * WSTEP);
       }
     }
 #pragma unroll
@@ -968,7 +982,7 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
   else store_out(C, ldc, e_m, e_n, v, epi);
 }
 
-template <int NW, int NT, int S, bool PAIR = false>
+template <int NW, int NT, int S, bool PAIR = false, bool TILED = false>
 int launch_rolling16(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
                      int M, int N, int K, int epi, hipStream_t stream) {
   const int steps_per_wave = (K / 32 + NW - 1) / NW;
@@ -980,8 +994,8 @@ int launch_rolling16(const bf16* A, int lda, const bf16* W, int ldw, const float
     rpb = rpb < 1 ? 1 : (rpb > 16 * NT ? 16 * NT : rpb);
     blocks = (N + rpb - 1) / rpb;
   }
-  rolling16_kernel<NW, NT, S, PAIR><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K,
-                                                                    steps_per_wave, epi, rpb);
+  rolling16_kernel<NW, NT, S, PAIR, TILED><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K,
+                                                                           steps_per_wave, epi, rpb);
   return mf_launch_status();
 }
 
@@ -1025,7 +1039,7 @@ struct NormArgs {
 // RING = NS the registers hold a whole item; for a long K (5120, 8192) the activations alone take
 // up to half the registers, so the weights go through a shorter ring, and a register is refilled
 // with the step RING further on, of this item or of the next one.
-template <int NS, int RING, int NT, bool PAIR, bool NORM>
+template <int NS, int RING, int NT, bool PAIR, bool NORM, bool TILED>
 __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restrict__ Av, int lda,
                                                            const bf16* __restrict__ W, int ldw,
                                                            const float* __restrict__ bias,
@@ -1033,6 +1047,8 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
                                                            int cols_total, int unit, int share, int extra, int epi,
                                                            NormArgs norm) {
   constexpr int NW = 8;
+  constexpr int KK = NW * NS * 32;         // K
+  constexpr int WSTEP = TILED ? 512 : 32;  // elements from one step's weights to the next's
   constexpr int COLS = 16 * NT;            // weight rows (output columns) of an item
   constexpr int RS = COLS + 4;             // row stride of the sums in LDS: conflict-free writes
   __shared__ float red[2][NW][16][RS];     // [buffer][wave][activation row][weight row of the item]
@@ -1071,9 +1087,9 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
   // wait after it, with the path that has fewer loads in flight, and the prologue would wait for
   // the activations until most of the first weights have arrived as well.
   auto first_loads = [&](int j) {
-    wcur[j] = Wp + (size_t)lane_wrow(c_begin, j) * ldw + k0;
+    wcur[j] = w_operand<TILED>(Wp, ldw, KK, lane_wrow(c_begin, j), k0);
 #pragma unroll
-    for (int s = 0; s < RING; ++s) w[j][s] = *reinterpret_cast<const bf16x8*>(wcur[j] + s * 32);
+    for (int s = 0; s < RING; ++s) w[j][s] = *reinterpret_cast<const bf16x8*>(wcur[j] + s * WSTEP);
   };
   bf16x8 afr[NS];
   float ss = 0.f;
@@ -1175,7 +1191,7 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
     const bool has_next = it + 1 < n_items;
 #pragma unroll
     for (int j = 0; j < NT; ++j)
-      wrow[j] = Wp + (has_next ? (size_t)lane_wrow(c0 + CH, j) * ldw : (size_t)0) + k0;
+      wrow[j] = w_operand<TILED>(Wp, ldw, KK, has_next ? lane_wrow(c0 + CH, j) : 0, k0);
     floatx4 acc[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -1206,8 +1222,8 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
           asm volatile("" : "+v"(acc[j]) : : "memory");
           __builtin_amdgcn_sched_barrier(0);
         }
-        w[j][s % RING] = s + RING < NS ? *reinterpret_cast<const bf16x8*>(wcur[j] + (s + RING) * 32)
-                                       : *reinterpret_cast<const bf16x8*>(wrow[j] + (s + RING - NS) * 32);
+        w[j][s % RING] = s + RING < NS ? *reinterpret_cast<const bf16x8*>(wcur[j] + (s + RING) * WSTEP)
+                                       : *reinterpret_cast<const bf16x8*>(wrow[j] + (s + RING - NS) * WSTEP);
         __builtin_amdgcn_sched_barrier(0);      // keep "use a register, then refill it" in this order
       }
       // (held here, or the compiler moves the two loads to where they are used)
@@ -1260,7 +1276,7 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
 }
 
 // true when the shape is one the register-resident kernel is built for
-template <int NS, int NT, bool PAIR>
+template <int NS, int NT, bool PAIR, bool TILED>
 int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
                         int M, int N, int epi, const NormArgs* norm, hipStream_t stream) {
   const int n_cu = cu_count();
@@ -1277,7 +1293,7 @@ int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const fl
   static_assert(NS % RING == 0 && 4 * NS + 4 * NT * RING <= 200, "activations and weight ring fit the registers");
   if (norm) {
     constexpr int smem = 8 * NS * 32 * (int)sizeof(float);       // the norm's weight
-    auto kern = stationary16_kernel<NS, RING, NT, PAIR, true>;
+    auto kern = stationary16_kernel<NS, RING, NT, PAIR, true, TILED>;
     static bool configured = false;
     if (!configured) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1288,7 +1304,7 @@ int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const fl
     kern<<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, cols_total, unit, units / grid, units % grid,
                                       epi, *norm);
   } else {
-    stationary16_kernel<NS, RING, NT, PAIR, false><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
+    stationary16_kernel<NS, RING, NT, PAIR, false, TILED><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
                                                                              cols_total, unit, units / grid,
                                                                              units % grid, epi,
                                                                              NormArgs{nullptr, nullptr, 0.f});
@@ -1723,26 +1739,29 @@ MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, c
 
 // The register-resident kernel for the shapes it is built for (K = 256 NS with enough tiles to
 // go round); MF_NOT_BUILT for any other, and nothing is launched.
-static int stationary16(const void* a, int lda, const bf16* w, int ldw, const float* bias, void* C, int ldc, int M,
-                 int N, int K, int epi, const NormArgs* norm, hipStream_t stream) {
+static int stationary16(const void* a, int lda, const bf16* w, const bf16* wt, int ldw, const float* bias, void* C,
+                        int ldc, int M, int N, int K, int epi, const NormArgs* norm, hipStream_t stream) {
   if (!stationary_takes(M, N, K, epi, norm != nullptr)) return MF_NOT_BUILT;
   // two tiles an item where a block's share is more than one: 128-byte rows of 32-bit output
   const int n_cu = cu_count();
   if (n_cu <= 0) return (int)hipErrorUnknown;
   const bool two = (N + n_cu - 1) / n_cu > 16;
-#define MF_STATIONARY(NS_)                                                                                  \
-  case NS_:                                                                                                 \
-    return epi == EPI_SWIGLU                                                                                \
-               ? launch_stationary16<NS_, 2, true>(a, lda, w, ldw, bias, C, ldc, M, N, epi, norm, stream)   \
-           : two ? launch_stationary16<NS_, 2, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, norm, stream) \
-                 : launch_stationary16<NS_, 1, false>(a, lda, w, ldw, bias, C, ldc, M, N, epi, norm, stream);
+#define MF_STATIONARY_T(NS_, T_, W_)                                                                          \
+  (epi == EPI_SWIGLU ? launch_stationary16<NS_, 2, true, T_>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, stream) \
+   : two             ? launch_stationary16<NS_, 2, false, T_>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, stream) \
+                     : launch_stationary16<NS_, 1, false, T_>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, stream))
+#define MF_STATIONARY(NS_) \
+  case NS_: return wt ? MF_STATIONARY_T(NS_, true, wt) : MF_STATIONARY_T(NS_, false, w);
   switch (K / 256) { MF_STATIONARY_NS(MF_STATIONARY) }
 #undef MF_STATIONARY
+#undef MF_STATIONARY_T
   return MF_NOT_BUILT;
 }
 
 // M <= 64.  `part` holds splits*M*N floats when splits > 1; k_per_split is a multiple of 256.
-MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, const float* bias,
+// `Wt`: the tiled copy of W (see w_operand), or null; the kernels that have a form for it read it
+// instead of W.
+MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, const void* Wt, int ldw, const float* bias,
                                void* C, int ldc, float* part, int M, int N, int K, int splits,
                                int k_per_split, int epi, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
@@ -1756,10 +1775,13 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
                      ((uintptr_t)W % 16 == 0) && (K % 8 == 0);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
+  const bf16* wt = (K % 32 == 0 && (uintptr_t)Wt % 16 == 0) ? (const bf16*)Wt : nullptr;
   const SkinnyChoice choice = skinny_choice(M, N, K, vec_ok, epi, splits, k_per_split, cu_count());
   switch (choice) {
-    case SK_STATIONARY: return stationary16(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, nullptr, stream);
-    case SK_ROLLING: return launch_rolling16<8, 1, 16>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+    case SK_STATIONARY: return stationary16(a, lda, w, wt, ldw, bias, C, ldc, M, N, K, epi, nullptr, stream);
+    case SK_ROLLING:
+      return wt ? launch_rolling16<8, 1, 16, false, true>(a, lda, wt, ldw, bias, C, ldc, M, N, K, epi, stream)
+                : launch_rolling16<8, 1, 16>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
     case SK_GUARDED_PAIR: return launch_skinny16<4, 2, 4, true>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case SK_GUARDED_4X2: return launch_skinny16<4, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case SK_GUARDED_8X2: return launch_skinny16<8, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
@@ -1781,14 +1803,15 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, int ldw, c
 // shapes the register-resident kernel does not cover: the caller then runs the norm and the
 // product one after the other.
 MF_API int mf_gemm_bf16_normed(const float* x, int ldx, const int* row_idx, const float* g, float eps,
-                               const void* W, int ldw, const float* bias, void* C, int ldc, int M, int N, int K,
-                               int epi, hipStream_t stream) {
+                               const void* W, const void* Wt, int ldw, const float* bias, void* C, int ldc, int M,
+                               int N, int K, int epi, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || epi < 0 || epi > EPI_SWIGLU) return (int)hipErrorInvalidValue;
   if (ldx % 4 != 0 || ldw % 8 != 0 || (uintptr_t)x % 16 != 0 || (uintptr_t)g % 16 != 0 || (uintptr_t)W % 16 != 0)
     return MF_NOT_BUILT;
   const NormArgs norm{g, row_idx, eps};
-  return stationary16(x, ldx, (const bf16*)W, ldw, bias, C, ldc, M, N, K, epi, &norm, stream);
+  const bf16* wt = (uintptr_t)Wt % 16 == 0 ? (const bf16*)Wt : nullptr;
+  return stationary16(x, ldx, (const bf16*)W, wt, ldw, bias, C, ldc, M, N, K, epi, &norm, stream);
 }
 
 // How a product of more than 64 rows is run: out[0] the variant for mf_gemm_bf16, or with out[1] > 1

@@ -12,7 +12,7 @@ from typing import Callable, Dict
 
 import torch
 
-from ..kernels import ops
+from ..kernels import ops, tuning
 from ..parts.base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, Runtime, make_part,
                           normed_input)
 from ..parts.spec import BlockSpec, ModelSpec
@@ -71,6 +71,25 @@ class DecoderModel:
             for part in block.parts():
                 part.load(lambda name, p=bs.prefix: get(p + name))
         self.loaded = True
+        self.decode_copy_bytes = self._make_decode_copies()
+
+    def _all_parts(self):
+        yield from (self.embedding, self.head, self.final_norm)
+        for block in self.blocks:
+            yield from block.parts()
+
+    def _make_decode_copies(self) -> int:
+        """The parts' second copies of their matrices for the steps of few tokens (a layout that
+        those steps' products read faster), all of them or none: made where they take at most a
+        third of the device memory that is free once the weights are in place, so that a model
+        that fills the device keeps its memory for the cache.  Returns their bytes."""
+        if not self.rt.is_bf16 or self.rt.device.type != "cuda" or tuning.NO_DECODE_COPIES:
+            return 0
+        need = sum(part.decode_copies(False) for part in self._all_parts())
+        free, _ = torch.cuda.mem_get_info(self.rt.device)
+        if need == 0 or need > free // 3:
+            return 0
+        return sum(part.decode_copies(True) for part in self._all_parts())
 
     # ------------------------------------------------------------ cache needs
     def cache_requests(self) -> Dict[int, object]:

@@ -55,9 +55,9 @@ _PROTOTYPES = {
         "mf_gemm_bf16": [_P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
         "mf_gemm_bf16_splitk": [_P, c_int, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_int,
                                 c_int, _P],
-        "mf_gemm_bf16_skinny": [_P, c_int, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int,
+        "mf_gemm_bf16_skinny": [_P, c_int, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int,
                                 c_int, c_int, _P],
-        "mf_gemm_bf16_normed": [_P, c_int, _P, _P, c_float, _P, c_int, _P, _P, c_int, c_int, c_int, c_int,
+        "mf_gemm_bf16_normed": [_P, c_int, _P, _P, c_float, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int,
                                 c_int, _P],
         "mf_gemm_bf16_plan": [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_char_p, c_int],
         "mf_gemm_bf16_tile_plan": [c_int, c_int, c_int, c_int, c_int, c_int, _P],
@@ -442,11 +442,32 @@ def plan_linear(m: int, n: int, k: int, swiglu: bool = False, normed: bool = Fal
     return dict(kernel=name.value.decode(), splits=splits, k_per_split=per)
 
 
+def tile_weight(weight: torch.Tensor) -> torch.Tensor:
+    """The tiled copy of a bfloat16 `[n][k]` matrix, k a multiple of 32: `[ceil(n / 16)][k / 32][16][32]`,
+    rows padded with zeros to a multiple of 16.  The products of at most 64 rows read their
+    weights a tile (a contiguous kilobyte) per wave and step from it; made once, when a model is
+    loaded, where memory allows a second copy."""
+    _need(weight, "tile_weight.weight", torch.bfloat16)
+    n, k = weight.shape
+    if k % 32:
+        raise KernelError(f"tile_weight: k {k} is not a multiple of 32")
+    n16 = (n + 15) // 16 * 16
+    if n16 != n:
+        weight = torch.cat([weight, torch.zeros((n16 - n, k), dtype=weight.dtype, device=weight.device)])
+    return weight.view(n16 // 16, 16, k // 32, 32).permute(0, 2, 1, 3).contiguous()
+
+
+def _need_tiled(tiled: Optional[torch.Tensor], name: str, n: int, k: int) -> None:
+    if tiled is not None:
+        _need(tiled, name, torch.bfloat16, ((n + 15) // 16, k // 32, 16, 32))
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-           accumulate: bool = False, variant: int = 0) -> None:
+           accumulate: bool = False, variant: int = 0, tiled: Optional[torch.Tensor] = None) -> None:
     """out (+)= x @ weight^T (+ bias).  weight is [out][in].  float32 weights take the true
     32-bit kernel; bfloat16 weights take the matrix-core kernels (a few rows: the streaming
-    kernel).  `out` is float32, or bfloat16 for a bfloat16 product that is stored."""
+    kernel).  `out` is float32, or bfloat16 for a bfloat16 product that is stored.  `tiled`:
+    `tile_weight(weight)`, which the kernels for at most 64 rows read instead where they can."""
     _need(x, "linear.x", _FLOATS)
     _need(weight, "linear.weight", x.dtype)
     m, k = x.shape
@@ -470,7 +491,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
     if m <= 64 and variant == 0:
         splits, per = _k_split(m, n, k, False, aligned)
         part = workspace("skinny", splits * m * n, x.device) if splits > 1 else None
-        _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(bias),
+        _need_tiled(tiled, "linear.tiled", n, k)
+        _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), _ptr(tiled), k, _ptr(bias),
                                                         _ptr(out), n, _ptr(part), m, n, k, splits, per,
                                                         epi, _stream()), f"gemm_bf16_skinny {m}x{n}x{k}")
         return
@@ -498,9 +520,10 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return torch.stack([gate.view(groups, 32, k), up.view(groups, 32, k)], dim=1).reshape(groups * 64, k).contiguous()
 
 
-def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, variant: int = 0) -> None:
+def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, variant: int = 0,
+                  tiled: Optional[torch.Tensor] = None) -> None:
     """out = silu(x @ Wg^T) * (x @ Wu^T) in one kernel; `weight` is `interleave_gate_up(Wg, Wu)`,
-    everything bfloat16, `out` is [rows][nf]."""
+    everything bfloat16, `out` is [rows][nf].  `tiled`: `tile_weight(weight)`."""
     _need(x, "linear_swiglu.x", torch.bfloat16)
     _need(weight, "linear_swiglu.weight", torch.bfloat16)
     m, k = x.shape
@@ -515,7 +538,8 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, vari
     if m <= 64 and variant == 0:
         splits, per = _k_split(m, n, k, True, aligned)
         part = workspace("skinny", splits * m * n, x.device) if m > 16 or splits > 1 else None
-        _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), k, _ptr(None), _ptr(out), nf,
+        _need_tiled(tiled, "linear_swiglu.tiled", n, k)
+        _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), _ptr(tiled), k, _ptr(None), _ptr(out), nf,
                                                         _ptr(part), m, n, k, splits, per, EPI_SWIGLU, _stream()),
                f"gemm_bf16_skinny(swiglu) {m}x{n}x{k}")
         return
@@ -536,12 +560,12 @@ NOT_BUILT = -2      # an entry point's answer for a shape it has no kernel for; 
 
 def linear_normed(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, row_idx: Optional[torch.Tensor],
                   weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-                  accumulate: bool = False, swiglu: bool = False) -> bool:
+                  accumulate: bool = False, swiglu: bool = False, tiled: Optional[torch.Tensor] = None) -> bool:
     """out (+)= rmsnorm(x[row_idx]) @ weight^T (+ bias) in one kernel, for the few-row shapes
     the register-resident decode product covers; with `swiglu`, `weight` is
     `interleave_gate_up(Wg, Wu)` and out = silu(gate) * up.  x is the float32 residual stream,
     weight bfloat16.  Returns False, having done nothing, when there is no such kernel for
-    the shape: the caller then norms and multiplies in two steps."""
+    the shape: the caller then norms and multiplies in two steps.  `tiled`: `tile_weight(weight)`."""
     _need(x, "linear_normed.x", torch.float32)
     _need(weight, "linear_normed.weight", torch.bfloat16)
     k = x.shape[1]
@@ -570,9 +594,10 @@ def linear_normed(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, row_id
         return True
     if m > 16 or tuning.NO_FOLD:
         return False
+    _need_tiled(tiled, "linear_normed.tiled", n, k)
     rc = _fn("gemm_bf16", "mf_gemm_bf16_normed")(_ptr(x), k, _ptr(row_idx), _ptr(norm_weight), float(eps),
-                                                 _ptr(weight), k, _ptr(bias), _ptr(out), ldc, m, n, k, epi,
-                                                 _stream())
+                                                 _ptr(weight), _ptr(tiled), k, _ptr(bias), _ptr(out), ldc, m, n, k,
+                                                 epi, _stream())
     if rc == NOT_BUILT:
         return False
     _check(rc, f"gemm_bf16_normed{'(swiglu)' if swiglu else ''} {m}x{n}x{k}")

@@ -16,6 +16,7 @@ Kernel choice, for measurements (each overrides what `ops` would pick by shape):
 * MF_ATTN_SPLITS=n      key splits of the bfloat16 decode attention
 * MF_SKINNY_TARGET=n    blocks the K-split decode product aims at (default: one per CU)
 * MF_NO_SHARED_PAGES=1  a block of queries of the prompt attention keeps all its pages to itself
+* MF_NO_DECODE_COPIES=1 a model keeps no second, tiled copy of its matrices for the steps of few tokens
 * MF_NO_FOLD=1          the RMS norm is a kernel of its own instead of being folded into the
                         product that follows it
 """
@@ -41,3 +42,4 @@ ATTN_SPLITS = _int("MF_ATTN_SPLITS")
 SKINNY_TARGET = _int("MF_SKINNY_TARGET")
 NO_FOLD = _flag("MF_NO_FOLD")
 NO_SHARED_PAGES = _flag("MF_NO_SHARED_PAGES")
+NO_DECODE_COPIES = _flag("MF_NO_DECODE_COPIES")

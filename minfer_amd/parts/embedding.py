@@ -66,5 +66,8 @@ class LinearHead(Head):
     def weight(self) -> torch.Tensor:
         return self.linear.weight
 
+    def decode_copies(self, make: bool) -> int:
+        return self.linear.decode_copy(make)
+
     def forward(self, x) -> torch.Tensor:
         return self.linear(x, out_dtype=torch.float32)

@@ -22,7 +22,7 @@ class SwiGLU(FeedForward):
         p = spec.params
         self.hidden, self.inter = int(p["hidden_size"]), int(p["intermediate_size"])
         self.names = {k: p[k] for k in ("gate", "up", "down")}
-        self.gate_up = self.down = self.fused = None
+        self.gate_up = self.down = self.fused = self.fused_tiled = None
 
     def tensor_specs(self):
         n = self.names
@@ -39,6 +39,16 @@ class SwiGLU(FeedForward):
             self.gate_up = Linear.stacked([gate, up])
         self.down = Linear(get(n["down"] + ".weight"))
 
+    def decode_copies(self, make: bool) -> int:
+        n = self.down.decode_copy(make)
+        if self.fused is not None and self.hidden % 32 == 0:
+            if make and self.fused_tiled is None:
+                self.fused_tiled = ops.tile_weight(self.fused)
+            n += self.fused.numel() * 2
+        elif self.gate_up is not None:
+            n += self.gate_up.decode_copy(make)
+        return n
+
     takes_normed = True
 
     def forward(self, x, h, ctx) -> None:
@@ -46,8 +56,8 @@ class SwiGLU(FeedForward):
         if self.fused is not None:
             fold = x.norm.rms_scale() if isinstance(x, Normed) else None
             if fold is None or not ops.linear_normed(x.h, fold[0], fold[1], x.row_idx, self.fused, None, y,
-                                                     swiglu=True):
-                ops.linear_swiglu(x.tensor() if isinstance(x, Normed) else x, self.fused, y)
+                                                     swiglu=True, tiled=self.fused_tiled):
+                ops.linear_swiglu(x.tensor() if isinstance(x, Normed) else x, self.fused, y, tiled=self.fused_tiled)
         else:
             ops.swiglu(self.gate_up(x, out_dtype=torch.float32), y)
         self.down(y, out=h, accumulate=True)

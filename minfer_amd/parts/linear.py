@@ -26,6 +26,17 @@ class Linear:
         self.weight = weight.contiguous()
         self.bias = None if bias is None else bias.to(torch.float32).contiguous()
         self.out_features, self.in_features = weight.shape
+        self.tiled: Optional[torch.Tensor] = None      # ops.tile_weight(weight), where the model keeps one
+
+    def decode_copy(self, make: bool) -> int:
+        """Bytes of the tiled copy of this matrix, which the products of few rows read faster than
+        the matrix itself (0: it has none: 32-bit, or a row length that is no multiple of 32);
+        made when `make`."""
+        if self.weight.dtype != torch.bfloat16 or self.in_features % 32:
+            return 0
+        if make and self.tiled is None:
+            self.tiled = ops.tile_weight(self.weight)
+        return (self.out_features + 15) // 16 * 16 * self.in_features * 2
 
     @classmethod
     def stacked(cls, weights: List[torch.Tensor], biases: Optional[List[Optional[torch.Tensor]]] = None):
@@ -48,7 +59,7 @@ class Linear:
         if isinstance(x, Normed):
             fold = x.norm.rms_scale() if self.weight.dtype == torch.bfloat16 else None
             if fold is not None and ops.linear_normed(x.h, fold[0], fold[1], x.row_idx, self.weight, self.bias,
-                                                      out, accumulate=accumulate):
+                                                      out, accumulate=accumulate, tiled=self.tiled):
                 return out
             x = x.tensor()
         if self.weight.dtype == torch.float32 and x.dtype != torch.float32:
@@ -60,5 +71,5 @@ class Linear:
             ops.linear(x, self.weight, self.bias, tmp)
             ops.convert(tmp, out)
             return out
-        ops.linear(x, self.weight, self.bias, out, accumulate=accumulate)
+        ops.linear(x, self.weight, self.bias, out, accumulate=accumulate, tiled=self.tiled)
         return out

@@ -99,7 +99,7 @@ def rope_inplace(qkv, cos, sin, positions, n_rot_heads, n_heads_total, head_dim)
     x[:, :n_rot_heads] = torch.cat([v0 * c - v1 * s, v0 * s + v1 * c], dim=-1).float()
 
 
-def linear(x, weight, bias, out, accumulate=False, variant=0):
+def linear(x, weight, bias, out, accumulate=False, variant=0, tiled=None):
     y = x.double() @ weight.double().t()
     if bias is not None:
         y = y + bias.double()
@@ -119,7 +119,7 @@ def interleave_gate_up(gate, up):
     return out
 
 
-def linear_swiglu(x, weight, out, variant=0):
+def linear_swiglu(x, weight, out, variant=0, tiled=None):
     nf = out.shape[1]
     idx = torch.arange(nf)
     g = x.double() @ weight.double()[(idx // 32) * 64 + idx % 32].t()
@@ -127,7 +127,7 @@ def linear_swiglu(x, weight, out, variant=0):
     out.copy_((g / (1.0 + torch.exp(-g)) * u).to(out.dtype))
 
 
-def linear_normed(x, norm_weight, eps, row_idx, weight, bias, out, accumulate=False, swiglu=False):
+def linear_normed(x, norm_weight, eps, row_idx, weight, bias, out, accumulate=False, swiglu=False, tiled=None):
     """The stand-in has no folded kernel: the caller norms and multiplies in two steps."""
     return False
 

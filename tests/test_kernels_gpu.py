@@ -544,6 +544,65 @@ def test_gemm_bf16_wide_few_rows(ops, m, n, k):
     close(ob, ref, tol + 1e-3, 1e-2)
 
 
+def test_tile_weight_layout(ops):
+    """[n][k] -> [ceil(n / 16)][k / 32][16][32], zero rows behind n."""
+    w = rnd((40, 96), torch.bfloat16, 5).to(DEV)
+    t = ops.tile_weight(w)
+    assert tuple(t.shape) == (3, 3, 16, 32)
+    for r, k in ((0, 0), (15, 31), (16, 32), (39, 95), (17, 70)):
+        assert t[r // 16, k // 32, r % 16, k % 32] == w[r, k]
+    assert not t[2, :, 8:].any()
+    with pytest.raises(Exception):
+        ops.tile_weight(rnd((16, 40), torch.bfloat16, 6).to(DEV))
+
+
+@pytest.mark.parametrize("m,n,k", [(8, 3584, 18944), (1, 1000, 8224), (16, 4608, 3584), (5, 152064, 1536),
+                                   (3, 2100, 8192), (16, 8192, 8192), (8, 90, 4096), (2, 2048, 96)])
+def test_gemm_bf16_tiled_copy_same_bits(ops, m, n, k):
+    """The products of at most 16 rows read the tiled copy of the weights where they are given one:
+    the same sums in the same order, so the same bits as from the matrix itself, for every
+    epilogue, with and without the folded norm; and right against the plain product."""
+    x, w, b = rnd((m, k), torch.bfloat16, 120), rnd((n, k), torch.bfloat16, 121, 0.05), rnd((n,), seed=122)
+    xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+    wt = ops.tile_weight(wd)
+    ref = x.double() @ w.double().t() + b.double()
+    base = rnd((m, n), seed=123).to(DEV)
+    got = []
+    for tiled in (None, wt):
+        out = torch.full((m, n), 7.0, device=DEV)
+        ops.linear(xd, wd, bd, out, tiled=tiled)
+        acc = base.clone()
+        ops.linear(xd, wd, None, acc, accumulate=True, tiled=tiled)
+        ob = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+        ops.linear(xd, wd, bd, ob, tiled=tiled)
+        xf, g = rnd((m + 3, k), seed=124).to(DEV), rnd((k,), seed=125).to(DEV)
+        idx = torch.arange(m, dtype=torch.int32, device=DEV) + 2
+        on = torch.full((m, n), 7.0, device=DEV)
+        folded = ops.linear_normed(xf, g, 1e-5, idx, wd, bd, on, tiled=tiled)
+        got.append((out, acc, ob, on if folded else out))
+    close(got[1][0], ref, 2e-5 * math.sqrt(k), 1e-5)
+    for a, c in zip(*got):
+        assert torch.equal(a, c)
+
+
+@pytest.mark.parametrize("m,nf,k", [(8, 18944, 3584), (1, 1024, 2048), (16, 1030, 4096), (3, 2100, 8192)])
+def test_gemm_bf16_swiglu_tiled_copy_same_bits(ops, m, nf, k):
+    gate, up = rnd((nf, k), torch.bfloat16, 130, 0.05), rnd((nf, k), torch.bfloat16, 131, 0.05)
+    w = ops.interleave_gate_up(gate.to(DEV), up.to(DEV))
+    wt = ops.tile_weight(w)
+    x = rnd((m, k), torch.bfloat16, 132).to(DEV)
+    xf, g = rnd((m, k), seed=133).to(DEV), rnd((k,), seed=134).to(DEV)
+    got = []
+    for tiled in (None, wt):
+        y = torch.empty(m, nf, dtype=torch.bfloat16, device=DEV)
+        ops.linear_swiglu(x, w, y, tiled=tiled)
+        yn = torch.empty(m, nf, dtype=torch.bfloat16, device=DEV)
+        folded = ops.linear_normed(xf, g, 1e-6, None, w, None, yn, swiglu=True, tiled=tiled)
+        got.append((y, yn if folded else y))
+    for a, c in zip(*got):
+        assert torch.equal(a, c)
+
+
 @pytest.mark.parametrize("variant", [0, 1, 2, 9, 12, 13])
 @pytest.mark.parametrize("m,nf,k", [(1, 176, 64), (8, 344, 128), (16, 32, 200), (17, 176, 64), (64, 1000, 344),
                                     (65, 232, 200), (300, 18944, 256), (130, 31, 72),
