@@ -595,13 +595,26 @@ __global__ __launch_bounds__(512) void skinny_kernel(const bf16* __restrict__ A,
     }
 }
 
+// The tiled copy of a weight matrix (K a multiple of 32, rows padded to a multiple of 16):
+// [rows / 16][K / 32][16 rows][32 k], 1 KB a tile.  A wave's load of an MFMA operand (lane ->
+// row lane % 16, eight k at 8 (lane / 16)) is one tile: a contiguous kilobyte of whole 128-byte
+// lines, where the row-major matrix gives it sixteen halves of lines K elements apart, and a
+// wave that walks along K reads tile after tile.  The kernels for at most 64 rows, which take their
+// weights straight from memory into MFMA operands, read this copy where the caller has one (the
+// down product at 8 rows: 26.7 us from 34.1).  WSTEP: elements from one step of 32 k to the next.
+template <bool TILED>
+__device__ __forceinline__ const bf16* w_operand(const bf16* W, int ldw, int K, int row, int k) {
+  if constexpr (TILED) return W + ((size_t)(row >> 4) * (K >> 5) + (k >> 5)) * 512 + (row & 15) * 32 + (k & 31);
+  else return W + (size_t)row * ldw + k;
+}
+
 // The same product where every chunk is whole (K and the splits in multiples of 256, aligned rows),
 // as a ring: each wave keeps its 8 weight fragments of a chunk in registers and refills one right
 // behind the MFMA that used it, with the next chunk's, so the loads in flight never run dry at a
 // chunk's end as they do above; the sums leave through an LDS tile, in rows of 512 bytes.
 constexpr int SR_LD = 128 + 4;      // row stride of that tile (floats)
 
-template <int MT>
+template <int MT, bool TILED>
 __global__ __launch_bounds__(512) void skinny_ring_kernel(const bf16* __restrict__ A, int lda,
                                                           const bf16* __restrict__ W, int ldw,
                                                           const float* __restrict__ bias,
@@ -615,7 +628,8 @@ __global__ __launch_bounds__(512) void skinny_ring_kernel(const bf16* __restrict
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int r16 = lane & 15, kq = (lane >> 4) * 8;
   const int n0 = blockIdx.x * 128;
-  const bf16* wrow = W + (size_t)min(n0 + wid * 16 + r16, N - 1) * ldw + kq;
+  constexpr int WSTEP = TILED ? 512 : 32;
+  const bf16* wrow = w_operand<TILED>(W, ldw, K, min(n0 + wid * 16 + r16, N - 1), kq);
   const int k_begin = blockIdx.y * k_per_split;
   const int k_end = min(K, k_begin + k_per_split);
   const int sk = (tid & 31) * 8;
@@ -626,7 +640,7 @@ __global__ __launch_bounds__(512) void skinny_ring_kernel(const bf16* __restrict
 #pragma unroll
   for (int i = 0; i < MT; ++i) stage[i] = *reinterpret_cast<const bf16x8*>(src[i] + k_begin);
 #pragma unroll
-  for (int s = 0; s < KC / 32; ++s) wr[s] = *reinterpret_cast<const bf16x8*>(wrow + k_begin + s * 32);
+  for (int s = 0; s < KC / 32; ++s) wr[s] = *reinterpret_cast<const bf16x8*>(wrow + ((k_begin >> 5) + s) * WSTEP);
 #pragma unroll
   for (int i = 0; i < MT; ++i)
     *reinterpret_cast<bf16x8*>(&As[(i * 16 + (tid >> 5)) * SK_LD + sk]) = stage[i];
@@ -648,7 +662,7 @@ __global__ __launch_bounds__(512) void skinny_ring_kernel(const bf16* __restrict
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(&as[(i * 16 + r16) * SK_LD + s * 32 + kq]);
         acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, wr[s], acc[i], 0, 0, 0);
       }
-      wr[s] = *reinterpret_cast<const bf16x8*>(wrow + kn + s * 32);
+      wr[s] = *reinterpret_cast<const bf16x8*>(wrow + ((kn >> 5) + s) * WSTEP);
       __builtin_amdgcn_sched_barrier(0);      // use a register, then refill it, in this order
     }
     buf ^= 1;
@@ -838,19 +852,6 @@ bool panel_takes(int M, int N, int K, bool aligned, int epi, int n_cu) {
 // the ring form of the K-split kernel needs whole chunks of 256 in every split
 bool ring_takes(bool aligned, int K, int splits, int k_per_split) {
   return aligned && K % 256 == 0 && (long)(splits - 1) * k_per_split < K;
-}
-
-// The tiled copy of a weight matrix (K a multiple of 32, rows padded to a multiple of 16):
-// [rows / 16][K / 32][16 rows][32 k], 1 KB a tile.  A wave's load of an MFMA operand (lane ->
-// row lane % 16, eight k at 8 (lane / 16)) is one tile: a contiguous kilobyte of whole 128-byte
-// lines, where the row-major matrix gives it sixteen halves of lines K elements apart, and a
-// wave that walks along K reads tile after tile.  The kernels for at most 64 rows, which take their
-// weights straight from memory into MFMA operands, read this copy where the caller has one (the
-// down product at 8 rows: 26.7 us from 34.1).  WSTEP: elements from one step of 32 k to the next.
-template <bool TILED>
-__device__ __forceinline__ const bf16* w_operand(const bf16* W, int ldw, int K, int row, int k) {
-  if constexpr (TILED) return W + ((size_t)(row >> 4) * (K >> 5) + (k >> 5)) * 512 + (row & 15) * 32 + (k & 31);
-  else return W + (size_t)row * ldw + k;
 }
 
 // The same split of the work as skinny16_kernel (a block owns 16 NT weight rows, its waves split
@@ -1330,7 +1331,7 @@ int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const fl
 constexpr int PANEL_TILES = 16;                 // tiles of a pass
 constexpr int OT_LD = PANEL_TILES * 16 + 4;     // row stride of the output tile in LDS (floats)
 
-template <int MT>
+template <int MT, bool TILED>
 __global__ __launch_bounds__(512) void panel_kernel(const bf16* __restrict__ A, int lda,
                                                     const bf16* __restrict__ W, int ldw,
                                                     const float* __restrict__ bias, void* __restrict__ C,
@@ -1341,6 +1342,7 @@ __global__ __launch_bounds__(512) void panel_kernel(const bf16* __restrict__ A, 
   float* ot = reinterpret_cast<float*>(smem + 2 * ROWS * SK_LD * sizeof(bf16));        // [ROWS][OT_LD]
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int r16 = lane & 15, kq = (lane >> 4) * 8;
+  constexpr int WSTEP = TILED ? 512 : 32;
   const bool pair = epi == EPI_SWIGLU;
   // a unit is 32 weight rows: 32 outputs, or (pair) 16 gate rows and the 16 up rows of the same outputs
   const int u_begin = (int)((long)blockIdx.x * units_total / gridDim.x);
@@ -1358,7 +1360,7 @@ __global__ __launch_bounds__(512) void panel_kernel(const bf16* __restrict__ A, 
     if (t >= cnt) return W;                                // no tile
     const int u = u_begin + p * per_u + (t >> 1), which = t & 1;
     const int row0 = pair ? (u >> 1) * 64 + (u & 1) * 16 + 32 * which : u * 32 + 16 * which;
-    return W + (size_t)min(row0 + r16, N - 1) * ldw + kq;
+    return w_operand<TILED>(W, ldw, K, min(row0 + r16, N - 1), kq);
   };
   // staging: this thread handles rows i * 16 + tid / 32, k (tid % 32) * 8 of a chunk
   const int sk = (tid & 31) * 8;
@@ -1381,8 +1383,8 @@ __global__ __launch_bounds__(512) void panel_kernel(const bf16* __restrict__ A, 
   load_stage(0);
 #pragma unroll
   for (int s = 0; s < KC / 32; ++s) {
-    wr[0][s] = *reinterpret_cast<const bf16x8*>(wp[0] + s * 32);
-    wr[1][s] = *reinterpret_cast<const bf16x8*>(wp[1] + s * 32);
+    wr[0][s] = *reinterpret_cast<const bf16x8*>(wp[0] + s * WSTEP);
+    wr[1][s] = *reinterpret_cast<const bf16x8*>(wp[1] + s * WSTEP);
   }
   store_stage(0);
   __syncthreads();
@@ -1414,7 +1416,7 @@ __global__ __launch_bounds__(512) void panel_kernel(const bf16* __restrict__ A, 
 #pragma unroll
         for (int i = 0; i < MT; ++i)
           acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], wr[j][s], acc[j][i], 0, 0, 0);
-        wr[j][s] = *reinterpret_cast<const bf16x8*>(wnext[j] + kn + s * 32);
+        wr[j][s] = *reinterpret_cast<const bf16x8*>(wnext[j] + ((kn >> 5) + s) * WSTEP);
         __builtin_amdgcn_sched_barrier(0);      // use a register, then refill it, in this order
       }
     }
@@ -1490,8 +1492,8 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
 }
 
 template <int MT, bool VEC>
-int launch_skinny_v(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
-                    float* part, int M, int N, int K, int splits, int k_per_split, int epi,
+int launch_skinny_v(const bf16* A, int lda, const bf16* W, const bf16* Wt, int ldw, const float* bias, void* C,
+                    int ldc, float* part, int M, int N, int K, int splits, int k_per_split, int epi,
                     hipStream_t stream) {
   constexpr int smem = 2 * MT * 16 * SK_LD * (int)sizeof(bf16);
   static bool configured = false;
@@ -1508,13 +1510,20 @@ int launch_skinny_v(const bf16* A, int lda, const bf16* W, int ldw, const float*
     constexpr int smem_ring = smem + MT * 16 * SR_LD * (int)sizeof(float);
     static bool ring_configured = false;
     if (!ring_configured) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_ring_kernel<MT>),
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_ring_kernel<MT, false>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, smem_ring);
+      if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_ring_kernel<MT, true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, smem_ring);
       if (e != hipSuccess) return (int)e;
       ring_configured = true;
     }
-    skinny_ring_kernel<MT><<<grid, 512, smem_ring, stream>>>(A, lda, W, ldw, bias, C, ldc,
-                                                             two_pass ? part : nullptr, M, N, K, k_per_split, epi);
+    if (Wt)
+      skinny_ring_kernel<MT, true><<<grid, 512, smem_ring, stream>>>(A, lda, Wt, ldw, bias, C, ldc, two_pass ? part : nullptr,
+                                                                     M, N, K, k_per_split, epi);
+    else
+      skinny_ring_kernel<MT, false><<<grid, 512, smem_ring, stream>>>(A, lda, W, ldw, bias, C, ldc, two_pass ? part : nullptr,
+                                                                      M, N, K, k_per_split, epi);
   } else {
     kern<<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, two_pass ? part : nullptr, M, N, K,
                                       k_per_split, epi);
@@ -1529,44 +1538,50 @@ int launch_skinny_v(const bf16* A, int lda, const bf16* W, int ldw, const float*
 }
 
 template <int MT>
-int launch_skinny(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
-                  float* part, int M, int N, int K, int splits, int k_per_split, int epi, int vec_ok,
+int launch_skinny(const bf16* A, int lda, const bf16* W, const bf16* Wt, int ldw, const float* bias, void* C,
+                  int ldc, float* part, int M, int N, int K, int splits, int k_per_split, int epi, int vec_ok,
                   hipStream_t stream) {
-  return vec_ok ? launch_skinny_v<MT, true>(A, lda, W, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split,
+  return vec_ok ? launch_skinny_v<MT, true>(A, lda, W, Wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split,
                                             epi, stream)
-                : launch_skinny_v<MT, false>(A, lda, W, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split,
-                                             epi, stream);
+                : launch_skinny_v<MT, false>(A, lda, W, nullptr, ldw, bias, C, ldc, part, M, N, K, splits,
+                                             k_per_split, epi, stream);
 }
 
 // The whole-K kernel for 17 to 64 rows, where the matrix is wide enough to give every CU at least
 // 8 tiles; MF_NOT_BUILT (nothing launched) for any other shape.
 constexpr int MF_NOT_BUILT = -2;
-template <int MT>
+template <int MT, bool TILED>
 int launch_panel_mt(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc, int M,
                     int N, int K, int epi, int grid, int units, hipStream_t stream) {
   constexpr int smem = 2 * MT * 16 * SK_LD * (int)sizeof(bf16) + MT * 16 * OT_LD * (int)sizeof(float);
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(panel_kernel<MT>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(panel_kernel<MT, TILED>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     configured = true;
   }
-  panel_kernel<MT><<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, units, epi);
+  panel_kernel<MT, TILED><<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, units, epi);
   return mf_launch_status();
 }
 
-int launch_panel(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc, int M, int N,
-                 int K, int epi, hipStream_t stream) {
+int launch_panel(const bf16* A, int lda, const bf16* W, const bf16* Wt, int ldw, const float* bias, void* C, int ldc,
+                 int M, int N, int K, int epi, hipStream_t stream) {
   const int n_cu = cu_count();
   if (n_cu <= 0) return (int)hipErrorUnknown;
   const bool aligned = ldw % 8 == 0 && (uintptr_t)W % 16 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0;
   if (!panel_takes(M, N, K, aligned, epi, n_cu)) return MF_NOT_BUILT;
   const int units = (N + 31) / 32;
   switch ((M + 15) / 16) {
-    case 2: return launch_panel_mt<2>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
-    case 3: return launch_panel_mt<3>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
-    case 4: return launch_panel_mt<4>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
+    case 2:
+      return Wt ? launch_panel_mt<2, true>(A, lda, Wt, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream)
+                : launch_panel_mt<2, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
+    case 3:
+      return Wt ? launch_panel_mt<3, true>(A, lda, Wt, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream)
+                : launch_panel_mt<3, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
+    case 4:
+      return Wt ? launch_panel_mt<4, true>(A, lda, Wt, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream)
+                : launch_panel_mt<4, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
   }
   return MF_NOT_BUILT;
 }
@@ -1786,14 +1801,14 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, const void
     case SK_GUARDED_4X2: return launch_skinny16<4, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case SK_GUARDED_8X2: return launch_skinny16<8, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case SK_GUARDED_8X1: return launch_skinny16<8, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    case SK_PANEL: return launch_panel(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+    case SK_PANEL: return launch_panel(a, lda, w, wt, ldw, bias, C, ldc, M, N, K, epi, stream);
     default: break;
   }
   switch ((M + 15) / 16) {
-    case 1: return launch_skinny<1>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
-    case 2: return launch_skinny<2>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
-    case 3: return launch_skinny<3>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
-    case 4: return launch_skinny<4>(a, lda, w, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
+    case 1: return launch_skinny<1>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
+    case 2: return launch_skinny<2>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
+    case 3: return launch_skinny<3>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
+    case 4: return launch_skinny<4>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
   }
   return (int)hipErrorInvalidValue;
 }

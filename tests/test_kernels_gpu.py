@@ -557,9 +557,12 @@ def test_tile_weight_layout(ops):
 
 
 @pytest.mark.parametrize("m,n,k", [(8, 3584, 18944), (1, 1000, 8224), (16, 4608, 3584), (5, 152064, 1536),
-                                   (3, 2100, 8192), (16, 8192, 8192), (8, 90, 4096), (2, 2048, 96)])
+                                   (3, 2100, 8192), (16, 8192, 8192), (8, 90, 4096), (2, 2048, 96),
+                                   # 17 to 64 rows: K split over blocks, and the whole-K kernel of a wide matrix
+                                   (64, 3584, 3584), (40, 3584, 18944), (17, 1000, 2048), (33, 40001, 768),
+                                   (64, 33000, 512)])
 def test_gemm_bf16_tiled_copy_same_bits(ops, m, n, k):
-    """The products of at most 16 rows read the tiled copy of the weights where they are given one:
+    """The products of at most 64 rows read the tiled copy of the weights where they are given one:
     the same sums in the same order, so the same bits as from the matrix itself, for every
     epilogue, with and without the folded norm; and right against the plain product."""
     x, w, b = rnd((m, k), torch.bfloat16, 120), rnd((n, k), torch.bfloat16, 121, 0.05), rnd((n,), seed=122)
@@ -585,7 +588,8 @@ def test_gemm_bf16_tiled_copy_same_bits(ops, m, n, k):
         assert torch.equal(a, c)
 
 
-@pytest.mark.parametrize("m,nf,k", [(8, 18944, 3584), (1, 1024, 2048), (16, 1030, 4096), (3, 2100, 8192)])
+@pytest.mark.parametrize("m,nf,k", [(8, 18944, 3584), (1, 1024, 2048), (16, 1030, 4096), (3, 2100, 8192),
+                                    (64, 18944, 512), (33, 16400, 256), (40, 300, 512)])
 def test_gemm_bf16_swiglu_tiled_copy_same_bits(ops, m, nf, k):
     gate, up = rnd((nf, k), torch.bfloat16, 130, 0.05), rnd((nf, k), torch.bfloat16, 131, 0.05)
     w = ops.interleave_gate_up(gate.to(DEV), up.to(DEV))
