@@ -287,7 +287,8 @@ def main() -> int:
                    "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
                    "global_batch": a.batch, "seq_len": a.context, "prompt_max": a.prompt_max,
                    "prefill_tokens": a.prefill_tokens, "parallelism": "single GPU",
-                   "decode_graph": not a.no_graph, "cache_tokens": plan["tokens"]},
+                   "decode_graph": not a.no_graph, "cache_tokens": plan["tokens"],
+                   "tiled_weight_copies_gib": round(getattr(llm.model, "decode_copy_bytes", 0) / 2 ** 30, 2)},
         "prefill": {"value": round(a.prefill_tokens / pre_s, 1), "tokens": a.prefill_tokens,
                     "ms": round(pre_s * 1e3, 3), "frac": round(flops / pre_s / PEAK_FLOPS[a.dtype], 4),
                     "measured_peak": round(mfma_flops / 1e12, 1), "unit": "TFLOP/s (bf16 MFMA loop in registers)"},

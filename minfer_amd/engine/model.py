@@ -41,6 +41,7 @@ class DecoderModel:
         self.head = make_part(HEADS, spec.head, self.rt, "head")
         self.stop_tokens = tuple(spec.stop_tokens)      # a loader may add to them (generation_config.json)
         self.loaded = False
+        self.decode_copy_bytes = 0      # of the parts' tiled second copies, once loaded
 
     # ------------------------------------------------------------ tensors
     def expected_tensors(self) -> Dict[str, TensorSpec]:
