@@ -377,21 +377,22 @@ def stationary_shape(n: int, k: int, folded: bool = False) -> bool:
 
 
 def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None,
-                swiglu: bool = False) -> Tuple[int, int]:
+                swiglu: bool = False, tiled: bool = False) -> Tuple[int, int]:
     """(splits, k_per_split) of a product with at most 64 rows.  One split: one kernel, K divided
     between the waves of a block.  More: blocks of 128 weight rows with the activations staged in
     LDS, K split so that there is about one block per CU, and a second kernel that adds the parts.
 
     At most 16 rows take the one-kernel form, except against a K of 8192 and more that the
     register-resident kernel does not hold, where it does badly from 9 rows on (every block reads
-    its own copy of the activations from L2) and where a CU's share of the weight rows fills its
-    16-row tiles poorly."""
+    its own copy of the activations from L2; from 13 rows on where it reads the tiled copy of the
+    weights: the down product of the 7B shape at 12 rows 28.9 us against 29.9, at 16 rows 32.4
+    against 30.4) and where a CU's share of the weight rows fills its 16-row tiles poorly."""
     if target_blocks is None:
         target_blocks = tuning.SKINNY_TARGET or cu_count()
     if m <= 16:
         share = (n + target_blocks - 1) // target_blocks          # weight rows of a block in the one-kernel form
         fill = share / float((share + 15) // 16 * 16)
-        if k < 8192 or (m <= 8 and fill >= 0.8) or stationary_shape(n, k, swiglu):
+        if k < 8192 or (m <= (12 if tiled else 8) and fill >= 0.8) or stationary_shape(n, k, swiglu):
             return 1, (k + 255) // 256 * 256
     n_blocks = (n + 127) // 128
     chunks = (k + 255) // 256
@@ -411,19 +412,22 @@ def tile_plan(m: int, n: int, k: int, epi: int, aligned: bool = True, n_cu: Opti
     return out[0], out[1], out[2]
 
 
-def _k_split(m: int, n: int, k: int, swiglu: bool, aligned: bool, n_cu: Optional[int] = None) -> Tuple[int, int]:
+def _k_split(m: int, n: int, k: int, swiglu: bool, aligned: bool, n_cu: Optional[int] = None,
+             tiled: bool = False) -> Tuple[int, int]:
     """(splits, k_per_split) as `linear` and `linear_swiglu` cut a bfloat16 product of at most 64 rows."""
     target = tuning.SKINNY_TARGET or n_cu
-    return skinny_plan(m, n, k, target_blocks=target, swiglu=swiglu)
+    return skinny_plan(m, n, k, target_blocks=target, swiglu=swiglu, tiled=tiled)
 
 
 def plan_linear(m: int, n: int, k: int, swiglu: bool = False, normed: bool = False, aligned: bool = True,
-                out_bf16: bool = False, accumulate: bool = False, n_cu: Optional[int] = None) -> Dict[str, object]:
+                out_bf16: bool = False, accumulate: bool = False, n_cu: Optional[int] = None,
+                tiled: bool = False) -> Dict[str, object]:
     """Which kernel `linear` / `linear_swiglu` / `linear_normed` runs for a bfloat16 product of
     `m` rows against `[n][k]` weights, as the library itself decides it, without launching
     anything: {'kernel': name, 'splits': s, 'k_per_split': per}.  With `normed` an empty name
     means that no kernel folds the norm in at this shape (norm and product then run one after
-    the other).  `n` counts the interleaved gate|up rows for `swiglu`."""
+    the other).  `n` counts the interleaved gate|up rows for `swiglu`; `tiled`: the product is
+    given the tiled copy of the weights (it moves the row count from which K is cut over blocks)."""
     n_cu = n_cu or cu_count()
     epi = EPI_SWIGLU if swiglu else (EPI_BF16 if out_bf16 else (EPI_ACC_F32 if accumulate else EPI_F32))
     splits, per = 1, k
@@ -431,7 +435,7 @@ def plan_linear(m: int, n: int, k: int, swiglu: bool = False, normed: bool = Fal
         if m > 16 or tuning.NO_FOLD:
             return dict(kernel="", splits=1, k_per_split=k)
     elif m <= 64:
-        splits, per = _k_split(m, n, k, swiglu, aligned, n_cu)
+        splits, per = _k_split(m, n, k, swiglu, aligned, n_cu, tiled)
     else:
         _, splits, per = tile_plan(m, n, k, epi, aligned, n_cu)
     name = ctypes.create_string_buffer(64)
@@ -489,7 +493,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
     epi = EPI_BF16 if out.dtype == torch.bfloat16 else (EPI_ACC_F32 if accumulate else EPI_F32)
     aligned = not (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8)
     if m <= 64 and variant == 0:
-        splits, per = _k_split(m, n, k, False, aligned)
+        splits, per = _k_split(m, n, k, False, aligned, tiled=tiled is not None)
         part = workspace("skinny", splits * m * n, x.device) if splits > 1 else None
         _need_tiled(tiled, "linear.tiled", n, k)
         _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), _ptr(tiled), k, _ptr(bias),
@@ -536,7 +540,7 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, vari
         return
     aligned = not (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8)
     if m <= 64 and variant == 0:
-        splits, per = _k_split(m, n, k, True, aligned)
+        splits, per = _k_split(m, n, k, True, aligned, tiled=tiled is not None)
         part = workspace("skinny", splits * m * n, x.device) if m > 16 or splits > 1 else None
         _need_tiled(tiled, "linear_swiglu.tiled", n, k)
         _check(_fn("gemm_bf16", "mf_gemm_bf16_skinny")(_ptr(x), k, _ptr(weight), _ptr(tiled), k, _ptr(None), _ptr(out), nf,
