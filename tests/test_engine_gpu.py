@@ -111,6 +111,33 @@ def test_truncate_then_feed_again_gives_the_same_rows(folders, plains, dtype):
         eng.truncate(s2, 5)
 
 
+def test_tiled_copies_of_the_weights_change_no_bit(folders):
+    """A bfloat16 model keeps tiled second copies of its matrices for the steps of few tokens
+    where the row length allows (a multiple of 32) and the device has room: the same logits, bit
+    for bit, as without them, for prompts whole and for tokens one by one; none in 32 bits."""
+    import numpy as np
+    from minfer_amd import Engine, load_model
+    from minfer_amd.kernels import tuning
+    reqs = requests_for(TINIES["B"]["vocab_size"], (40, 7, 90), seed=8)
+    out = {}
+    for copies in (True, False):
+        tuning.NO_DECODE_COPIES = not copies
+        try:
+            model = load_model(folders["B"], dtype="bfloat16", device="cuda:0")
+        finally:
+            tuning.NO_DECODE_COPIES = False
+        assert (model.decode_copy_bytes > 0) == copies
+        assert (model.blocks[0].mixer.qkv.tiled is not None) == copies
+        assert model.blocks[0].feed_forward.down.tiled is None        # rows of 344: no multiple of 32
+        eng = Engine(model, max_tokens=64 * 8, poison_cache=True)
+        out[copies] = (run_steps(eng, tail_steps(reqs)), run_steps(eng, batch_steps(reqs, [list(reqs)])))
+    for with_copies, without in zip(out[True], out[False]):
+        assert with_copies.keys() == without.keys()
+        for key in with_copies:
+            assert np.array_equal(with_copies[key], without[key]), key
+    assert load_model(folders["B"], dtype="float32", device="cuda:0").decode_copy_bytes == 0
+
+
 def test_random_model_on_the_device_is_the_written_folder(tmp_path):
     """`write_random_model` + `load_model` and `random_model` give the same tensors for the same
     configuration and seed, in both run types: one stream of random numbers, host and device."""
