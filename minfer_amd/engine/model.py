@@ -81,16 +81,19 @@ class DecoderModel:
 
     def _make_decode_copies(self) -> int:
         """The parts' second copies of their matrices for the steps of few tokens (a layout that
-        those steps' products read faster), all of them or none: made where they take at most a
-        third of the device memory that is free once the weights are in place, so that a model
-        that fills the device keeps its memory for the cache.  Returns their bytes."""
+        those steps' products read faster): of all matrices where that takes at most a third of
+        the device memory that is free once the weights are in place, else of those with rows of
+        16,384 and more (the down products, which gain most) under the same condition, else
+        none, so that a model that fills the device keeps its memory for the cache.  Returns
+        their bytes."""
         if not self.rt.is_bf16 or self.rt.device.type != "cuda" or tuning.NO_DECODE_COPIES:
             return 0
-        need = sum(part.decode_copies(False) for part in self._all_parts())
         free, _ = torch.cuda.mem_get_info(self.rt.device)
-        if need == 0 or need > free // 3:
-            return 0
-        return sum(part.decode_copies(True) for part in self._all_parts())
+        for min_row_length in (0, 16384):
+            need = sum(part.decode_copies(False, min_row_length) for part in self._all_parts())
+            if 0 < need <= free // 3:
+                return sum(part.decode_copies(True, min_row_length) for part in self._all_parts())
+        return 0
 
     # ------------------------------------------------------------ cache needs
     def cache_requests(self) -> Dict[int, object]:

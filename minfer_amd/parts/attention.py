@@ -62,8 +62,8 @@ class GQAttention(Mixer):
     def cache_request(self):
         return KVRequest(self.nk, self.hd, None if self.window is None else int(self.window))
 
-    def decode_copies(self, make: bool) -> int:
-        return self.qkv.decode_copy(make) + self.o.decode_copy(make)
+    def decode_copies(self, make: bool, min_row_length: int = 0) -> int:
+        return self.qkv.decode_copy(make, min_row_length) + self.o.decode_copy(make, min_row_length)
 
     def prepare(self, max_len: int) -> None:
         self.position.prepare(max_len)

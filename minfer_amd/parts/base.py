@@ -48,10 +48,11 @@ class Part:
         """Called before steps that may reach `max_len` positions (tables, workspaces), so
         that a captured step allocates nothing of its own."""
 
-    def decode_copies(self, make: bool) -> int:
-        """Bytes of the second copies of its matrices that this part would keep for the steps of
-        few tokens (`Linear.decode_copy`); made when `make`.  The model asks all parts first and
-        makes the copies only where the device has the memory to spare."""
+    def decode_copies(self, make: bool, min_row_length: int = 0) -> int:
+        """Bytes of the second copies of its matrices (those with rows of at least
+        `min_row_length`) that this part would keep for the steps of few tokens
+        (`Linear.decode_copy`); made when `make`.  The model asks all parts first and makes the
+        copies only where the device has the memory to spare."""
         return 0
 
 

@@ -66,8 +66,8 @@ class LinearHead(Head):
     def weight(self) -> torch.Tensor:
         return self.linear.weight
 
-    def decode_copies(self, make: bool) -> int:
-        return self.linear.decode_copy(make)
+    def decode_copies(self, make: bool, min_row_length: int = 0) -> int:
+        return self.linear.decode_copy(make, min_row_length)
 
     def forward(self, x) -> torch.Tensor:
         return self.linear(x, out_dtype=torch.float32)

@@ -39,14 +39,15 @@ class SwiGLU(FeedForward):
             self.gate_up = Linear.stacked([gate, up])
         self.down = Linear(get(n["down"] + ".weight"))
 
-    def decode_copies(self, make: bool) -> int:
-        n = self.down.decode_copy(make)
-        if self.fused is not None and self.hidden % 32 == 0:
-            if make and self.fused_tiled is None:
-                self.fused_tiled = ops.tile_weight(self.fused)
-            n += self.fused.numel() * 2
+    def decode_copies(self, make: bool, min_row_length: int = 0) -> int:
+        n = self.down.decode_copy(make, min_row_length)
+        if self.fused is not None:
+            if self.hidden % 32 == 0 and self.hidden >= min_row_length:
+                if make and self.fused_tiled is None:
+                    self.fused_tiled = ops.tile_weight(self.fused)
+                n += self.fused.numel() * 2
         elif self.gate_up is not None:
-            n += self.gate_up.decode_copy(make)
+            n += self.gate_up.decode_copy(make, min_row_length)
         return n
 
     takes_normed = True

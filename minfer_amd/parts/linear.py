@@ -28,11 +28,11 @@ class Linear:
         self.out_features, self.in_features = weight.shape
         self.tiled: Optional[torch.Tensor] = None      # ops.tile_weight(weight), where the model keeps one
 
-    def decode_copy(self, make: bool) -> int:
+    def decode_copy(self, make: bool, min_row_length: int = 0) -> int:
         """Bytes of the tiled copy of this matrix, which the products of few rows read faster than
-        the matrix itself (0: it has none: 32-bit, or a row length that is no multiple of 32);
-        made when `make`."""
-        if self.weight.dtype != torch.bfloat16 or self.in_features % 32:
+        the matrix itself (0: it has none: 32-bit, a row length that is no multiple of 32, or a
+        row shorter than `min_row_length`: the long rows gain most); made when `make`."""
+        if self.weight.dtype != torch.bfloat16 or self.in_features % 32 or self.in_features < min_row_length:
             return 0
         if make and self.tiled is None:
             self.tiled = ops.tile_weight(self.weight)
