@@ -20,9 +20,9 @@
 //    staged in LDS and shared by the block, K may be split over blocks with a fixed-order
 //    reduction afterwards.
 // Both operands have K contiguous, which is exactly the MFMA operand layout (8 consecutive
-// k per lane), so nothing is transposed.  The kernels for at most 64 rows (all but the two tile
-// kernels and skinny16_kernel) can read the weights from a tiled copy instead (`w_operand`),
-// where the caller has one.
+// k per lane), so nothing is transposed.  Four of the kernels for at most 64 rows (stationary16,
+// rolling16, skinny_ring and panel) can read the weights from a tiled copy instead
+// (`w_operand`), where the caller has one.
 //
 // Epilogues: 0 store fp32, 1 add into fp32 (residual stream), 2 store bf16, 3 SwiGLU.
 // SwiGLU (y = silu(g) * u, silu(z) = z / (1 + exp(-z)), src/graph/cpu_backend.rs:323-329):
