@@ -588,6 +588,22 @@ def test_gemm_bf16_tiled_copy_same_bits(ops, m, n, k):
         assert torch.equal(a, c)
 
 
+def test_gemm_bf16_tiled_copy_moves_the_one_kernel_limit(ops):
+    """9 to 12 rows against a long K: with the tiled copy the one-kernel form is the faster one,
+    without it K cut over blocks and a second kernel.  Two orders of addition: both right, not
+    the same bits."""
+    m, n, k = 10, 3584, 18944
+    assert ops.plan_linear(m, n, k)["kernel"] == "skinny_ring_kernel"
+    assert ops.plan_linear(m, n, k, tiled=True)["kernel"] == "rolling16_kernel"
+    x, w = rnd((m, k), torch.bfloat16, 140), rnd((n, k), torch.bfloat16, 141, 0.05)
+    xd, wd = x.to(DEV), w.to(DEV)
+    ref = x.double() @ w.double().t()
+    for tiled in (None, ops.tile_weight(wd)):
+        out = torch.empty(m, n, device=DEV)
+        ops.linear(xd, wd, None, out, tiled=tiled)
+        close(out, ref, 2e-5 * math.sqrt(k), 1e-5)
+
+
 @pytest.mark.parametrize("m,nf,k", [(8, 18944, 3584), (1, 1024, 2048), (16, 1030, 4096), (3, 2100, 8192),
                                     (64, 18944, 512), (33, 16400, 256), (40, 300, 512)])
 def test_gemm_bf16_swiglu_tiled_copy_same_bits(ops, m, nf, k):
