@@ -20,9 +20,9 @@
 //    staged in LDS and shared by the block, K may be split over blocks with a fixed-order
 //    reduction afterwards.
 // Both operands have K contiguous, which is exactly the MFMA operand layout (8 consecutive
-// k per lane), so nothing is transposed.  Four of the kernels for at most 64 rows (stationary16,
-// rolling16, skinny_ring and panel) can read the weights from a tiled copy instead
-// (`w_operand`), where the caller has one.
+// k per lane), so nothing is transposed.  The kernels for at most 64 rows (all but the guarded
+// skinny16_kernel) can read the weights from a tiled copy instead (`w_operand`), where the
+// caller has one.
 //
 // Epilogues: 0 store fp32, 1 add into fp32 (residual stream), 2 store bf16, 3 SwiGLU.
 // SwiGLU (y = silu(g) * u, silu(z) = z / (1 + exp(-z)), src/graph/cpu_backend.rs:323-329):
@@ -503,13 +503,26 @@ int launch_tile(const bf16* A, int lda, const bf16* W, int ldw, const float* bia
 constexpr int KC = 256;          // k per staging step
 constexpr int SK_LD = KC + 8;    // LDS row stride in elements
 
+// The tiled copy of a weight matrix (K a multiple of 32, rows padded to a multiple of 16):
+// [rows / 16][K / 32][16 rows][32 k], 1 KB a tile.  A wave's load of an MFMA operand (lane ->
+// row lane % 16, eight k at 8 (lane / 16)) is one tile: a contiguous kilobyte of whole 128-byte
+// lines, where the row-major matrix gives it sixteen halves of lines K elements apart, and a
+// wave that walks along K reads tile after tile.  The kernels for at most 64 rows, which take their
+// weights straight from memory into MFMA operands, read this copy where the caller has one (the
+// down product at 8 rows: 26.7 us from 34.1).  WSTEP: elements from one step of 32 k to the next.
+template <bool TILED>
+__device__ __forceinline__ const bf16* w_operand(const bf16* W, int ldw, int K, int row, int k) {
+  if constexpr (TILED) return W + ((size_t)(row >> 4) * (K >> 5) + (k >> 5)) * 512 + (row & 15) * 32 + (k & 31);
+  else return W + (size_t)row * ldw + k;
+}
+
 // 17 to 64 rows.  A block of 8 waves owns 128 weight rows; each wave streams its 16 rows from
 // HBM straight into MFMA operands, a chunk (256 k) ahead; the activation rows of a chunk are
 // staged in LDS once per block (double-buffered: the next chunk travels global -> registers
 // while this one is multiplied, and is written to the other buffer afterwards, so there is
 // one barrier per chunk).  Partial sums go to part[split][M][N]; with one split the epilogue
 // runs in place.
-template <int MT, bool VEC>
+template <int MT, bool VEC, bool TILED>
 __global__ __launch_bounds__(512) void skinny_kernel(const bf16* __restrict__ A, int lda,
                                                      const bf16* __restrict__ W, int ldw,
                                                      const float* __restrict__ bias, void* __restrict__ C,
@@ -541,12 +554,21 @@ __global__ __launch_bounds__(512) void skinny_kernel(const bf16* __restrict__ A,
   auto load_chunk = [&](int k0, bf16x8 (&wd)[KC / 32]) {
     if (VEC && k0 + KC <= k_end) {                     // inside: no guards, nothing waits
 #pragma unroll
-      for (int s = 0; s < KC / 32; ++s) wd[s] = load8_inside(W, ldw, n_ld, k0 + s * 32 + kq);
+      for (int s = 0; s < KC / 32; ++s)
+        wd[s] = *reinterpret_cast<const bf16x8*>(w_operand<TILED>(W, ldw, K, n_ld, k0 + s * 32 + kq));
 #pragma unroll
       for (int i = 0; i < MT; ++i) stage[i] = load8_inside(A, lda, min(srow[i], M - 1), k0 + sk[i]);
     } else {
 #pragma unroll
-      for (int s = 0; s < KC / 32; ++s) wd[s] = load8<VEC>(W, ldw, n_ld, k0 + s * 32 + kq, k_end);
+      for (int s = 0; s < KC / 32; ++s) {
+        const int k = k0 + s * 32 + kq;
+        if constexpr (TILED) {          // K in whole steps of 32: eight elements are all inside or all outside
+          const bf16x8 v = *reinterpret_cast<const bf16x8*>(w_operand<true>(W, ldw, K, n_ld, min(k, K - 8)));
+          wd[s] = k + 8 <= k_end ? v : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        } else {
+          wd[s] = load8<VEC>(W, ldw, n_ld, k, k_end);
+        }
+      }
 #pragma unroll
       for (int i = 0; i < MT; ++i) stage[i] = load8<VEC>(A, lda, min(srow[i], M - 1), k0 + sk[i], k_end);
     }
@@ -595,19 +617,6 @@ __global__ __launch_bounds__(512) void skinny_kernel(const bf16* __restrict__ A,
         store_out(C, ldc, m, n_row, acc[i][r] + (bias ? bias[n_row] : 0.f), epi);
       }
     }
-}
-
-// The tiled copy of a weight matrix (K a multiple of 32, rows padded to a multiple of 16):
-// [rows / 16][K / 32][16 rows][32 k], 1 KB a tile.  A wave's load of an MFMA operand (lane ->
-// row lane % 16, eight k at 8 (lane / 16)) is one tile: a contiguous kilobyte of whole 128-byte
-// lines, where the row-major matrix gives it sixteen halves of lines K elements apart, and a
-// wave that walks along K reads tile after tile.  The kernels for at most 64 rows, which take their
-// weights straight from memory into MFMA operands, read this copy where the caller has one (the
-// down product at 8 rows: 26.7 us from 34.1).  WSTEP: elements from one step of 32 k to the next.
-template <bool TILED>
-__device__ __forceinline__ const bf16* w_operand(const bf16* W, int ldw, int K, int row, int k) {
-  if constexpr (TILED) return W + ((size_t)(row >> 4) * (K >> 5) + (k >> 5)) * 512 + (row & 15) * 32 + (k & 31);
-  else return W + (size_t)row * ldw + k;
 }
 
 // The same product where every chunk is whole (K and the splits in multiples of 256, aligned rows),
@@ -1499,10 +1508,14 @@ int launch_skinny_v(const bf16* A, int lda, const bf16* W, const bf16* Wt, int l
                     hipStream_t stream) {
   constexpr int smem = 2 * MT * 16 * SK_LD * (int)sizeof(bf16);
   static bool configured = false;
-  auto kern = skinny_kernel<MT, VEC>;
+  const bool tiled = VEC && Wt != nullptr;
+  auto kern = tiled ? skinny_kernel<MT, VEC, VEC> : skinny_kernel<MT, VEC, false>;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_kernel<MT, VEC, false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_kernel<MT, VEC, VEC>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     configured = true;
   }
@@ -1527,7 +1540,7 @@ int launch_skinny_v(const bf16* A, int lda, const bf16* W, const bf16* Wt, int l
       skinny_ring_kernel<MT, false><<<grid, 512, smem_ring, stream>>>(A, lda, W, ldw, bias, C, ldc, two_pass ? part : nullptr,
                                                                       M, N, K, k_per_split, epi);
   } else {
-    kern<<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, two_pass ? part : nullptr, M, N, K,
+    kern<<<grid, 512, smem, stream>>>(A, lda, tiled ? Wt : W, ldw, bias, C, ldc, two_pass ? part : nullptr, M, N, K,
                                       k_per_split, epi);
   }
   int rc = mf_launch_status();

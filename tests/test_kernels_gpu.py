@@ -560,7 +560,9 @@ def test_tile_weight_layout(ops):
                                    (3, 2100, 8192), (16, 8192, 8192), (8, 90, 4096), (2, 2048, 96),
                                    # 17 to 64 rows: K split over blocks, and the whole-K kernel of a wide matrix
                                    (64, 3584, 3584), (40, 3584, 18944), (17, 1000, 2048), (33, 40001, 768),
-                                   (64, 33000, 512)])
+                                   (64, 33000, 512),
+                                   # 17 to 64 rows and a K that is no multiple of 256: the staged kernel
+                                   (40, 2048, 29568), (33, 1000, 1120), (64, 300, 96)])
 def test_gemm_bf16_tiled_copy_same_bits(ops, m, n, k):
     """The products of at most 64 rows read the tiled copy of the weights where they are given one:
     the same sums in the same order, so the same bits as from the matrix itself, for every
