@@ -427,7 +427,7 @@ __global__ __launch_bounds__(NT) void top_p_kernel(float* __restrict__ logits, i
 
 // ---------------------------------------------------------------- top-k, top-p and the draw in one
 // With a small k the three steps above need the row only once.  A first kernel cuts the row
-// into CAND_CHUNKS pieces, one block each, and lists each piece's k largest entries and every
+// into CAND_CHUNKS pieces, one wave each, and lists each piece's k largest entries and every
 // further entry equal to the k-th (largest first, equal values in index order): the row's k
 // largest and their ties are among them.  A second kernel, one block per row, merges the lists
 // into the row's survivors (the k largest and the ties of the k-th), and then does on these few
@@ -435,85 +435,128 @@ __global__ __launch_bounds__(NT) void top_p_kernel(float* __restrict__ logits, i
 // (probabilities as float, sums in double in index order).  The logits are not changed.  A piece
 // or a row with more ties than a list holds (a constant row, say) takes the kernels above
 // instead, inside the second kernel, which then does change the row.
-constexpr int CAND_CHUNKS = 32;      // pieces of a row
+constexpr int CAND_CHUNKS = 64;      // pieces of a row (the merge gives a lane to each)
 constexpr int CAND_CAP = 64;         // entries of a piece's list
-constexpr int CAND_EPT = 32;         // entries per thread of a piece: vocab <= 32 * 256 * 32
+constexpr int CAND_EPT = 64;         // most entries per lane of a piece: vocab <= 64 * 64 * 64
 constexpr int FAST_K_MAX = 48;       // the largest k that takes this path
 constexpr int SURV_CAP = 128;        // survivors of a row
 
-__global__ __launch_bounds__(256) void topk_candidates_kernel(const float* __restrict__ logits, int ld,
-                                                              int vocab, int k, float* __restrict__ cand_val,
-                                                              int* __restrict__ cand_idx,
-                                                              int* __restrict__ cand_n) {
-  __shared__ uint32_t s_key[2][4];
-  __shared__ int s_idx[2][4];
-  __shared__ float l_val[CAND_CAP];
-  __shared__ int l_idx[CAND_CAP];
-  const int rowi = blockIdx.y, chunk = blockIdx.x;
+// The largest entry of every piece, as a key (0: the piece has none above -inf).  The k-th largest
+// of a row's piece maxima is a bound from below on the row's k-th largest entry (they are k entries
+// of the row themselves), so the lists need nothing smaller: most pieces then list nothing or one.
+__global__ __launch_bounds__(256) void piece_max_kernel(const float* __restrict__ logits, int ld, int vocab,
+                                                        uint32_t* __restrict__ piece_max) {
+  const int lane = threadIdx.x & 63;
+  const int rowi = blockIdx.y, chunk = blockIdx.x * 4 + (threadIdx.x >> 6);
   const float* row = logits + (size_t)rowi * ld;
   const int per = (vocab + CAND_CHUNKS - 1) / CAND_CHUNKS;
   const int lo = chunk * per, n = max(0, min(per, vocab - lo));
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  // this thread's entries: lo + j * 256 + tid, as keys; 0 marks one that is out of play (no entry
-  // above -inf has a key that small, and those at or below -inf are never listed)
-  uint32_t key[CAND_EPT];
+  uint32_t best = 0;
+  for (int i0 = 0; i0 < n; i0 += 8 * 64) {            // eight loads on their way at a time
+    float x[8];
 #pragma unroll
-  for (int j = 0; j < CAND_EPT; ++j) {
-    const int i = j * 256 + (int)threadIdx.x;
+    for (int u = 0; u < 8; ++u) x[u] = row[lo + min(i0 + u * 64 + lane, n - 1)];     // (the last one again: a maximum does not mind)
+#pragma unroll
+    for (int u = 0; u < 8; ++u) best = max(best, order_key(x[u]));
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) best = max(best, (uint32_t)__shfl_xor((int)best, o, MF_WAVE));
+  if (lane == 0) piece_max[rowi * CAND_CHUNKS + chunk] = best <= 0x007FFFFFu ? 0u : best;
+}
+
+// One wave lists one piece (no barrier anywhere: a block is four pieces that know nothing of each
+// other): each lane holds its entries of the piece as keys, the wave takes the largest that is
+// still in play until the k-th and its ties are out or the next one is below the row's bound,
+// lane 0 writes it out.
+template <int EPT>      // entries per lane: a piece has at most 64 EPT
+__global__ __launch_bounds__(256) void topk_candidates_kernel(const float* __restrict__ logits, int ld,
+                                                              int vocab, int k,
+                                                              const uint32_t* __restrict__ piece_max,
+                                                              float* __restrict__ cand_val,
+                                                              int* __restrict__ cand_idx,
+                                                              int* __restrict__ cand_n) {
+  const int lane = threadIdx.x & 63;
+  const int rowi = blockIdx.y, chunk = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const float* row = logits + (size_t)rowi * ld;
+  const int per = (vocab + CAND_CHUNKS - 1) / CAND_CHUNKS;
+  const int lo = chunk * per, n = max(0, min(per, vocab - lo));
+  // the bound: lane c holds piece c's maximum; its place among the 64 (larger first, the lower piece
+  // among equals) is the number of lanes that come before it; the one at place k - 1 is the bound
+  static_assert(CAND_CHUNKS == 64 && FAST_K_MAX <= CAND_CHUNKS, "a lane for every piece, k pieces at least");
+  const uint32_t mine = piece_max[rowi * CAND_CHUNKS + lane];
+  int place = 0;
+  for (int c = 0; c < 64; ++c) {
+    const uint32_t other = (uint32_t)__shfl((int)mine, c, MF_WAVE);
+    place += (other > mine || (other == mine && c < lane)) ? 1 : 0;
+  }
+  const unsigned long long at = __builtin_amdgcn_ballot_w64(place == k - 1);
+  const uint32_t bound = (uint32_t)__shfl((int)mine, (int)__builtin_ctzll(at), MF_WAVE);    // 0: no bound
+  // this lane's entries: lo + j * 64 + lane, as keys; 0 marks one that is out of play (no entry
+  // above -inf has a key that small, and those at or below -inf are never listed)
+  uint32_t key[EPT];
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int i = j * 64 + lane;
     key[j] = i < n ? order_key(row[lo + i]) : 0u;
   }
+  const size_t base = ((size_t)rowi * CAND_CHUNKS + chunk) * CAND_CAP;
   int count = 0, over = 0;
   uint32_t kth = 0;
-  for (int it = 0;; ++it) {
-    // the largest entry of the block that is still in play, the lowest index among equals
+  for (;;) {
+    // the largest entry of the piece that is still in play, the lowest index among equals
     uint32_t bk = 0;
     int bj = 0;
 #pragma unroll
-    for (int j = 0; j < CAND_EPT; ++j)
+    for (int j = 0; j < EPT; ++j)
       if (key[j] > bk) { bk = key[j]; bj = j; }
-    const int bi = bj * 256 + (int)threadIdx.x;
-    uint32_t rk = bk;
-    int ri = bi;
+    const int bi = bj * 64 + lane;
+    uint32_t gk = bk;
+    int gi = bi;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
-      const uint32_t ok = __shfl_xor(rk, o, MF_WAVE);
-      const int oi = __shfl_xor(ri, o, MF_WAVE);
-      if (ok > rk || (ok == rk && oi < ri)) { rk = ok; ri = oi; }
-    }
-    const int b = it & 1;
-    if (lane == 0) { s_key[b][w] = rk; s_idx[b][w] = ri; }
-    __syncthreads();
-    uint32_t gk = s_key[b][0];
-    int gi = s_idx[b][0];
-#pragma unroll
-    for (int ww = 1; ww < 4; ++ww) {
-      const uint32_t ok = s_key[b][ww];
-      const int oi = s_idx[b][ww];
+      const uint32_t ok = __shfl_xor(gk, o, MF_WAVE);
+      const int oi = __shfl_xor(gi, o, MF_WAVE);
       if (ok > gk || (ok == gk && oi < gi)) { gk = ok; gi = oi; }
     }
     if (gk <= 0x007FFFFFu) break;                      // nothing left above -inf (which no step keeps alive)
+    if (gk < bound) break;                             // below the row's k-th largest for certain
     if (count >= k && gk != kth) break;                // past the k-th and its ties
     if (count == CAND_CAP) { over = 1; break; }        // more ties than the list holds
     if (count == k - 1) kth = gk;
-    if (threadIdx.x == 0) {
-      l_val[count] = key_value(gk);
-      l_idx[count] = lo + gi;
+    if (lane == 0) {
+      cand_val[base + count] = key_value(gk);
+      cand_idx[base + count] = lo + gi;
     }
     if (bk == gk && bi == gi) {
 #pragma unroll
-      for (int j = 0; j < CAND_EPT; ++j)
+      for (int j = 0; j < EPT; ++j)
         if (j == bj) key[j] = 0u;
     }
     ++count;
   }
-  __syncthreads();
-  const size_t base = ((size_t)rowi * CAND_CHUNKS + chunk) * CAND_CAP;
-  for (int i = threadIdx.x; i < count; i += 256) {
-    cand_val[base + i] = l_val[i];
-    cand_idx[base + i] = l_idx[i];
-  }
-  if (threadIdx.x == 0) cand_n[rowi * CAND_CHUNKS + chunk] = over ? -1 : count;
+  if (lane == 0) cand_n[rowi * CAND_CHUNKS + chunk] = over ? -1 : count;
 }
+
+// Sums that have to run one after the other (doubles, in a fixed order) run in wave 0 with the
+// terms in registers, place r in lane r % 64 (register r / 64), read out by lane number: a
+// thread that walks an LDS array instead waits for every element in turn.
+__device__ __forceinline__ float at_place(float lo, float hi, int r) {       // r the same in every lane
+  const int l = __builtin_amdgcn_readfirstlane(r & 63);
+  return __int_as_float(r < 64 ? __builtin_amdgcn_readlane(__float_as_int(lo), l)
+                               : __builtin_amdgcn_readlane(__float_as_int(hi), l));
+}
+__device__ __forceinline__ int at_place(int lo, int hi, int r) {
+  const int l = __builtin_amdgcn_readfirstlane(r & 63);
+  return r < 64 ? __builtin_amdgcn_readlane(lo, l) : __builtin_amdgcn_readlane(hi, l);
+}
+__device__ __forceinline__ double at_place(double lo, double hi, int r) {
+  const int l = __builtin_amdgcn_readfirstlane(r & 63);
+  const double x = r < 64 ? lo : hi;
+  const int a = __builtin_amdgcn_readlane(__double2loint(x), l), b = __builtin_amdgcn_readlane(__double2hiint(x), l);
+  return __hiloint2double(b, a);
+}
+
+constexpr int RANK_MAX = 512;        // candidates up to which each finds its place by counting the ones before it
 
 __global__ __launch_bounds__(NT) void sample_filtered_kernel(float* __restrict__ logits, int ld, int vocab, int k,
                                                              float top_p, float temp,
@@ -524,42 +567,91 @@ __global__ __launch_bounds__(NT) void sample_filtered_kernel(float* __restrict__
                                                              const int* __restrict__ cand_idx,
                                                              const int* __restrict__ cand_n,
                                                              int* __restrict__ out) {
-  __shared__ float v[SURV_CAP];        // survivors: value, index, probability, rank, alive
+  __shared__ float v[SURV_CAP];        // survivors: value, index, probability, alive
   __shared__ int ix[SURV_CAP];
   __shared__ float pr[SURV_CAP];
-  __shared__ int rank_p[SURV_CAP];     // place in (probability descending, index ascending)
-  __shared__ int rank_i[SURV_CAP];     // place in index order
   __shared__ int alive[SURV_CAP];
   __shared__ int order[SURV_CAP];      // survivor at a place
-  __shared__ int s_n, s_over;
-  __shared__ float c_val[CAND_CHUNKS * CAND_CAP];      // the pieces' lists
-  __shared__ int c_idx[CAND_CHUNKS * CAND_CAP];
-  __shared__ int c_n[CAND_CHUNKS];
+  __shared__ int s_n, s_over, s_total, s_keep;
+  __shared__ uint32_t s_kth;
+  __shared__ uint32_t d_key[CAND_CHUNKS * CAND_CAP];   // the pieces' lists one after the other, as keys
+  __shared__ int d_idx[CAND_CHUNKS * CAND_CAP];
+  __shared__ int c_n[CAND_CHUNKS], c_off[CAND_CHUNKS];
   const int rowi = blockIdx.x;
   float* row = logits + (size_t)rowi * ld;
   const int tid = threadIdx.x, lane = tid & 63;
-  if (tid == 0) { s_n = 0; s_over = 0; }
-  if (tid < CAND_CHUNKS) c_n[tid] = cand_n[rowi * CAND_CHUNKS + tid];
+  if (tid == 0) { s_n = 0; s_over = 0; s_kth = 0; }
   __syncthreads();
-  for (int i = tid; i < CAND_CHUNKS * CAND_CAP; i += NT) {
-    if ((i % CAND_CAP) < c_n[i / CAND_CAP]) {
-      c_val[i] = cand_val[(size_t)rowi * CAND_CHUNKS * CAND_CAP + i];
-      c_idx[i] = cand_idx[(size_t)rowi * CAND_CHUNKS * CAND_CAP + i];
+  if (tid < 64) {
+    // where each piece's list begins in the row's list
+    static_assert(CAND_CHUNKS == 64, "a lane for every piece");
+    const int cn = cand_n[rowi * CAND_CHUNKS + lane];
+    const bool piece_over = __builtin_amdgcn_ballot_w64(cn < 0) != 0;
+    const int cnt = max(cn, 0);
+    int incl = cnt;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o, MF_WAVE);
+      if (lane >= o) incl += up;
+    }
+    c_n[lane] = cnt;
+    c_off[lane] = incl - cnt;
+    if (lane == 63) s_total = incl;
+    if (lane == 0 && piece_over) s_over = 1;
+  }
+  __syncthreads();
+  const int C = s_total;
+  if (!s_over) {
+    // every piece's first entries in the first round (the lists are short as a rule: one wait for
+    // memory, not one per piece)
+    for (int s0 = 0; s0 < CAND_CAP; s0 += NT / CAND_CHUNKS) {
+      const int piece = tid % CAND_CHUNKS, slot = s0 + tid / CAND_CHUNKS;
+      if (slot < c_n[piece]) {
+        const size_t src = (size_t)rowi * CAND_CHUNKS * CAND_CAP + piece * CAND_CAP + slot;
+        d_key[c_off[piece] + slot] = order_key(cand_val[src]);
+        d_idx[c_off[piece] + slot] = cand_idx[src];
+      }
     }
   }
   __syncthreads();
-  if (tid < 64) {
-    // the pieces' lists are sorted: lane c holds the head of piece c's, the wave takes the best
-    // head (the lower piece among equals, which is the lower index) until the k-th and its ties are out
+  if (!s_over && C <= RANK_MAX) {
+    // Few candidates (the rule): each counts the ones that come before it (larger first, the lower
+    // index among equals), which is its place; the one at place k - 1 names the k-th value, and
+    // what is at least that survives, at its place.
+    static_assert(RANK_MAX <= NT, "a thread for every candidate");
+    uint32_t mk = 0;
+    int mi = 0, place = 0;
+    if (tid < C) {
+      mk = d_key[tid];
+      mi = d_idx[tid];
+      for (int j = 0; j < C; ++j) {
+        const uint32_t ok = d_key[j];
+        const int oi = d_idx[j];
+        place += (ok > mk || (ok == mk && oi < mi)) ? 1 : 0;
+      }
+      if (place == k - 1) s_kth = mk;
+    }
+    __syncthreads();
+    if (tid < C && mk >= s_kth) {
+      if (place < SURV_CAP) {
+        v[place] = key_value(mk);
+        ix[place] = mi;
+      } else {
+        s_over = 1;
+      }
+      atomicAdd(&s_n, 1);
+    }
+  } else if (!s_over && tid < 64) {
+    // many candidates: the pieces' lists are sorted, lane c holds the head of piece c's, the wave
+    // takes the best head (the lower piece among equals, which is the lower index) until the k-th
+    // and its ties are out
     const int c = lane;
-    int cn = c < CAND_CHUNKS ? c_n[c] : 0;
-    const bool piece_over = __builtin_amdgcn_ballot_w64(cn < 0) != 0;
-    const int base = c * CAND_CAP;
-    int head = 0, count = 0, over = piece_over ? 1 : 0;
+    const int cn = c_n[c], base = c_off[c];
+    int head = 0, count = 0, over = 0;
     uint32_t kth = 0;
-    while (!over) {
+    for (;;) {
       const bool has = head < cn;
-      uint32_t hk = has ? order_key(c_val[base + head]) : 0;
+      const uint32_t hk = has ? d_key[base + head] : 0;
       uint32_t rk = hk;
       int rc = has ? c : 0x7fffffff;
 #pragma unroll
@@ -573,13 +665,13 @@ __global__ __launch_bounds__(NT) void sample_filtered_kernel(float* __restrict__
       if (count == SURV_CAP) { over = 1; break; }
       if (count == k - 1) kth = rk;
       if (c == rc) {
-        v[count] = c_val[base + head];
-        ix[count] = c_idx[base + head];
+        v[count] = key_value(d_key[base + head]);
+        ix[count] = d_idx[base + head];
         ++head;
       }
       ++count;
     }
-    if (lane == 0) { s_n = count; s_over = over; }
+    if (lane == 0) { s_n = count; if (over) s_over = 1; }
   }
   __syncthreads();
   if (s_over) {            // too many equal values for the lists: the whole-row kernels, in place
@@ -592,16 +684,16 @@ __global__ __launch_bounds__(NT) void sample_filtered_kernel(float* __restrict__
   if (tid < n) alive[tid] = 1;
   __syncthreads();
   const float mx = n > 0 ? v[0] : -INFINITY;
+  const int r0 = lane, r1 = lane + 64;                 // wave 0: the two places of a lane
   if (top_p > 0.f && top_p < 1.f && mx > -INFINITY) {
     // as top_p_row: p_i = exp(l_i - max) / sum over finite entries, the sum in double
     __shared__ double s_tot;
-    __shared__ double ed[SURV_CAP];
-    if (tid < n) ed[tid] = v[tid] > -INFINITY ? exp((double)(v[tid] - mx)) : 0.0;
-    __syncthreads();
-    if (tid == 0) {
+    if (tid < 64) {
+      const double e0 = r0 < n && v[r0] > -INFINITY ? exp((double)(v[r0] - mx)) : 0.0;
+      const double e1 = r1 < n && v[r1] > -INFINITY ? exp((double)(v[r1] - mx)) : 0.0;
       double t = 0.0;
-      for (int i = 0; i < n; ++i) t += ed[i];
-      s_tot = t;
+      for (int i = 0; i < n; ++i) t += at_place(e0, e1, i);
+      if (lane == 0) s_tot = t;
     }
     __syncthreads();
     const float tot_f = (float)s_tot;
@@ -611,22 +703,22 @@ __global__ __launch_bounds__(NT) void sample_filtered_kernel(float* __restrict__
       int r = 0;
       for (int j = 0; j < n; ++j)
         if (pr[j] > pr[tid] || (pr[j] == pr[tid] && ix[j] < ix[tid])) ++r;
-      rank_p[tid] = r;
       order[r] = tid;
     }
     __syncthreads();
-    if (tid == 0) {
+    if (tid < 64) {
       // descending, stable: the shortest prefix whose mass exceeds p stays
+      const float p0 = r0 < n ? pr[order[r0]] : -1.f, p1 = r1 < n ? pr[order[r1]] : -1.f;
       double cum = 0.0;
       int keep = n;
       for (int r = 0; r < n; ++r) {
-        const int i = order[r];
-        if (pr[i] < 0.f) { keep = min(keep, r); break; }       // entries that are not finite stay as they are
-        cum += (double)pr[i];
+        const float p = at_place(p0, p1, r);
+        if (p < 0.f) { keep = min(keep, r); break; }           // entries that are not finite stay as they are
+        cum += (double)p;
         if (cum > (double)top_p) { keep = r + 1; break; }
       }
-      for (int r = keep; r < n; ++r)
-        if (pr[order[r]] >= 0.f) alive[order[r]] = 0;
+      if (r0 < n && r0 >= keep && p0 >= 0.f) alive[order[r0]] = 0;
+      if (r1 < n && r1 >= keep && p1 >= 0.f) alive[order[r1]] = 0;
     }
     __syncthreads();
   }
@@ -635,49 +727,36 @@ __global__ __launch_bounds__(NT) void sample_filtered_kernel(float* __restrict__
     int r = 0;
     for (int j = 0; j < n; ++j)
       if (ix[j] < ix[tid]) ++r;
-    rank_i[tid] = r;
+    order[r] = tid;
   }
   __syncthreads();
-  if (tid < n) order[rank_i[tid]] = tid;
-  __shared__ float s_mxt, s_inv;
-  __shared__ float ev[SURV_CAP];       // exp(l - max) of a survivor, 0 for one that is out
+  if (tid >= 64) return;
+  // wave 0 alone from here on: lane holds the survivors at places r0 and r1 of the index order
   const float inv_t = 1.0f / temp;
-  __syncthreads();
-  if (tid == 0) {
-    float mxt = -INFINITY;
-    for (int i = 0; i < n; ++i)
-      if (alive[i]) mxt = fmaxf(mxt, scaled(v[i], inv_t));
-    s_mxt = mxt;
+  const int i0 = r0 < n ? order[r0] : 0, i1 = r1 < n ? order[r1] : 0;
+  const bool on0 = r0 < n && alive[i0], on1 = r1 < n && alive[i1];
+  const float l0 = on0 ? scaled(v[i0], inv_t) : -INFINITY, l1 = on1 ? scaled(v[i1], inv_t) : -INFINITY;
+  float mxt = fmaxf(l0, l1);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mxt = fmaxf(mxt, __shfl_xor(mxt, o, MF_WAVE));
+  const float e0 = l0 > -INFINITY ? exp_rel(l0, mxt) : 0.f, e1 = l1 > -INFINITY ? exp_rel(l1, mxt) : 0.f;
+  double total = 0.0;
+  for (int r = 0; r < n; ++r) total += (double)at_place(e0, e1, r);
+  const float inv = (float)(1.0 / total);
+  const float q0 = e0 * inv, q1 = e1 * inv;            // the probability, as prob_of forms it
+  const int x0 = r0 < n ? ix[i0] : 0, x1 = r1 < n ? ix[i1] : 0;
+  const float rnd = forced_r ? forced_r[rowi]
+                             : uniform01((uint64_t)streams[rowi], (uint64_t)(uint32_t)steps[rowi]);
+  const double rr = fmax((double)rnd, 1e-30);
+  double cum = 0.0;
+  int pick = vocab - 1;                // fallback: the last index (src/sampler.rs:266)
+  for (int r = 0; r < n; ++r) {
+    const float p = at_place(q0, q1, r);
+    if (p <= 0.f) continue;
+    cum += (double)p;
+    if (rr <= cum) { pick = at_place(x0, x1, r); break; }
   }
-  __syncthreads();
-  if (tid < n) {
-    const float l = scaled(v[tid], inv_t);
-    ev[tid] = (alive[tid] && l > -INFINITY) ? exp_rel(l, s_mxt) : 0.f;
-  }
-  __syncthreads();
-  if (tid == 0) {
-    double total = 0.0;
-    for (int r = 0; r < n; ++r) total += (double)ev[order[r]];
-    s_inv = (float)(1.0 / total);
-  }
-  __syncthreads();
-  if (tid < n) ev[tid] = ev[tid] * s_inv;              // the probability, as prob_of forms it
-  __syncthreads();
-  if (tid == 0) {
-    const float rnd = forced_r ? forced_r[rowi]
-                               : uniform01((uint64_t)streams[rowi], (uint64_t)(uint32_t)steps[rowi]);
-    const double rr = fmax((double)rnd, 1e-30);
-    double cum = 0.0;
-    int pick = vocab - 1;                // fallback: the last index (src/sampler.rs:266)
-    for (int r = 0; r < n; ++r) {
-      const int i = order[r];
-      const float p = ev[i];
-      if (p <= 0.f) continue;
-      cum += (double)p;
-      if (rr <= cum) { pick = ix[i]; break; }
-    }
-    out[rowi] = pick;
-  }
+  if (lane == 0) out[rowi] = pick;
 }
 
 // after a decode step: feed the sampled token back, move every sequence on by one, and (when
@@ -732,20 +811,27 @@ MF_API int mf_sample(const float* logits, int ld, int rows, int vocab, float tem
 }
 
 // top-k (1 <= k <= 48), top-p (outside (0,1): off) and the temperature draw (temp >= 1e-6) in two
-// kernels that read the row once; `work` holds rows * 32 * 64 floats, as many ints, and rows * 32
-// ints.  The logits stay as they are unless a row has more equal values than the lists hold.
+// kernels that read the row once (and a small one before them that reads it for the pieces'
+// maxima); `work` holds rows * 64 * 64 floats, as many ints, and twice rows * 64 ints.  The logits stay as they are unless a row has more equal values than the lists hold.
 MF_API int mf_sample_filtered(float* logits, int ld, int rows, int vocab, int k, float top_p, float temp,
                               const long long* streams, const int* steps, const float* forced_r,
                               void* work, int* out, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0 || ld < vocab || k < 1 || k > FAST_K_MAX || !(temp >= 1e-6f) || !work ||
-      vocab > CAND_CHUNKS * 256 * CAND_EPT)
+      vocab > CAND_CHUNKS * 64 * CAND_EPT)
     return (int)hipErrorInvalidValue;
   float* cand_val = (float*)work;
   int* cand_idx = (int*)(cand_val + (size_t)rows * CAND_CHUNKS * CAND_CAP);
   int* cand_n = cand_idx + (size_t)rows * CAND_CHUNKS * CAND_CAP;
-  topk_candidates_kernel<<<dim3(CAND_CHUNKS, rows), 256, 0, stream>>>(logits, ld, vocab, k, cand_val, cand_idx,
-                                                                      cand_n);
+  uint32_t* piece_max = (uint32_t*)(cand_n + (size_t)rows * CAND_CHUNKS);
+  const dim3 grid(CAND_CHUNKS / 4, rows);
+  piece_max_kernel<<<grid, 256, 0, stream>>>(logits, ld, vocab, piece_max);
+  if (int rc0 = mf_launch_status()) return rc0;
+  const int ept = ((vocab + CAND_CHUNKS - 1) / CAND_CHUNKS + 63) / 64;     // entries per lane of a piece
+  if (ept <= 16) topk_candidates_kernel<16><<<grid, 256, 0, stream>>>(logits, ld, vocab, k, piece_max, cand_val, cand_idx, cand_n);
+  else if (ept <= 32) topk_candidates_kernel<32><<<grid, 256, 0, stream>>>(logits, ld, vocab, k, piece_max, cand_val, cand_idx, cand_n);
+  else if (ept <= 48) topk_candidates_kernel<48><<<grid, 256, 0, stream>>>(logits, ld, vocab, k, piece_max, cand_val, cand_idx, cand_n);
+  else topk_candidates_kernel<CAND_EPT><<<grid, 256, 0, stream>>>(logits, ld, vocab, k, piece_max, cand_val, cand_idx, cand_n);
   int rc = mf_launch_status();
   if (rc) return rc;
   sample_filtered_kernel<<<rows, NT, 0, stream>>>(logits, ld, vocab, k, top_p, temp, streams, steps, forced_r,

@@ -815,7 +815,7 @@ def top_p(logits: torch.Tensor, p: float) -> None:
 
 
 FILTERED_K_MAX = 48            # the largest top-k that `sample_filtered` takes
-FILTERED_VOCAB_MAX = 32 * 256 * 32
+FILTERED_VOCAB_MAX = 64 * 64 * 64
 
 
 def sample_filtered_takes(vocab: int, k: int, temp: float) -> bool:
@@ -827,7 +827,7 @@ def sample_filtered(logits: torch.Tensor, k: int, p: float, temp: float, streams
                     steps: torch.Tensor, out: torch.Tensor, forced_r: Optional[torch.Tensor] = None) -> None:
     """top-k, then top-p (off unless 0 < p < 1), then the temperature draw, as `top_k`, `top_p` and
     `sample` one after the other give it, but reading each row once: its k largest entries and their
-    ties are picked out by 32 blocks a row and the rest runs on those few.  The logits stay as they
+    ties are picked out by 64 waves a row and the rest runs on those few.  The logits stay as they
     are, except for rows with more equal values than the lists hold, which take the whole-row
     kernels in place."""
     rows, vocab = _logit_rows(logits, "sample_filtered.logits")
@@ -838,7 +838,7 @@ def sample_filtered(logits: torch.Tensor, k: int, p: float, temp: float, streams
     _need(out, "sample_filtered.out", torch.int32, (rows,))
     if forced_r is not None:
         _need(forced_r, "sample_filtered.forced_r", torch.float32, (rows,))
-    work = workspace("sample_filtered", rows * 32 * (2 * 64 + 1), logits.device)
+    work = workspace("sample_filtered", rows * 64 * (2 * 64 + 2), logits.device)
     _check(_fn("sampling", "mf_sample_filtered")(_ptr(logits), vocab, rows, vocab, int(k), float(p), float(temp),
                                                   _ptr(streams), _ptr(steps), _ptr(forced_r), _ptr(work),
                                                   _ptr(out), _stream()),
