@@ -164,6 +164,34 @@ def test_sample_filtered_is_top_k_top_p_and_the_draw(ops, rows, vocab, k, p, tem
     assert got.cpu().tolist() == want.cpu().tolist()
 
 
+def test_sample_filtered_with_many_candidates(ops):
+    """A row whose pieces' maxima bound its k-th largest entry loosely: the 40 largest sit in one
+    piece, every other piece has a dozen entries at its own maximum, which is the bound, so the
+    lists hold some 800 candidates for 40 survivors (more than find their places by counting: the
+    lists' heads are taken one by one).  A second row with 300 candidates takes the counting."""
+    vocab, k, p, temp = 152064, 40, 0.95, 0.8
+    per = (vocab + 63) // 64
+    l = logits_rows(2, vocab, 21).clamp(-1.0, 1.0)
+    for row, dozen in ((0, 12), (1, 4)):
+        l[row, 100:100 + k] = 10.0 + 0.01 * torch.arange(k)
+        for piece in range(1, 64):
+            l[row, piece * per + 7 * torch.arange(dozen)] = 5.0
+    rs = torch.tensor([0.3, 0.97], device=DEV)
+    keys = torch.zeros(2, dtype=torch.int64, device=DEV)
+    steps = torch.zeros(2, dtype=torch.int32, device=DEV)
+    chain = l.to(DEV).clone()
+    want = torch.empty(2, dtype=torch.int32, device=DEV)
+    ops.top_k(chain, k)
+    ops.top_p(chain, p)
+    ops.sample(chain, temp, keys, steps, want, rs)
+    d = l.to(DEV).clone()
+    got = torch.empty(2, dtype=torch.int32, device=DEV)
+    ops.sample_filtered(d, k, p, temp, keys, steps, got, rs)
+    assert got.cpu().tolist() == want.cpu().tolist()
+    assert all(100 <= t < 100 + k for t in got.cpu().tolist())
+    assert torch.equal(d.cpu(), l)
+
+
 def test_device_uniform_is_the_host_uniform_and_draws_follow_softmax(ops):
     rows, vocab = 4000, 3
     small = torch.tensor([0.0, 1.0, 2.0]).repeat(rows, 1).to(DEV)
