@@ -29,9 +29,20 @@ QWEN25_7B = dict(
     intermediate_size=18944, vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-6,
     max_position_embeddings=32768, tie_word_embeddings=False, use_sliding_window=False,
     initializer_range=0.02)
-# the larger shapes of the same architecture (for measurements beyond the default run)
+# other shapes of the same architecture (for measurements beyond the default run)
 SHAPES = {
     "7b": ("Qwen2.5-7B", QWEN25_7B),
+    "0.5b": ("Qwen2.5-0.5B", dict(QWEN25_7B, num_hidden_layers=24, hidden_size=896, num_attention_heads=14,
+                                  num_key_value_heads=2, intermediate_size=4864, vocab_size=151936,
+                                  tie_word_embeddings=True)),
+    "1.5b": ("Qwen2.5-1.5B", dict(QWEN25_7B, num_hidden_layers=28, hidden_size=1536, num_attention_heads=12,
+                                  num_key_value_heads=2, intermediate_size=8960, vocab_size=151936,
+                                  tie_word_embeddings=True)),
+    "3b": ("Qwen2.5-3B", dict(QWEN25_7B, num_hidden_layers=36, hidden_size=2048, num_attention_heads=16,
+                              num_key_value_heads=2, intermediate_size=11008, vocab_size=151936,
+                              tie_word_embeddings=True)),
+    "14b": ("Qwen2.5-14B", dict(QWEN25_7B, num_hidden_layers=48, hidden_size=5120, num_attention_heads=40,
+                                num_key_value_heads=8, intermediate_size=13824, rms_norm_eps=1e-5)),
     "32b": ("Qwen2.5-32B", dict(QWEN25_7B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=40,
                                 num_key_value_heads=8, intermediate_size=27648, rms_norm_eps=1e-5)),
     "72b": ("Qwen2.5-72B", dict(QWEN25_7B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
@@ -48,7 +59,7 @@ def parse():
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prompt-max", type=int, default=2048)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes (default: Qwen2.5-7B)")
+    ap.add_argument("--shape", default="7b", choices=list(SHAPES), help="layer sizes (default: Qwen2.5-7B)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip the further points (batch 1 and 64, long contexts, other prefills)")
