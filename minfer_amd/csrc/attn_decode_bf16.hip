@@ -76,40 +76,94 @@ template <int HD, bool ROPE>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16* __restrict__ q, bf16* kc, bf16* vt,
     const int* __restrict__ page_table, int pt_stride, const int* __restrict__ positions,
-    const int* __restrict__ seq_of_tok, bf16* __restrict__ out, float* __restrict__ part, int nh, int nk,
-    float scale, int window, int n_splits, RopeArgs rope) {
+    const int* __restrict__ seq_of_tok, bf16* __restrict__ out, float* __restrict__ part, int n_tok, int nh, int nk,
+    float scale, int window, int n_splits, int base_splits, RopeArgs rope) {
   constexpr int KS = (HD + 31) / 32;      // 32-wide steps over head_dim in the first product
   constexpr int CT = HD / 16;             // 16-wide column tiles of the output
   constexpr int O_LD = HD + 4;
   __shared__ float sm_o[4][16][O_LD];
   __shared__ float sm_ml[4][16][2];
 
-  const int t = blockIdx.x;
-  const int G = nh / nk;
-  const int n_gc = (G + 15) / 16;
-  const int hk = blockIdx.y / n_gc;
-  const int g0 = (blockIdx.y % n_gc) * 16;
-  const int gcount = min(16, G - g0);
-  const int h0 = hk * G + g0;
-  const int split = blockIdx.z;
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, q4 = lane >> 4;
+  const int G = nh / nk;
+  const int n_gc = (G + 15) / 16;
+  // Which token, group of heads and split this block has, and how many splits the token's keys go
+  // over (`active`, at most its n_splits places in `part`).
+  int t, hg, split, active, p;
+  if (base_splits == 0) {
+    // Every token has n_splits splits.  Blocks are numbered with the split running fastest, then
+    // the group of heads, then the token: consecutive blocks go to consecutive dies, so a
+    // sequence's splits are dealt over all of them (with the token running fastest and 8 sequences
+    // on 8 dies every die had one sequence to itself).
+    split = blockIdx.x % n_splits;
+    hg = (blockIdx.x / n_splits) % (nk * n_gc);
+    t = blockIdx.x / (n_splits * nk * n_gc);
+    active = n_splits;
+    p = positions[t];
+  } else {
+    // The step's tokens (at most 64) share n_tok * base_splits splits, as many blocks per group of
+    // heads as without sharing (one per CU is what the plan aims at; a block more on some CUs
+    // would double their time): one split each, and the rest in proportion to their keys (token
+    // i's part ends where the keys up to and with its own end on that scale, rounded down), so
+    // that blocks have about equal work whatever the lengths: a step is as long as its longest
+    // block.  Blocks are numbered through the tokens' splits one after the other; every wave works
+    // the shares out for itself, lane i for token i, in integers, so all blocks of a launch agree.
+    const int nb = n_tok * base_splits;
+    const int b = blockIdx.x % nb;
+    hg = blockIdx.x / nb;
+    const int p_i = lane < n_tok ? positions[lane] : 0;
+    const int len_i = lane < n_tok ? (window > 0 ? min(p_i + 1, window) : p_i + 1) : 0;
+    long long keys = len_i;                // of the tokens up to and with lane's
+    for (int o = 1; o < n_tok; o <<= 1) {
+      const long long v = __shfl_up(keys, o, MF_WAVE);
+      if (lane >= o) keys += v;
+    }
+    const long long total = __shfl(keys, n_tok - 1, MF_WAVE);
+    const int end_i = (int)(keys * (nb - n_tok) / total);
+    const int begin_i = __shfl_up(end_i, 1, MF_WAVE);
+    const int s_i = lane < n_tok ? min(n_splits, 1 + end_i - (lane ? begin_i : 0)) : 0;
+    int behind = s_i;                      // splits of the tokens up to and with lane's
+    for (int o = 1; o < n_tok; o <<= 1) {
+      const int v = __shfl_up(behind, o, MF_WAVE);
+      if (lane >= o) behind += v;
+    }
+    const unsigned long long mine = __ballot(b >= behind - s_i && b < behind);
+    if (mine == 0) return;                 // a block beyond the shares (a token whose share its places cut)
+    t = __ffsll((long long)mine) - 1;
+    split = __builtin_amdgcn_readfirstlane(b - (__shfl(behind, t, MF_WAVE) - __shfl(s_i, t, MF_WAVE)));
+    active = __builtin_amdgcn_readfirstlane(__shfl(s_i, t, MF_WAVE));
+    p = __builtin_amdgcn_readfirstlane(__shfl(p_i, t, MF_WAVE));
+  }
+  const int hk = hg / n_gc;
+  const int g0 = (hg % n_gc) * 16;
+  const int gcount = min(16, G - g0);
+  const int h0 = hk * G + g0;
 
-  const int p = positions[t];
   const int* pt = page_table + (size_t)seq_of_tok[t] * pt_stride;
   const int lo = window > 0 ? max(0, p - window + 1) : 0;
-  // split length: this token's keys over the splits, in whole block rounds of 4 steps
-  const int per = (p + 1 - lo + n_splits - 1) / n_splits;
+  if (split == 0 && active < n_splits) {
+    // the places this token leaves unused say "nothing here" (maximum -inf, sum 0; the merge reads
+    // no further)
+    for (int i = threadIdx.x; i < (n_splits - active) * gcount; i += 256) {
+      float* o = part + (((size_t)t * nh + h0 + i % gcount) * n_splits + active + i / gcount) * (HD + 2);
+      o[HD] = -INFINITY;
+      o[HD + 1] = 0.f;
+    }
+  }
+  // split length: this token's keys over its splits, in whole block rounds of 4 steps
+  const int per = (p + 1 - lo + active - 1) / active;
   const int split_len = (per + 4 * STEP - 1) / (4 * STEP) * (4 * STEP);
   const int j_begin = lo + split * split_len;
   const int j_end = min(p + 1, j_begin + split_len);
   if (j_begin >= j_end) {
     // A split past the token's keys (a short sequence under a split count made for long ones):
-    // its partials say "nothing here" (zeros, maximum -inf, sum 0) and the block is done.
-    for (int i = threadIdx.x; i < gcount * (HD + 2); i += 256) {
-      const int g = i / (HD + 2), d = i % (HD + 2);
-      part[(((size_t)t * nh + h0 + g) * n_splits + split) * (HD + 2) + d] = d == HD ? -INFINITY : 0.f;
+    // the same mark, and the block is done.
+    for (int g = threadIdx.x; g < gcount; g += 256) {
+      float* o = part + (((size_t)t * nh + h0 + g) * n_splits + split) * (HD + 2);
+      o[HD] = -INFINITY;
+      o[HD + 1] = 0.f;
     }
     return;
   }
@@ -142,7 +196,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     if (own_split) {
       const int tid = threadIdx.x;
       const float* row = rope.qkv + (size_t)t * (nh + 2 * nk) * HD;
-      const bool store = blockIdx.y % n_gc == 0;           // one block per kv head fills the cache
+      const bool store = g0 == 0;                          // one block per kv head fills the cache
       const int page = pt[p / MF_PAGE];
       if (tid < KS * 4) {
         bf16x8 k8 = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
@@ -340,15 +394,19 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 template <int HD>
 int launch(const bf16* q, bf16* kc, bf16* vt, const int* page_table, int pt_stride, const int* positions,
            const int* seq_of_tok, bf16* out, float* part, int n_tok, int nh, int nk, float scale, int window,
-           int n_splits, const RopeArgs* rope, hipStream_t stream) {
+           int n_splits, int base_splits, const RopeArgs* rope, hipStream_t stream) {
   const int G = nh / nk;
-  dim3 grid(n_tok, nk * ((G + 15) / 16), n_splits);
+  const long blocks = (long)n_tok * nk * ((G + 15) / 16) * (base_splits ? base_splits : n_splits);
+  if (blocks > 0x7fffffffL) return (int)hipErrorInvalidValue;
+  dim3 grid((unsigned)blocks);
   if (rope)
     attn_decode_kernel<HD, true><<<grid, 256, 0, stream>>>(q, kc, vt, page_table, pt_stride, positions, seq_of_tok,
-                                                           out, part, nh, nk, scale, window, n_splits, *rope);
+                                                           out, part, n_tok, nh, nk, scale, window, n_splits,
+                                                           base_splits, *rope);
   else
     attn_decode_kernel<HD, false><<<grid, 256, 0, stream>>>(q, kc, vt, page_table, pt_stride, positions,
-                                                            seq_of_tok, out, part, nh, nk, scale, window, n_splits,
+                                                            seq_of_tok, out, part, n_tok, nh, nk, scale, window,
+                                                            n_splits, base_splits,
                                                             RopeArgs{nullptr, nullptr, nullptr, 0});
   int rc = mf_launch_status();
   if (rc == 0 && n_splits > 1) {
@@ -360,15 +418,17 @@ int launch(const bf16* q, bf16* kc, bf16* vt, const int* page_table, int pt_stri
 
 int dispatch(const void* q, void* kc, void* vt, const int* page_table, int pt_stride, const int* positions,
              const int* seq_of_tok, void* out, float* part, int n_tok, int nh, int nk, int hd, float scale,
-             int window, int n_splits, const RopeArgs* rope, hipStream_t stream) {
+             int window, int n_splits, int base_splits, const RopeArgs* rope, hipStream_t stream) {
   if (n_tok <= 0) return 0;
+  if (base_splits == n_splits) base_splits = 0;       // nothing to share out
   if (hd % 16 != 0 || hd < 16 || hd > 256 || nk <= 0 || nh % nk != 0 || n_splits < 1 || n_splits > 64 ||
-      (n_splits > 1 && part == nullptr))
+      (n_splits > 1 && part == nullptr) || base_splits < 0 || base_splits > n_splits || (base_splits && n_tok > 64))
     return (int)hipErrorInvalidValue;
 #define MF_CASE(E)                                                                                          \
   case E:                                                                                                   \
     return launch<16 * E>((const bf16*)q, (bf16*)kc, (bf16*)vt, page_table, pt_stride, positions,           \
-                          seq_of_tok, (bf16*)out, part, n_tok, nh, nk, scale, window, n_splits, rope, stream);
+                          seq_of_tok, (bf16*)out, part, n_tok, nh, nk, scale, window, n_splits,    \
+                          base_splits, rope, stream);
   switch (hd / 16) {
     MF_CASE(1) MF_CASE(2) MF_CASE(3) MF_CASE(4) MF_CASE(5) MF_CASE(6) MF_CASE(7) MF_CASE(8)
     MF_CASE(9) MF_CASE(10) MF_CASE(11) MF_CASE(12) MF_CASE(13) MF_CASE(14) MF_CASE(15) MF_CASE(16)
@@ -381,12 +441,17 @@ int dispatch(const void* q, void* kc, void* vt, const int* page_table, int pt_st
 
 // q, out: [n_tok][nh][hd]; kc: [pages][nk][64][hd]; vt: [pages][nk][2][hd][32] (V transposed inside
 // a page, in two halves of 32 keys); part: n_tok * nh * n_splits * (hd + 2) floats when n_splits > 1 (at most 64 splits).
+// base_splits: 0 or n_splits: every token's keys go over n_splits splits; a number below n_splits
+// (and at most 64 tokens): the step's tokens share n_tok * base_splits splits, one each and the
+// rest in proportion to their keys, none taking more than n_splits (the places it leaves unused
+// are marked empty), so that a long sequence among short ones does not make the step as long as
+// its own n_splits-th.
 MF_API int mf_attn_decode_bf16(const void* q, const void* kc, const void* vt, const int* page_table,
                                int pt_stride, const int* positions, const int* seq_of_tok, void* out,
                                float* part, int n_tok, int nh, int nk, int hd, float scale, int window,
-                               int n_splits, hipStream_t stream) {
+                               int n_splits, int base_splits, hipStream_t stream) {
   return dispatch(q, const_cast<void*>(kc), const_cast<void*>(vt), page_table, pt_stride, positions, seq_of_tok,
-                  out, part, n_tok, nh, nk, hd, scale, window, n_splits, nullptr, stream);
+                  out, part, n_tok, nh, nk, hd, scale, window, n_splits, base_splits, nullptr, stream);
 }
 
 // The same with the rotation and the cache write of the step's own q|k|v folded in: qkv is the
@@ -397,11 +462,11 @@ MF_API int mf_attn_decode_bf16(const void* q, const void* kc, const void* vt, co
 MF_API int mf_attn_decode_rope_bf16(const float* qkv, const float* cs, const float* sn, void* kc, void* vt,
                                     const int* page_table, int pt_stride, const int* positions,
                                     const int* seq_of_tok, void* out, float* part, int n_tok, int nh, int nk,
-                                    int hd, float scale, int window, int n_splits, int write_kv,
+                                    int hd, float scale, int window, int n_splits, int base_splits, int write_kv,
                                     hipStream_t stream) {
   const RopeArgs rope{qkv, cs, sn, write_kv};
   return dispatch(nullptr, kc, vt, page_table, pt_stride, positions, seq_of_tok, out, part, n_tok, nh, nk, hd,
-                  scale, window, n_splits, &rope, stream);
+                  scale, window, n_splits, base_splits, &rope, stream);
 }
 
 // ------------------------------------------------------------------ the entry point that allocates nothing
@@ -450,5 +515,5 @@ MF_API int mf_attn_decode_bf16_noalloc(const void* q, const void* kc, const void
     if (!part) return rc;
   }
   return dispatch(q, const_cast<void*>(kc), const_cast<void*>(vt), page_table, pt_stride, positions, seq_of_tok,
-                  out, part, n_tok, nh, nk, hd, scale, window, n_splits, nullptr, stream);
+                  out, part, n_tok, nh, nk, hd, scale, window, n_splits, 0, nullptr, stream);
 }

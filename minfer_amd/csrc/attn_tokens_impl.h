@@ -242,15 +242,24 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
   const float mm = wave_max(ms);
   const float wv = (ms == -INFINITY) ? 0.f : exp_for<T>(ms - mm);
   wgt[lane] = wv;
-  // fixed order: lane 0 adds the weighted sums one after another
+  // the splits behind the last one with keys (places a token does not use) are not read at all
+  const unsigned long long with_keys = __ballot(ms != -INFINITY);
+  const int n_used = with_keys ? 64 - __clzll((long long)with_keys) : 0;
+  // fixed order: every lane adds the weighted sums one after another
   __syncthreads();
   float L = 0.f;
-  for (int s = 0; s < n_splits; ++s) L += __shfl(ls, s, MF_WAVE) * wgt[s];
+  for (int s = 0; s < n_used; ++s) L += __shfl(ls, s, MF_WAVE) * wgt[s];
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   for (int d = lane; d < hd; d += 64) {
     float a = 0.f;
 #pragma unroll 8
-    for (int s = 0; s < n_splits; ++s) a += base[(size_t)s * (hd + 2) + d] * wgt[s];
+    for (int s = 0; s < n_used; ++s) {
+      // weight 0: a split without keys, whose sums nobody wrote.  Its load goes to the first split's
+      // line instead (no branch, so the loads of a round are in flight together) and counts as 0.
+      const float w = wgt[s];
+      const float v = base[(w != 0.f ? (size_t)s * (hd + 2) : 0) + d];
+      a += (w != 0.f ? v : 0.f) * w;
+    }
     out[th * hd + d] = from_f32<T>(a * inv);
   }
 }

@@ -26,7 +26,8 @@
 
 extern "C" {
 
-// Arguments as mf_attn_decode_bf16 without `part`: q, out [n_tok][nh][hd] bfloat16; kc
+// Arguments as mf_attn_decode_bf16 without `part` and `base_splits` (every token's keys go over
+// all n_splits splits): q, out [n_tok][nh][hd] bfloat16; kc
 // [pages][nk][64][hd]; vt [pages][nk][2][hd][32]; page_table [sequences][pt_stride] int32;
 // positions, seq_of_tok [n_tok] int32; 1 <= n_splits <= 64.  Returns 0, a hipError_t, or
 // MF_NOALLOC_TOO_LARGE.

@@ -68,9 +68,9 @@ _PROTOTYPES = {
     },
     "attn_decode_bf16": {
         "mf_attn_decode_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
-                                c_float, c_int, c_int, _P],
+                                c_float, c_int, c_int, c_int, _P],
         "mf_attn_decode_rope_bf16": [_P, _P, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int,
-                                     c_int, c_float, c_int, c_int, c_int, _P],
+                                     c_int, c_float, c_int, c_int, c_int, c_int, _P],
     },
     "attn_prefill_bf16": {
         "mf_attn_prefill_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, c_int,
@@ -634,15 +634,26 @@ def _need_caches(what: str, kcache: torch.Tensor, vcache: torch.Tensor, dtype, n
                           f"{[kcache.shape[0]] + list(want)}")
 
 
-def decode_split_plan(n_tok: int, n_kv_heads: int, group: int, max_len: int, target_blocks: int = 256) -> int:
-    """Key splits of the bfloat16 decode attention: about one block per CU, at least 256 keys of
-    the longest possible sequence per split, at most 32 (the merge reads every split).  The kernel
-    divides each token's own length by this number in rounds of 128 keys; a split left without
-    keys writes an empty partial and ends."""
+# Sequences that can be this long share their step's key splits by length: working the shares out
+# costs a block about a microsecond, which shorter ones do not gain back.
+SHARED_SPLITS_FROM = 8192
+
+
+def decode_split_plan(n_tok: int, n_kv_heads: int, group: int, max_len: int,
+                      target_blocks: int = 256) -> Tuple[int, int]:
+    """(places, splits) of the bfloat16 decode attention's key splits.  `splits`: about one block
+    per CU, at least 256 keys of the longest possible sequence per split, at most 32.  A step of
+    one token, of more than 64, of sequences that cannot be long, or without splits, gives every
+    token that many (`places` = `splits`); otherwise the
+    step's tokens share tokens x splits between them in proportion to their keys, a token taking
+    at most `places` = 4 x splits (at most 32), so that a long sequence among short ones is cut
+    finer and the blocks have about equal work.  The kernel divides a token's keys in rounds of
+    128; a place without keys is marked empty and the merge passes it over."""
     blocks = n_tok * n_kv_heads * ((group + 15) // 16)
-    if tuning.ATTN_SPLITS:
-        return tuning.ATTN_SPLITS
-    return max(1, min(target_blocks // max(1, blocks), (max_len + 255) // 256, 32))
+    splits = tuning.ATTN_SPLITS or max(1, min(target_blocks // max(1, blocks), (max_len + 255) // 256, 32))
+    if n_tok == 1 or n_tok > 64 or splits == 1 or max_len < SHARED_SPLITS_FROM or tuning.ATTN_EQUAL_SPLITS:
+        return splits, splits
+    return max(splits, min(4 * splits, 32)), splits
 
 
 def attn_tokens(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
@@ -665,12 +676,12 @@ def attn_tokens(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pag
     if max_len > page_table.shape[1] * PAGE:
         raise KernelError(f"attention: max_len {max_len} exceeds the page table ({page_table.shape[1]} pages)")
     if q.dtype == torch.bfloat16:
-        n_splits = decode_split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, max_len)
+        n_splits, base = decode_split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, max_len)
         part = workspace("attn", n_tok * n_heads * n_splits * (head_dim + 2), q.device) if n_splits > 1 else None
         _check(_fn("attn_decode_bf16", "mf_attn_decode_bf16")(
             _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(positions),
             _ptr(seq_of_tok), _ptr(out), _ptr(part), n_tok, n_heads, n_kv_heads, head_dim, float(scale),
-            int(window or 0), n_splits, _stream()), "attn_decode_bf16")
+            int(window or 0), n_splits, base, _stream()), "attn_decode_bf16")
         return
     n_splits, split_len = split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, head_dim, max_len)
     part = workspace("attn", n_tok * n_heads * n_splits * (head_dim + 2), q.device) if n_splits > 1 else None
@@ -705,12 +716,12 @@ def attn_decode_rope(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, kc
     if max_len > page_table.shape[1] * PAGE or max_len > cos.shape[0]:
         raise KernelError(f"attention: max_len {max_len} exceeds the page table ({page_table.shape[1]} pages) "
                           f"or the rotation table ({cos.shape[0]} positions)")
-    n_splits = decode_split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, max_len)
+    n_splits, base = decode_split_plan(n_tok, n_kv_heads, n_heads // n_kv_heads, max_len)
     part = workspace("attn", n_tok * n_heads * n_splits * (head_dim + 2), qkv.device) if n_splits > 1 else None
     _check(_fn("attn_decode_bf16", "mf_attn_decode_rope_bf16")(
         _ptr(qkv), _ptr(cos), _ptr(sin), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1],
         _ptr(positions), _ptr(seq_of_tok), _ptr(out), _ptr(part), n_tok, n_heads, n_kv_heads, head_dim,
-        float(scale), int(window or 0), n_splits, 1 if write_kv else 0, _stream()), "attn_decode_rope_bf16")
+        float(scale), int(window or 0), n_splits, base, 1 if write_kv else 0, _stream()), "attn_decode_rope_bf16")
 
 
 def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,

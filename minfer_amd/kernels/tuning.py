@@ -14,6 +14,8 @@ src/cuda.rs:53-70,378-395 and src/main.rs:552-609 of yusiwen/minfer):
 Kernel choice, for measurements (each overrides what `ops` would pick by shape):
 
 * MF_ATTN_SPLITS=n      key splits of the bfloat16 decode attention
+* MF_ATTN_EQUAL_SPLITS=1 every token of a decode step gets the same number of key splits, whatever
+                        the lengths (default: shares in proportion to the keys)
 * MF_SKINNY_TARGET=n    blocks the K-split decode product aims at (default: one per CU)
 * MF_NO_SHARED_PAGES=1  a block of queries of the prompt attention keeps all its pages to itself
 * MF_NO_DECODE_COPIES=1 a model keeps no second, tiled copy of its matrices for the steps of few tokens
@@ -39,6 +41,7 @@ def _int(name: str) -> int:
 DEBUG_SYNC = _flag("MF_DEBUG_SYNC")
 TIMING = _flag("MF_TIMING")
 ATTN_SPLITS = _int("MF_ATTN_SPLITS")
+ATTN_EQUAL_SPLITS = _flag("MF_ATTN_EQUAL_SPLITS")
 SKINNY_TARGET = _int("MF_SKINNY_TARGET")
 NO_FOLD = _flag("MF_NO_FOLD")
 NO_SHARED_PAGES = _flag("MF_NO_SHARED_PAGES")

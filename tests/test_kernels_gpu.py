@@ -332,7 +332,10 @@ def test_attn_decode_rope(ops, nh, nk, hd, window, write_kv):
     """Rotation + cache write + attention of a decode step in one kernel against the two-step
     plain path.  The row of the token's own position is poisoned beforehand when the kernel
     is to write it: it must take k and v from the product's output, not from the cache."""
-    lengths = [1, 2, 31, 32, 33, 64, 65, 129, 500, 1000]
+    decode_rope_case(ops, nh, nk, hd, window, write_kv, [1, 2, 31, 32, 33, 64, 65, 129, 500, 1000])
+
+
+def decode_rope_case(ops, nh, nk, hd, window, write_kv, lengths):
     rng = np.random.default_rng(31)
     n_cols = max((l + 63) // 64 for l in lengths)
     n_pages = sum((l + 63) // 64 for l in lengths) + 3
@@ -351,15 +354,16 @@ def test_attn_decode_rope(ops, nh, nk, hd, window, write_kv):
     pos = torch.tensor([l - 1 for l in lengths], dtype=torch.int32)
     seq = torch.arange(len(lengths), dtype=torch.int32)
     qkv = rnd((len(lengths), (nh + 2 * nk) * hd), seed=33)
-    cs, sn = plain_ops.rope_table(1024, hd // 2, 1e4, 1.0, "cpu")
+    longest = max(lengths)
+    cs, sn = plain_ops.rope_table(longest + 24, hd // 2, 1e4, 1.0, "cpu")
     scale = 1.0 / math.sqrt(hd)
     kr, vr = kc.clone(), vc.clone()
     ref = torch.empty(len(lengths), nh * hd, dtype=torch.float64)
-    plain_ops.attn_decode_rope(qkv, cs, sn, kr, vr, table, pos, seq, ref, nh, nk, hd, scale, window, 1000, write_kv)
+    plain_ops.attn_decode_rope(qkv, cs, sn, kr, vr, table, pos, seq, ref, nh, nk, hd, scale, window, longest, write_kv)
     kd, vd = kc.to(DEV), vc.to(DEV)
     out = torch.empty(len(lengths), nh * hd, dtype=torch.bfloat16, device=DEV)
     ops.attn_decode_rope(qkv.to(DEV), cs.to(DEV), sn.to(DEV), kd, vd, table.to(DEV), pos.to(DEV), seq.to(DEV),
-                         out, nh, nk, hd, scale, window, 1000, write_kv)
+                         out, nh, nk, hd, scale, window, longest, write_kv)
     close(out, ref, 1.5e-2, 1.5e-2)
     # the cache afterwards: the own rows written (or nothing touched), everything else as before
     same = lambda a, b: torch.equal(torch.nan_to_num(a.float(), nan=7e7), torch.nan_to_num(b.float(), nan=7e7))
@@ -371,6 +375,67 @@ def test_attn_decode_rope(ops, nh, nk, hd, window, write_kv):
             assert not torch.isnan(kd[page, :, off].float()).any() and not torch.isnan(vd[page, :, off // 32, :, off % 32].float()).any()
     else:
         assert same(kd.cpu(), kc) and same(vd.cpu(), vc)
+
+
+# Sequences of very unequal lengths, the longest past the length from which a step's tokens share
+# its key splits in proportion to their keys (`ops.SHARED_SPLITS_FROM`).
+UNEQUAL = [9000, 70, 1, 2300, 64, 129, 700, 3000]
+
+
+@pytest.mark.parametrize("nh,nk,hd,window", [(8, 2, 64, 0), (28, 4, 128, 0), (6, 1, 48, 300), (4, 2, 16, 5000)])
+def test_attn_tokens_splits_shared_by_length(ops, monkeypatch, nh, nk, hd, window):
+    from minfer_amd.kernels import tuning
+    places, splits = ops.decode_split_plan(3 * len(UNEQUAL), nk, nh // nk, max(UNEQUAL))
+    assert places > splits > 1, "this case is meant to share the splits out"
+    q, kc, vc, table, pos, seq = build_attention_case(nh, nk, hd, UNEQUAL, torch.bfloat16, 41)
+    scale = 1.0 / math.sqrt(hd)
+    ref = torch.empty(q.shape, dtype=torch.float64)
+    plain_ops.attn_tokens(q, kc, vc, table, pos, seq, ref, nh, nk, hd, scale, window, max(UNEQUAL))
+    dq, dk, dv, dt, dp, ds = (t.to(DEV) for t in (q, kc, vc, table, pos, seq))
+    shared = torch.empty(q.shape, dtype=torch.bfloat16, device=DEV)
+    ops.attn_tokens(dq, dk, dv, dt, dp, ds, shared, nh, nk, hd, scale, window, max(UNEQUAL))
+    close(shared, ref, 1.5e-2, 1.5e-2)
+    again = torch.full(q.shape, float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.attn_tokens(dq, dk, dv, dt, dp, ds, again, nh, nk, hd, scale, window, max(UNEQUAL))
+    assert torch.equal(again, shared), "two runs differ"
+    # every token with the same number of splits: the same values up to the rounding of the sums
+    monkeypatch.setattr(tuning, "ATTN_EQUAL_SPLITS", True)
+    assert ops.decode_split_plan(3 * len(UNEQUAL), nk, nh // nk, max(UNEQUAL)) == (splits, splits)
+    equal = torch.empty(q.shape, dtype=torch.bfloat16, device=DEV)
+    ops.attn_tokens(dq, dk, dv, dt, dp, ds, equal, nh, nk, hd, scale, window, max(UNEQUAL))
+    close(equal, ref, 1.5e-2, 1.5e-2)
+    close(shared, equal.double().cpu(), 1.5e-2, 1.5e-2)
+
+
+def test_attn_tokens_shared_splits_lose_no_key(ops):
+    """One key of the long sequence scaled so that its score stands out, at every place in turn where
+    a split could begin or end wrongly: the output is that key's value row."""
+    nh, nk, hd = 8, 8, 16
+    lengths = [9000, 40, 1500, 300]
+    places, splits = ops.decode_split_plan(len(lengths), nk, nh // nk, max(lengths))
+    assert places > splits > 1, "this case is meant to share the splits out"
+    q, kc, vc, table, _, _ = build_attention_case(nh, nk, hd, lengths, torch.bfloat16, 43)
+    pos = torch.tensor([l - 1 for l in lengths], dtype=torch.int32)
+    seq = torch.arange(len(lengths), dtype=torch.int32)
+    q = q[:len(lengths)].clone()
+    v_rows = vc.float()                      # [pages][nk][2][hd][32]
+    out = torch.empty(len(lengths), nh * hd, dtype=torch.bfloat16, device=DEV)
+    dv, dt, dp, ds = (t.to(DEV) for t in (vc, table, pos, seq))
+    for far in (0, 127, 128, 1023, 1024, 4095, 4607, 4608, 7000, 8191, 8192, 8959, 8960, 8998, 8999):
+        k = kc.clone()
+        page, off = int(table[0, far // 64]), far % 64
+        k[page, 0, off] = (q[0].view(nh, hd)[0].float() * 40.0).to(k.dtype)
+        ops.attn_tokens(q.to(DEV), k.to(DEV), dv, dt, dp, ds, out, nh, nk, hd, 1.0, 0, max(lengths))
+        want = v_rows[page, 0, off // 32, :, off % 32]
+        assert torch.allclose(out[0].float().cpu().view(nh, hd)[0], want, atol=2e-2), far
+
+
+@pytest.mark.parametrize("write_kv", [True, False])
+@pytest.mark.parametrize("nh,nk,hd,window", [(8, 2, 64, 0), (28, 4, 128, 0), (6, 3, 48, 300)])
+def test_attn_decode_rope_splits_shared_by_length(ops, nh, nk, hd, window, write_kv):
+    assert ops.decode_split_plan(len(UNEQUAL), nk, nh // nk, max(UNEQUAL))[0] > \
+        ops.decode_split_plan(len(UNEQUAL), nk, nh // nk, max(UNEQUAL))[1]
+    decode_rope_case(ops, nh, nk, hd, window, write_kv, UNEQUAL)
 
 
 def test_attention_one_key_gives_v_and_far_key_is_found(ops):

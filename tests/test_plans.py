@@ -70,10 +70,13 @@ def test_split_plan_of_the_32_bit_attention():
 
 def test_decode_split_plan_bounds():
     for n_tok, nk, group, max_len in itertools.product((1, 8, 64, 300), (1, 2, 4), (1, 5, 7, 17), (1, 64, 4096, 32768)):
-        n = ops.decode_split_plan(n_tok, nk, group, max_len)
-        assert 1 <= n <= 32
+        places, n = ops.decode_split_plan(n_tok, nk, group, max_len)
+        assert 1 <= n <= places <= 32
         assert n == 1 or n * 256 <= max_len + 255
-    assert ops.decode_split_plan(1, 4, 7, 32768) == 32 and ops.decode_split_plan(64, 4, 7, 32768) == 1
+        assert places == n or (1 < n_tok <= 64 and n > 1 and max_len >= 8192 and places == min(4 * n, 32))
+    assert ops.decode_split_plan(1, 4, 7, 32768) == (32, 32) and ops.decode_split_plan(64, 4, 7, 32768) == (1, 1)
+    assert ops.decode_split_plan(8, 4, 7, 32768) == (32, 8)          # shares in proportion to the keys
+    assert ops.decode_split_plan(8, 4, 7, 4096) == (8, 8)
 
 
 def test_plan_linear_names_the_kernels_of_the_model_shapes():

@@ -164,7 +164,7 @@ def test_long_context_through_the_captured_decode_step(needle, dtype):
     folder, tokens, ref = needle
     eng = Engine(load_model(folder, dtype=dtype), max_tokens=64 * 40, max_seqs=2, poison_cache=True)
     if dtype == "bfloat16":
-        assert ops.decode_split_plan(1, 4, 7, 2304) >= 8, "the decode attention splits the keys here"
+        assert ops.decode_split_plan(1, 4, 7, 2304)[1] >= 8, "the decode attention splits the keys here"
     slot = eng.new_sequence()
     head = CONTEXT - TAIL
     eng.step([slot], [tokens[:head]], [[]])

@@ -20,7 +20,7 @@ def library():
     lib = build.load("attn_decode_bf16")
     P = c_void_p
     lib.mf_attn_decode_bf16.argtypes = [P, P, P, P, c_int, P, P, P, P, c_int, c_int, c_int, c_int, c_float, c_int,
-                                        c_int, P]
+                                        c_int, c_int, P]
     lib.mf_attn_decode_bf16.restype = c_int
     lib.mf_attn_decode_bf16_noalloc.argtypes = [P, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_float,
                                                 c_int, c_int, P]
@@ -58,7 +58,7 @@ def run_both(lib, tensors, nh, nk, hd, n_splits, scale=0.11):
     got = torch.full_like(want, float("nan"))
     part = torch.empty(max(1, n_tok * nh * n_splits * (hd + 2)), dtype=torch.float32, device=DEV)
     rc = lib.mf_attn_decode_bf16(p(q), p(kc), p(vt), p(table), table.shape[1], p(pos), p(seq), p(want), p(part),
-                                 n_tok, nh, nk, hd, scale, 0, n_splits, stream)
+                                 n_tok, nh, nk, hd, scale, 0, n_splits, 0, stream)
     assert rc == 0
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
