@@ -410,7 +410,7 @@ int launch(const bf16* q, bf16* kc, bf16* vt, const int* page_table, int pt_stri
                                                             RopeArgs{nullptr, nullptr, nullptr, 0});
   int rc = mf_launch_status();
   if (rc == 0 && n_splits > 1) {
-    attn_tokens::attn_combine_kernel<bf16><<<n_tok * nh, 64, 0, stream>>>(part, out, HD, n_splits);
+    attn_tokens::attn_combine_kernel<bf16><<<n_tok * nh, 64 * ((HD + 63) / 64), 0, stream>>>(part, out, HD, n_splits);
     rc = mf_launch_status();
   }
   return rc;

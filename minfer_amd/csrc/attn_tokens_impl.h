@@ -229,39 +229,42 @@ __global__ __launch_bounds__(256) void attn_tokens_kernel(
 }
 
 // out[t][h][:] = sum_s acc_s exp(m_s - M) / sum_s l_s exp(m_s - M); at most 64 splits.
-// One wave per (token, head): lane s weighs split s, then the lanes share the head's elements.
+// One block per (token, head), a thread per element of the head (64 ceil(hd / 64) threads): in
+// every wave lane s weighs split s, for itself, so the waves need nothing from each other; then a
+// thread adds its element's weighted sums one after another, in the order of the splits.
 template <typename T>
-__global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restrict__ part,
-                                                          T* __restrict__ out, int hd, int n_splits) {
-  __shared__ float wgt[64];
+__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ part,
+                                                           T* __restrict__ out, int hd, int n_splits) {
   const size_t th = blockIdx.x;   // t * nh + h
   const float* base = part + th * n_splits * (hd + 2);
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63, d = threadIdx.x;
   const float ms = lane < n_splits ? base[(size_t)lane * (hd + 2) + hd] : -INFINITY;
   const float ls = lane < n_splits ? base[(size_t)lane * (hd + 2) + hd + 1] : 0.f;
   const float mm = wave_max(ms);
   const float wv = (ms == -INFINITY) ? 0.f : exp_for<T>(ms - mm);
-  wgt[lane] = wv;
   // the splits behind the last one with keys (places a token does not use) are not read at all
   const unsigned long long with_keys = __ballot(ms != -INFINITY);
   const int n_used = with_keys ? 64 - __clzll((long long)with_keys) : 0;
-  // fixed order: every lane adds the weighted sums one after another
-  __syncthreads();
+  auto of_split = [](float x, int s) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), s)); };
   float L = 0.f;
-  for (int s = 0; s < n_used; ++s) L += __shfl(ls, s, MF_WAVE) * wgt[s];
+  for (int s = 0; s < n_used; ++s) L += of_split(ls, s) * of_split(wv, s);
   const float inv = L > 0.f ? 1.0f / L : 0.f;
-  for (int d = lane; d < hd; d += 64) {
-    float a = 0.f;
-#pragma unroll 8
-    for (int s = 0; s < n_used; ++s) {
-      // weight 0: a split without keys, whose sums nobody wrote.  Its load goes to the first split's
-      // line instead (no branch, so the loads of a round are in flight together) and counts as 0.
-      const float w = wgt[s];
-      const float v = base[(w != 0.f ? (size_t)s * (hd + 2) : 0) + d];
-      a += (w != 0.f ? v : 0.f) * w;
+  if (d >= hd) return;
+  float a = 0.f;
+  // Eight splits a round, their loads in flight together (a round that is not full would otherwise
+  // run split by split, a trip to memory each).  Weight 0: a split without keys, whose sums nobody
+  // wrote, or one behind the last; its load goes to the first split's line instead and counts as 0.
+  for (int s0 = 0; s0 < n_used; s0 += 8) {
+    float w[8], v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      w[j] = of_split(wv, s0 + j);
+      v[j] = base[(w[j] != 0.f ? (size_t)(s0 + j) * (hd + 2) : 0) + d];
     }
-    out[th * hd + d] = from_f32<T>(a * inv);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) a += (w[j] != 0.f ? v[j] : 0.f) * w[j];
   }
+  out[th * hd + d] = from_f32<T>(a * inv);
 }
 
 template <typename T, int EPL>
@@ -276,7 +279,7 @@ int launch_one(const T* q, const T* kc, const T* vc, const int* page_table, int 
                                                        n_splits, split_len);
   int rc = mf_launch_status();
   if (rc == 0 && n_splits > 1) {
-    attn_combine_kernel<T><<<n_tok * nh, 64, 0, stream>>>(part, out, 16 * EPL, n_splits);
+    attn_combine_kernel<T><<<n_tok * nh, 64 * ((16 * EPL + 63) / 64), 0, stream>>>(part, out, 16 * EPL, n_splits);
     rc = mf_launch_status();
   }
   return rc;
