@@ -58,6 +58,47 @@ def test_greedy_and_sampled_generation_match_plain(folders, name):
     assert not lb.engine.cache.live_slots()
 
 
+def test_captured_step_with_room_for_long_sequences_shares_the_key_splits(tmp_path):
+    """A session made for 8,320 positions: the captured decode step's attention deals its key splits
+    out by the sequences' lengths (eight sequences of 1 to 300 tokens here; most splits of a share
+    lie past the keys), the eager step, which knows the lengths, gives every sequence the same
+    number.  The same tokens from both, and the logits of the plain implementation."""
+    from minfer_amd import LLM, config_from_dict, write_random_model
+    from minfer_amd.kernels import ops
+    cfg = dict(TINIES["A"], max_position_embeddings=8320)
+    folder = str(tmp_path / "tiny_A_long")
+    write_random_model(folder, config_from_dict(cfg), 11)
+    places, splits = ops.decode_split_plan(8, cfg["num_key_value_heads"], 2, 8320)
+    assert places > splits > 1, "this session is meant to share the splits out"
+    lens = (5, 300, 33, 64, 129, 70, 1, 200)
+    prompts = [random_tokens(cfg["vocab_size"], n, 30 + i) for i, n in enumerate(lens)]
+    llm = LLM(folder, dtype="bfloat16", n_ctx=8320, n_slots=8)
+    eager = llm.generate(prompts, max_new=6, temp=0.0, repeat_penalty=1.0, stop_tokens=[], use_graph=False)
+    graph = llm.generate(prompts, max_new=6, temp=0.0, repeat_penalty=1.0, stop_tokens=[], use_graph=True)
+    assert eager.tokens == graph.tokens and all(len(t) == 6 for t in graph.tokens)
+    # the decode step itself, through the session, against the plain implementation
+    plain = pq.PlainQwen2.from_folder(folder)
+    eng = llm.engine
+    from minfer_amd.sampling import Sampler, SamplingParams
+    slots = [eng.new_sequence() for _ in prompts]
+    eng.step(slots, prompts, [[] for _ in prompts])
+    sess = eng.decode_session(len(prompts), 8320, Sampler(SamplingParams(temp=0.0, repeat_penalty=1.0)), use_graph=True)
+    sess.bind(slots, [t[0] for t in graph.tokens], list(range(len(prompts))), [1] * len(prompts))
+    sess.set_windows(prompts)
+    for step in range(1, 4):                   # eager, captured, replayed
+        sampled = sess.step()
+        assert sampled == [t[step] for t in graph.tokens]
+        got = sess.last_logits.float().cpu().numpy()
+        for i, p in enumerate(prompts):
+            want = plain.forward(list(p) + graph.tokens[i][:step])[-1]
+            sd = want.std()
+            err = got[i] - want
+            assert np.sqrt((err ** 2).mean()) <= 0.01 * sd and np.abs(err).max() <= 0.055 * sd, (step, i)
+    for s in slots:
+        eng.end_sequence(s)
+    assert not eng.cache.live_slots()
+
+
 def test_stop_tokens_end_sequences_early_and_batches_follow_each_other(folders):
     from minfer_amd import LLM
     plain = pq.PlainQwen2.from_folder(folders["A"])
