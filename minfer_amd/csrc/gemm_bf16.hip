@@ -1480,25 +1480,53 @@ __global__ __launch_bounds__(512) void panel_kernel(const bf16* __restrict__ A, 
   }
 }
 
+// The parts of a split are added in rounds of up to eight, a round's loads in flight together, in
+// the order of the splits (a plain loop over a count that is not known here is left to run split
+// by split, a trip to memory each).
+template <int CNT>
+__device__ __forceinline__ float add_parts(float v, const float* __restrict__ p, size_t stride) {
+  float x[CNT];
+#pragma unroll
+  for (int j = 0; j < CNT; ++j) x[j] = p[(size_t)j * stride];
+#pragma unroll
+  for (int j = 0; j < CNT; ++j) v += x[j];
+  return v;
+}
+
+__device__ __forceinline__ float sum_of_parts(const float* __restrict__ part, size_t stride, size_t at, int splits) {
+  float v = 0.f;
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    const float* p = part + (size_t)s0 * stride + at;
+    switch (min(8, splits - s0)) {
+      case 8: v = add_parts<8>(v, p, stride); break;
+      case 7: v = add_parts<7>(v, p, stride); break;
+      case 6: v = add_parts<6>(v, p, stride); break;
+      case 5: v = add_parts<5>(v, p, stride); break;
+      case 4: v = add_parts<4>(v, p, stride); break;
+      case 3: v = add_parts<3>(v, p, stride); break;
+      case 2: v = add_parts<2>(v, p, stride); break;
+      default: v = add_parts<1>(v, p, stride); break;
+    }
+  }
+  return v;
+}
+
 __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restrict__ part,
                                                             const float* __restrict__ bias,
                                                             void* __restrict__ C, int ldc, int M, int N,
                                                             int splits, int epi) {
   const int n = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
+  const size_t stride = (size_t)M * N;
   if (epi == EPI_SWIGLU) {       // n runs over the ldc outputs
     if (n >= ldc) return;
     const int ng = (n >> 5) * 64 + (n & 31);
-    float g = 0.f, u = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      g += part[((size_t)s * M + m) * N + ng];
-      u += part[((size_t)s * M + m) * N + ng + 32];
-    }
+    const float g = sum_of_parts(part, stride, (size_t)m * N + ng, splits);
+    const float u = sum_of_parts(part, stride, (size_t)m * N + ng + 32, splits);
     ((bf16*)C)[(size_t)m * ldc + n] = (bf16)swiglu_f(g, u);
     return;
   }
   if (n >= N) return;
-  float v = 0.f;
-  for (int s = 0; s < splits; ++s) v += part[((size_t)s * M + m) * N + n];
+  const float v = sum_of_parts(part, stride, (size_t)m * N + n, splits);
   store_out(C, ldc, m, n, v + (bias ? bias[n] : 0.f), epi);
 }
 
