@@ -19,6 +19,7 @@
 //
 // Used for decode in both precisions and for whole prompts in the 32-bit path.
 #pragma once
+#include <type_traits>
 #include "common.h"
 
 namespace attn_tokens {
@@ -250,20 +251,26 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
   for (int s = 0; s < n_used; ++s) L += of_split(ls, s) * of_split(wv, s);
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   if (d >= hd) return;
-  float a = 0.f;
-  // Eight splits a round, their loads in flight together (a round that is not full would otherwise
-  // run split by split, a trip to memory each).  Weight 0: a split without keys, whose sums nobody
-  // wrote, or one behind the last; its load goes to the first split's line instead and counts as 0.
-  for (int s0 = 0; s0 < n_used; s0 += 8) {
-    float w[8], v[8];
+  // Eight splits a round (sixteen where there are more than eight), their loads in flight together:
+  // a round that is not full, left to a plain loop, would run split by split, a trip to memory
+  // each.  Weight 0: a split without keys, whose sums nobody wrote, or one behind the last; its
+  // load goes to the first split's line instead and counts as 0.
+  auto rounds = [&](auto WIDTH) {
+    constexpr int W = decltype(WIDTH)::value;
+    float a = 0.f;
+    for (int s0 = 0; s0 < n_used; s0 += W) {
+      float w[W], v[W];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      w[j] = of_split(wv, s0 + j);
-      v[j] = base[(w[j] != 0.f ? (size_t)(s0 + j) * (hd + 2) : 0) + d];
+      for (int j = 0; j < W; ++j) {
+        w[j] = s0 + j < 64 ? of_split(wv, s0 + j) : 0.f;
+        v[j] = base[(w[j] != 0.f ? (size_t)(s0 + j) * (hd + 2) : 0) + d];
+      }
+#pragma unroll
+      for (int j = 0; j < W; ++j) a += (w[j] != 0.f ? v[j] : 0.f) * w[j];
     }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) a += (w[j] != 0.f ? v[j] : 0.f) * w[j];
-  }
+    return a;
+  };
+  const float a = n_used <= 8 ? rounds(std::integral_constant<int, 8>{}) : rounds(std::integral_constant<int, 16>{});
   out[th * hd + d] = from_f32<T>(a * inv);
 }
 
