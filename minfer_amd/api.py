@@ -46,7 +46,7 @@ class LLM:
         wanted = n_slots * ((self.n_ctx + PAGE - 1) // PAGE * PAGE)
         fits = None
         if max_tokens is None:
-            fits = tokens_that_fit(self.model)
+            fits = tokens_that_fit(self.model, max_seqs=n_slots)
             max_tokens = min(wanted, fits)
         self.engine = Engine(self.model, max_tokens=max_tokens, max_seqs=n_slots)
         per_token = cache_bytes_per_token(self.model.cache_requests(), self.model.rt.dtype)

@@ -44,23 +44,53 @@ def cache_bytes_per_token(requests: Dict[int, object], dtype: torch.dtype) -> in
     return sum(2 * r.n_kv_heads * r.head_dim * elem for r in requests.values() if isinstance(r, KVRequest))
 
 
-def tokens_that_fit(model: DecoderModel, max_step_tokens: int = 8192) -> int:
-    """How many tokens the cache can hold in the device memory that is free now (the weights are
-    loaded), after a reserve for everything else a step needs.  The reference divides a given
-    context over its slots (src/server/slot.rs:27-32 of yusiwen/minfer); here the given is what
-    the GPU has left."""
-    if model.rt.device.type != "cuda":
-        return 1 << 30                       # (tests drive the engine through stand-ins on the host)
-    free, total = torch.cuda.mem_get_info(model.rt.device)
-    s = model.spec
-    step = max_step_tokens * s.hidden_size * 4 * 12          # residual, q|k|v, feed-forward rows of a large step
-    reserve = max(RESERVE_BYTES_MIN, int(RESERVE_FRACTION * total)) + step
-    per_token = max(1, cache_bytes_per_token(model.cache_requests(), model.rt.dtype))
-    tokens = (free - reserve) // per_token // PAGE * PAGE
+def state_bytes_per_sequence(requests: Dict[int, object]) -> int:
+    """Bytes of fixed-size state one sequence slot takes, over all entries that ask for state."""
+    from ..cache.paged import StateRequest
+    total = 0
+    for r in requests.values():
+        if isinstance(r, StateRequest):
+            n = torch.empty((), dtype=r.dtype).element_size()
+            for d in r.shape:
+                n *= int(d)
+            total += n
+    return total
+
+
+# Sequence slots assumed for the fixed-size state when the caller names no number of sequences
+DEFAULT_STATE_SLOTS = 1024
+
+
+def plan_cache_tokens(free: int, total: int, per_token: int, state_bytes: int, step_bytes: int) -> int:
+    """Tokens (whole pages) a cache can hold in `free` bytes of a device of `total` bytes, after
+    the reserve (the larger of RESERVE_BYTES_MIN and RESERVE_FRACTION of the device), the
+    activations of the largest step (`step_bytes`) and the sequences' fixed-size state
+    (`state_bytes`, for all slots).  CacheError where not even one page fits."""
+    reserve = max(RESERVE_BYTES_MIN, int(RESERVE_FRACTION * total)) + int(step_bytes) + int(state_bytes)
+    per_token = max(1, int(per_token))
+    tokens = (int(free) - reserve) // per_token // PAGE * PAGE
     if tokens < PAGE:
-        raise CacheError(f"no room for a cache: {free >> 20} MiB free, {reserve >> 20} MiB held back, "
-                         f"{per_token} bytes a token")
+        raise CacheError(f"no room for a cache: {int(free) >> 20} MiB free, {reserve >> 20} MiB held back "
+                         f"({int(state_bytes) >> 20} MiB of them per-sequence state), {per_token} bytes a token")
     return int(tokens)
+
+
+def tokens_that_fit(model: DecoderModel, max_step_tokens: int = 8192, max_seqs: Optional[int] = None,
+                    mem_info=None) -> int:
+    """How many tokens the cache can hold in the device memory that is free now (the weights are
+    loaded), after a reserve for everything else a step needs and the fixed-size state of
+    `max_seqs` sequences.  The reference divides a given context over its slots
+    (src/server/slot.rs:27-32 of yusiwen/minfer); here the given is what the GPU has left.
+    `mem_info()` returns (free, total) bytes; by default the device's own figures."""
+    if mem_info is None:
+        if model.rt.device.type != "cuda":
+            return 1 << 30                   # (tests drive the engine through stand-ins on the host)
+        mem_info = lambda: torch.cuda.mem_get_info(model.rt.device)
+    free, total = mem_info()
+    requests = model.cache_requests()
+    step = max_step_tokens * model.spec.hidden_size * 4 * 12      # residual, q|k|v, feed-forward rows of a large step
+    state = state_bytes_per_sequence(requests) * int(max_seqs or DEFAULT_STATE_SLOTS)
+    return plan_cache_tokens(free, total, cache_bytes_per_token(requests, model.rt.dtype), state, step)
 
 
 class Engine:
@@ -74,7 +104,7 @@ class Engine:
         self.model = model
         self.device = model.rt.device
         if max_tokens is None:
-            max_tokens = tokens_that_fit(model)
+            max_tokens = tokens_that_fit(model, max_seqs=max_seqs)
             if max_seqs:
                 max_tokens = min(max_tokens, int(max_seqs) * ((model.spec.max_positions + PAGE - 1) // PAGE * PAGE))
         n_pages = (max_tokens + PAGE - 1) // PAGE

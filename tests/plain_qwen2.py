@@ -108,6 +108,46 @@ def swiglu_ffn(x: np.ndarray, w_gate, w_up, w_down) -> np.ndarray:
 
 # --------------------------------------------------------------------------- model
 
+class StreamedWeights:
+    """Tensors of one safetensors file by name, each read (and widened) when it is asked for and
+    not kept."""
+
+    def __init__(self, path: str, dtype=np.float64):
+        from safetensors import safe_open
+        self._file = safe_open(path, framework="pt")
+        self._names = set(self._file.keys())
+        self._dtype = dtype
+
+    def __contains__(self, name: str) -> bool:
+        return name in self._names
+
+    def __getitem__(self, name: str) -> np.ndarray:
+        import torch
+        return self._file.get_tensor(name).to(torch.float64).numpy().astype(self._dtype, copy=False)
+
+    def get(self, name: str, default=None):
+        return self[name] if name in self._names else default
+
+
+class _LayerWeights(dict):
+    """One layer's tensors, read once on first use and kept while the layer runs."""
+
+    def __init__(self, source, prefix: str):
+        super().__init__()
+        self._source, self._prefix = source, prefix
+
+    def __missing__(self, name: str):
+        self[name] = self._source[name]
+        return self[name]
+
+    def get(self, name: str, default=None):
+        if name in self:
+            return self[name]
+        v = self._source.get(name, default)
+        if v is not None:
+            self[name] = v
+        return v
+
 class PlainQwen2:
     """Weights as float64 arrays by their names in the file, hyper-parameters by their
     config.json keys.  ``forward`` runs one whole sequence from position 0."""
@@ -126,19 +166,28 @@ class PlainQwen2:
         self.tied = bool(c.get("tie_word_embeddings", False))
 
     @classmethod
-    def from_folder(cls, folder: str, dtype=np.float64) -> "PlainQwen2":
+    def from_folder(cls, folder: str, dtype=np.float64, streamed: bool = False) -> "PlainQwen2":
+        """`streamed`: tensors are read from the file each time they are used instead of all at
+        once, so a model of many gigabytes takes the host memory of one tensor at a time (run such
+        a model with `forward_many`, which reads every layer once for all requests)."""
         import torch
         from safetensors.torch import load_file
         with open(os.path.join(folder, "config.json")) as f:
             config = json.load(f)
-        raw = load_file(os.path.join(folder, "model.safetensors"))
+        path = os.path.join(folder, "model.safetensors")
+        if streamed:
+            model = cls(config, {}, dtype)
+            model.w = StreamedWeights(path, dtype)
+            return model
+        raw = load_file(path)
         weights = {k: t.to(torch.float64).numpy() for k, t in raw.items()}
         return cls(config, weights, dtype)
 
-    def layer(self, i: int, h: np.ndarray, positions) -> np.ndarray:
+    def layer(self, i: int, h: np.ndarray, positions, w=None) -> np.ndarray:
         """norm -> QKV(+bias) -> rope(q,k) -> attention -> O -> add -> norm -> SwiGLU -> add.
-        src/models/qwen2/graph.rs:59-177; scale 1/sqrt(hd) src/models/qwen2/loader.rs:36-38."""
-        w, p = self.w, f"model.layers.{i}."
+        src/models/qwen2/graph.rs:59-177; scale 1/sqrt(hd) src/models/qwen2/loader.rs:36-38.
+        `w`: the layer's tensors if the caller holds them already (`forward_many`)."""
+        w, p = self.w if w is None else w, f"model.layers.{i}."
         xn = rms_norm(h, w[p + "input_layernorm.weight"], self.eps)
         q = linear(xn, w[p + "self_attn.q_proj.weight"], w.get(p + "self_attn.q_proj.bias"))
         k = linear(xn, w[p + "self_attn.k_proj.weight"], w.get(p + "self_attn.k_proj.bias"))
@@ -170,6 +219,18 @@ class PlainQwen2:
     def forward(self, tokens) -> np.ndarray:
         """Logits [len(tokens), vocab] for one sequence starting at position 0."""
         return self.head(self.hidden(tokens))
+
+    def forward_many(self, requests: dict) -> dict:
+        """`forward` for every request of {id: tokens}, layer by layer over all of them, so that
+        streamed weights are read once.  The requests do not see each other."""
+        hs = {r: embedding(self.w["model.embed_tokens.weight"], toks) for r, toks in requests.items()}
+        for i in range(self.n_layers):
+            layer = _LayerWeights(self.w, f"model.layers.{i}.")
+            for r, toks in requests.items():
+                hs[r] = self.layer(i, hs[r], np.arange(len(toks)), layer)
+        xs = {r: rms_norm(h, self.w["model.norm.weight"], self.eps) for r, h in hs.items()}
+        wout = self.w["model.embed_tokens.weight"] if self.tied else self.w["lm_head.weight"]
+        return {r: linear(x, wout) for r, x in xs.items()}
 
 
 # --------------------------------------------------------------------------- sampling

@@ -6,7 +6,7 @@ import pytest
 from plain_qwen2 import PlainQwen2
 from replays import (batch_steps, chunk_steps, compare, plain_logits, requests_for, run_steps, tail_steps,
                      whole_steps)
-from tiny import TINIES, write_tiny
+from tiny import TINIES, TINY_LONG, write_tiny
 
 pytestmark = pytest.mark.gpu
 
@@ -190,3 +190,99 @@ def test_sessions_and_memory_stay_flat_over_many_seeds(folders):
         llm.generate(prompts, max_new=3, temp=0.5 + 0.01 * k, seed=1, stop_tokens=[])
     assert len(llm.engine._sessions) <= MAX_SESSIONS
     assert not llm.engine.cache.live_slots()
+
+
+# ------------------------------------------------------------------ long prompts
+@pytest.fixture(scope="module")
+def long_model(tmp_path_factory):
+    """Two layers with room for 4,096 positions.  The q and k matrices are scaled up so that the
+    scores of a query spread over several units: a softmax over two thousand keys then rests on a
+    few of them, wherever they lie, and a page of keys left out, read twice or taken from another
+    sequence moves the logits by far more than the bounds (with the plain random weights every
+    key weighs the same two-thousandth and such a fault hides in the rounding)."""
+    import torch
+    from safetensors.torch import load_file, save_file
+    from minfer_amd import config_from_dict, write_random_model
+    folder = write_random_model(str(tmp_path_factory.mktemp("long") / "m"), config_from_dict(TINY_LONG), seed=21)
+    path = folder + "/model.safetensors"
+    t = load_file(path)
+    for name in list(t):
+        if "q_proj.weight" in name or "k_proj.weight" in name:
+            t[name] = (t[name].float() * 5.0).to(t[name].dtype)
+    save_file(t, path)
+    plain = PlainQwen2.from_folder(folder)
+    reqs = requests_for(TINY_LONG["vocab_size"], (2100, 700, 1500), seed=22)
+    ref = plain_logits(plain, reqs)
+    # the construction does what it says: the last query's largest softmax weight in layer 0 is
+    # far above 1 / keys
+    import numpy as np
+    import plain_qwen2 as pq
+    toks = reqs["r0"]
+    h = pq.embedding(plain.w["model.embed_tokens.weight"], toks)
+    xn = pq.rms_norm(h, plain.w["model.layers.0.input_layernorm.weight"], plain.eps)
+    pos = np.arange(len(toks))
+    q = pq.rope_neox(pq.linear(xn[-1:], plain.w["model.layers.0.self_attn.q_proj.weight"],
+                               plain.w["model.layers.0.self_attn.q_proj.bias"]), pos[-1:], plain.nh, plain.hd, plain.theta)
+    k = pq.rope_neox(pq.linear(xn, plain.w["model.layers.0.self_attn.k_proj.weight"],
+                               plain.w["model.layers.0.self_attn.k_proj.bias"]), pos, plain.nk, plain.hd, plain.theta)
+    s = (k.reshape(len(toks), plain.nk, plain.hd)[:, 0] @ q.reshape(plain.nh, plain.hd)[0]) / np.sqrt(plain.hd)
+    w = pq.softmax_rows(s[None])[0]
+    assert w.max() > 20.0 / len(toks), f"scores are too flat for this test (largest weight {w.max():.4f})"
+    return folder, reqs, ref
+
+
+def _wanted(n_new: int, first: int = 0):
+    """The last 16 rows of a step's new tokens and a few in the middle, as offsets."""
+    mid = [o for o in (0, 1, 63, 64, 65, n_new // 3, n_new // 2, n_new // 2 + 1) if 0 <= o < n_new - 16]
+    return sorted(set(mid + list(range(max(0, n_new - 16), n_new))))
+
+
+def _step_rows(eng, slots, ids, chunks, starts, rows):
+    """One engine step through its three stages (so the test can look at the step's context);
+    logits of the wanted offsets into `rows` as (request, position)."""
+    want = [_wanted(len(c)) for c in chunks]
+    ctx = eng.build_context([slots[r] for r in ids], chunks, want)
+    logits = eng.model.forward(ctx).cpu().numpy()
+    eng.cache.commit(ctx.new_lengths)
+    eng.cache.check_invariants()
+    r = 0
+    for rid, offs, start in zip(ids, want, starts):
+        for o in offs:
+            rows[(rid, start + o)] = logits[r]
+            r += 1
+    assert r == logits.shape[0]
+    return ctx
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompts_agree_with_plain(long_model, dtype):
+    """Prompts of 2,100, 700 and 1,500 tokens in one step, and then, on the same engine (pages
+    used again, poisoned in between), 64 new tokens of each on some 2,000, 600 and 1,400 cached
+    ones: the case in which the prompt attention shares a block of queries' pages between several
+    workgroups.  Logits of the last 16 rows of every portion and of some in the middle against the
+    plain implementation."""
+    folder, reqs, ref = long_model
+    ids = list(reqs)
+    eng = engine_for(folder, dtype, max_tokens=64 * 70)
+    # all three whole, in one step
+    slots = {r: eng.new_sequence() for r in ids}
+    rows = {}
+    _step_rows(eng, slots, ids, [reqs[r] for r in ids], [0, 0, 0], rows)
+    for r in ids:
+        eng.end_sequence(slots[r])
+    compare(rows, ref, dtype, "long prompts, one step", layers=2)
+    # all but the last 100 tokens, then 64 on top of them, then the rest
+    slots = {r: eng.new_sequence() for r in ids}
+    rows = {}
+    heads = [len(reqs[r]) - 100 for r in ids]
+    _step_rows(eng, slots, ids, [reqs[r][:n] for r, n in zip(ids, heads)], [0, 0, 0], rows)
+    ctx = _step_rows(eng, slots, ids, [reqs[r][n:n + 64] for r, n in zip(ids, heads)], heads, rows)
+    if dtype == "bfloat16":
+        shared = [v for k, v in ctx._memo.items() if k[0] == "shared_query_tiles"]
+        assert shared and shared[0] is not None, "this step was meant to share its query blocks' pages"
+        assert shared[0][4] > 1
+    _step_rows(eng, slots, ids, [reqs[r][n + 64:] for r, n in zip(ids, heads)], [n + 64 for n in heads], rows)
+    for r in ids:
+        eng.end_sequence(slots[r])
+    compare(rows, ref, dtype, "long prompts, 64 tokens on a long cache", layers=2)
+    assert not eng.cache.live_slots()

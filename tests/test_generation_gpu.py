@@ -211,6 +211,93 @@ def test_command_line(folders, tmp_path):
     assert r.returncode == 1 and "requires a value" in r.stderr
 
 
+def test_debug_switches_change_no_token(folders):
+    """MF_DEBUG_SYNC=1 (a synchronisation and an error check behind every launch, its name
+    printed) and MF_TIMING=1 (a token's time split into forward and sampling): the same tokens as
+    without them, and the lines they promise (the reference's MINFER_CUDA_DEBUG and
+    MINFER_TIMING, src/cuda.rs:378-395 and src/main.rs:552-609 of yusiwen/minfer)."""
+    exe = [sys.executable, os.path.join(ROOT, "bin", "minfer"), folders["A"], "--prompt-tokens", "5,6,7;9,10,11,12",
+           "--temp", "0.7", "--seed", "5", "-n", "6", "--n-ctx", "64", "--stop-token", "100000"]
+    runs = {}
+    for switch in ("", "MF_DEBUG_SYNC", "MF_TIMING"):
+        env = dict(os.environ, PYTHONPATH=ROOT)
+        env.pop("MF_DEBUG_SYNC", None)
+        env.pop("MF_TIMING", None)
+        if switch:
+            env[switch] = "1"
+        r = subprocess.run(exe, capture_output=True, text=True, env=env, timeout=300)
+        assert r.returncode == 0, r.stderr
+        runs[switch] = r
+    plain_out = runs[""].stdout
+    assert len(plain_out.strip().splitlines()) == 2
+    assert runs["MF_DEBUG_SYNC"].stdout == plain_out and runs["MF_TIMING"].stdout == plain_out
+    ok = [l for l in runs["MF_DEBUG_SYNC"].stderr.splitlines() if l.startswith("[minfer_amd] ") and l.endswith(" OK")]
+    assert len(ok) > 50 and any("attn" in l for l in ok) and any("gemm" in l for l in ok) and any("sample" in l or "argmax" in l for l in ok)
+    assert " OK" not in runs[""].stderr and "[MF_TIMING]" not in runs[""].stderr
+    timing = [l for l in runs["MF_TIMING"].stderr.splitlines() if l.startswith("[MF_TIMING]")]
+    assert len(timing) == 1 and "sample" in timing[0] and "forward" in timing[0] and "ms/tok" in timing[0]
+
+
+def test_trace_names_every_launch_of_a_step(folders):
+    """`ops.start_trace` / `stop_trace`: one (name, microseconds) entry per kernel launch, in launch
+    order.  A 32-bit prompt step of the two-layer model is: the embedding; per layer norm, q|k|v,
+    rotation + cache write, attention, o, norm, gate|up, SwiGLU, down, with the wanted rows
+    gathered before the last feed-forward; final norm; head."""
+    from minfer_amd import Engine, load_model
+    from minfer_amd.kernels import ops
+    eng = Engine(load_model(folders["A"], dtype="float32"), max_tokens=128)
+    s = eng.new_sequence()
+    eng.step([s], [[1, 2, 3]], "last")                  # builds tables and workspaces outside the trace
+    eng.end_sequence(s)
+    s = eng.new_sequence()
+    ops.start_trace()
+    eng.step([s], [[4, 5, 6, 7, 8]], "last")
+    entries = ops.stop_trace()
+    eng.end_sequence(s)
+    layer = ["rmsnorm", "gemm_f32", "rope_kvwrite", "attn_tokens_f32", "gemm_f32", "rmsnorm", "gemm_f32", "swiglu", "gemm_f32"]
+    last = layer[:5] + ["gather_rows"] + layer[5:]
+    want = ["embed"] + layer + last + ["rmsnorm", "gemm_f32"]
+    assert [name.split()[0] for name, _ in entries] == want
+    assert all(us >= 0.0 for _, us in entries) and sum(us for _, us in entries) > 0.0
+    assert ops.stop_trace() == []                       # nothing is recorded once stopped
+    s = eng.new_sequence()
+    eng.step([s], [[1]], "last")
+    eng.end_sequence(s)
+    assert ops.stop_trace() == []
+
+
+def test_cache_is_sized_from_the_free_memory_when_that_is_less(folders, monkeypatch):
+    """With little device memory free, the cache takes what fits instead of slots x context
+    (`cache_plan` says so), generation plans its batches by that capacity, and with no room at all
+    the error says why."""
+    import torch
+    from minfer_amd import LLM
+    from minfer_amd.cache import CacheError
+    from minfer_amd.engine.engine import RESERVE_BYTES_MIN
+    real = torch.cuda.mem_get_info
+    total = real()[1]
+    reserve = max(RESERVE_BYTES_MIN, int(0.06 * total)) + 8192 * 64 * 4 * 12
+    per_token = 2 * 2 * 2 * 16 * 2                      # two layers, K and V, two kv heads of 16, bfloat16
+    state = {"free": reserve + 5 * 64 * per_token + 100}
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (state["free"], total))
+    llm = LLM(folders["A"], dtype="bfloat16", n_ctx=128, n_slots=4)
+    plan = llm.cache_plan
+    assert plan["limited_by_memory"] and plan["fits"] == 5 * 64 and plan["tokens"] == 5 * 64
+    assert plan["bytes_per_token"] == per_token and llm.engine.capacity_tokens() == 320
+    prompts = [random_tokens(512, n, 60 + i) for i, n in enumerate((70, 30, 90, 20))]      # 2 + 1 + 2 + 1 pages and growth
+    res = llm.generate(prompts, max_new=40, temp=0.0, stop_tokens=[])
+    assert [len(t) for t in res.tokens] == [min(40, 128 - len(p) + 1) for p in prompts]    # 128 positions end the longest
+    assert len(res.batches) > 1, "four requests cannot be live together in five pages"
+    monkeypatch.setattr(torch.cuda, "mem_get_info", real)
+    roomy = LLM(folders["A"], dtype="bfloat16", n_ctx=128, n_slots=4)
+    assert not roomy.cache_plan["limited_by_memory"] and roomy.cache_plan["tokens"] == 4 * 128
+    assert roomy.generate(prompts, max_new=40, temp=0.0, stop_tokens=[]).tokens == res.tokens
+    state["free"] = reserve + 10
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (state["free"], total))
+    with pytest.raises(CacheError, match="no room for a cache"):
+        LLM(folders["A"], dtype="bfloat16", n_ctx=128, n_slots=4)
+
+
 def replay_program(folder, dtype, steps, out_dir, max_tokens):
     """Runs bin/trace_run as a program; sends each step only after the last `done`."""
     exe = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,

@@ -118,6 +118,18 @@ def test_rope_table(ops, theta, half):
     close(sn, rs, 2e-7)
 
 
+def test_rope_table_frequency_ladder_by_hand(ops):
+    """freq_i = theta^(-2i/hd): with head_dim 8 and theta 10^4 the frequencies are 1, 0.1, 0.01
+    and 0.001, so row 1000 of the table holds cos and sin of 1000, 100, 10 and 1 radians (values
+    from tables, not from the formula; src/graph/cpu_backend.rs:415 of yusiwen/minfer)."""
+    cs, sn = ops.rope_table(1001, 4, 10000.0, 1.0, DEV)
+    want_c = [0.5623790762907029, 0.8623188722876839, -0.8390715290764524, 0.5403023058681398]
+    want_s = [0.8268795405320025, -0.5063656411097588, -0.5440211108893698, 0.8414709848078965]
+    assert (cs[1000].double().cpu() - torch.tensor(want_c, dtype=torch.float64)).abs().max() < 1e-6
+    assert (sn[1000].double().cpu() - torch.tensor(want_s, dtype=torch.float64)).abs().max() < 1e-6
+    assert abs(cs[1, 0].item() - 0.5403023058681398) < 1e-7 and abs(sn[1, 0].item() - 0.8414709848078965) < 1e-7
+
+
 def make_cache(n_pages, nk, hd, dtype, seed=0):
     """K and V as [pages][kv_heads][64][head_dim]: for V this is the logical view, `stored_v`
     gives what the kernels take."""

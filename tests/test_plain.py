@@ -92,6 +92,30 @@ def test_rope_pairs_are_half_split_and_the_sign_is_right():
     assert np.allclose(out[..., :hd // 2], z.real) and np.allclose(out[..., hd // 2:], z.imag)
 
 
+# cos and sin of 1, 10, 100 and 1000 radians, from tables, not from the formula under test
+COS_1_10_100_1000 = (0.5403023058681398, -0.8390715290764524, 0.8623188722876839, 0.5623790762907029)
+SIN_1_10_100_1000 = (0.8414709848078965, -0.5440211108893698, -0.5063656411097588, 0.8268795405320025)
+
+
+def test_rope_frequency_ladder_by_hand():
+    """freq_i = theta^(-2i/hd) (src/graph/cpu_backend.rs:415, scripts/verify_rope.py:44 of
+    yusiwen/minfer).  With hd 8 and theta 10^4 the four frequencies are exactly 1, 0.1, 0.01 and
+    0.001, so at position 1000 the angles are 1000, 100, 10 and 1 radians: a ladder with another
+    exponent (i/hd, 2i/(hd/2), (2i+1)/hd), another base or the frequencies in another order gives
+    other numbers here, which no invariant of the rotation notices."""
+    hd = 8
+    for i in range(4):
+        x = np.zeros((1, hd))
+        x[0, i] = 1.0
+        y = pq.rope_neox(x, [1000], 1, hd, 10000.0)[0]
+        assert abs(y[i] - COS_1_10_100_1000[3 - i]) < 1e-9 and abs(y[i + 4] - SIN_1_10_100_1000[3 - i]) < 1e-9, i
+    # position 1: angles 1, 0.1, 0.01, 0.001; the first pair turns by one radian exactly
+    x = np.zeros((1, hd))
+    x[0, 0] = 1.0
+    y = pq.rope_neox(x, [1], 1, hd, 10000.0)[0]
+    assert abs(y[0] - COS_1_10_100_1000[0]) < 1e-12 and abs(y[4] - SIN_1_10_100_1000[0]) < 1e-12
+
+
 def test_rope_keeps_norms_and_depends_on_distance_only():
     hd = 16
     q, k = rnd(1, hd, seed=12), rnd(1, hd, seed=13)

@@ -1,9 +1,10 @@
 """The widths of Qwen2.5-7B (hidden 3584, 28 heads over 4 kv heads of 128, feed-forward 18944,
 vocabulary 152064) with random weights against the plain implementation in 64 bits:
 
-* four layers with an untied head (of the model's 28: the plain implementation's time and the
-  4 GB folder bound the depth), 32-bit logits within 1e-4 and bfloat16 within the suite's bound
+* four layers with an untied head, 32-bit logits within 1e-4 and bfloat16 within the suite's bound
   under all the ways of cutting requests into steps;
+* all 28 layers (the benchmark's model; the plain implementation streams the 15 GB file tensor by
+  tensor), whole, one by one and in unequal batches;
 * one layer with a tied head, the same, and a batch of twenty;
 * a context of 2,150 tokens whose last tokens are decoded one by one through the captured decode
   step (key splits and their merge in bfloat16), with weights made so that the one key that
@@ -103,6 +104,49 @@ def test_four_layers_untied_head_at_7b_widths(folder4, reference4, dtype):
     assert model.head.weight.data_ptr() != model.embedding.weight.data_ptr() and len(model.blocks) == 4
     eng = Engine(model, max_tokens=64 * 4, poison_cache=True)
     worst = all_replays(eng, reqs, ref, dtype, "7B widths, 4 layers, untied", layers=4)
+    print(f"{dtype}: worst abs err {worst:.3e} (logit std {float(ref['r1'].std()):.3f})")
+
+
+# ------------------------------------------------------------------ the whole depth: all 28 layers
+SHAPE_7B_FULL = dict(WIDTHS_7B, num_hidden_layers=28, tie_word_embeddings=False)
+
+
+@pytest.fixture(scope="module")
+def full_depth(tmp_path_factory):
+    """The model of the benchmark, every layer of it (a folder of 15 GB), and the plain
+    implementation's logits for four short requests.  The plain side reads the file tensor by
+    tensor and runs all requests through a layer before it reads the next, so the host holds one
+    matrix in 64 bits at a time."""
+    import shutil
+    import time
+    from minfer_amd import config_from_dict, write_random_model
+    root = tmp_path_factory.mktemp("shape7b28")
+    t0 = time.time()
+    folder = write_random_model(str(root / "m"), config_from_dict(SHAPE_7B_FULL), seed=11)
+    t1 = time.time()
+    reqs = requests_for(152064, (5, 13, 9, 21), seed=12)
+    ref = PlainQwen2.from_folder(folder, dtype=np.float64, streamed=True).forward_many(reqs)
+    print(f"28 layers: folder written in {t1 - t0:.0f} s, plain implementation {time.time() - t1:.0f} s", flush=True)
+    yield folder, reqs, ref
+    shutil.rmtree(str(root), ignore_errors=True)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_all_28_layers_at_7b_widths(full_depth, dtype):
+    """The configuration the benchmark measures, whole: 32-bit logits within 1e-4 of the plain
+    implementation, bfloat16 within the bound for 28 layers, each request alone and whole, its last
+    tokens one by one, and in unequal batches whose slots are used again (the reference's check of
+    a real model's prompt and decode logits, src/models/qwen2/graph.rs:486-589 of yusiwen/minfer)."""
+    from minfer_amd import Engine, load_model
+    folder, reqs, ref = full_depth
+    model = load_model(folder, dtype=dtype)
+    assert len(model.blocks) == 28 and model.head.weight.data_ptr() != model.embedding.weight.data_ptr()
+    eng = Engine(model, max_tokens=64 * 8, poison_cache=True)
+    ids = list(reqs)
+    worst = max(compare(run_steps(eng, whole_steps(reqs)), ref, dtype, "28 layers whole", 28),
+                compare(run_steps(eng, tail_steps(reqs, tail=8)), ref, dtype, "28 layers one by one", 28),
+                compare(run_steps(eng, batch_steps(reqs, [ids[:3], ids[3:] + ids[:1]])), ref, dtype,
+                        "28 layers batches", 28))
     print(f"{dtype}: worst abs err {worst:.3e} (logit std {float(ref['r1'].std()):.3f})")
 
 

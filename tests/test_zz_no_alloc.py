@@ -1,7 +1,8 @@
 """The entry point that allocates nothing (csrc/noalloc.h), called through ctypes: the same
 output as the entry point that takes the caller's workspace, on two calls in a row of which the
-second is smaller (so it finds the first one's partials in the library's array), a size beyond the
-array refused, and no device memory allocated by the calls."""
+second is smaller (so it finds the first one's partials in the library's array), both against
+plain attention in 64 bits, a size beyond the array refused, and the device's free memory (the
+driver's figure, not torch's) the same before and after a call."""
 import ctypes
 from ctypes import c_float, c_int, c_size_t, c_void_p
 
@@ -61,46 +62,68 @@ def run_both(lib, tensors, nh, nk, hd, n_splits, scale=0.11):
                                  n_tok, nh, nk, hd, scale, 0, n_splits, 0, stream)
     assert rc == 0
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # what the device itself has free (the driver's figure, which a hipMalloc inside the library
+    # would move; torch's own counters see only torch's allocator) and what torch has reserved
+    free_before, reserved_before = torch.cuda.mem_get_info(DEV)[0], torch.cuda.memory_reserved(DEV)
     rc = lib.mf_attn_decode_bf16_noalloc(p(q), p(kc), p(vt), p(table), table.shape[1], p(pos), p(seq), p(got),
                                          n_tok, nh, nk, hd, scale, 0, n_splits, stream)
     assert rc == 0, f"noalloc entry point returned {rc}"
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.memory_reserved(DEV) == reserved_before
+    assert torch.cuda.mem_get_info(DEV)[0] == free_before, "the call changed the device's free memory"
     return want, got
+
+
+def plain_attention(tensors, nh, nk, hd, scale=0.11):
+    """softmax(q.k scale) v in 64 bits from the pages, one head at a time: [tokens][heads * hd]."""
+    q, kc, vt, table, pos, seq = [t.cpu() for t in tensors]
+    out = torch.zeros(q.shape, dtype=torch.float64)
+    for b in range(q.shape[0]):
+        n = int(pos[b]) + 1
+        pages = table[int(seq[b]), :(n + PAGE - 1) // PAGE].long()
+        k = kc[pages].double().permute(1, 0, 2, 3).reshape(nk, -1, hd)[:, :n]                 # [nk][keys][hd]
+        v = vt[pages].double().permute(1, 0, 2, 4, 3).reshape(nk, -1, hd)[:, :n]              # [pages][nk][2][hd][32] -> keys
+        qh = q[b].double().view(nh, hd)
+        for h in range(nh):
+            s = (k[h // (nh // nk)] @ qh[h]) * scale
+            out[b, h * hd:(h + 1) * hd] = torch.softmax(s, 0) @ v[h // (nh // nk)]
+    return out
+
+
+def close_to_plain(got, tensors, nh, nk, hd):
+    """Against plain attention in 64 bits, so that "equal" is not "equally wrong": the output is
+    rounded to bfloat16 (values up to about 1) and the probabilities are before the second product."""
+    want = plain_attention(tensors, nh, nk, hd)
+    err = (got.double().cpu() - want).abs().max().item()
+    assert err < 2e-2, err
 
 
 def test_noalloc_entry_point_matches_the_workspace_one_twice_in_a_row():
     lib = library()
     assert lib.mf_attn_decode_bf16_noalloc_capacity() == 1 << 20
     nh, nk, hd = 28, 4, 128
+    # a first, small call, so that the library's set-up (the address of its array) is behind us
+    # when free memory is compared around the calls below
+    run_both(lib, case(1, [70], nh, nk, hd, seed=9), nh, nk, hd, n_splits=2)
     # first call: 6 sequences of up to 2,000 keys in 8 splits; second: fewer, shorter, fewer splits,
     # so the array still holds the first call's partials beyond and between what the second writes
     first = case(6, [2000, 1300, 777, 64, 65, 1], nh, nk, hd, seed=1)
     want, got = run_both(lib, first, nh, nk, hd, n_splits=8)
     assert torch.isfinite(want.float()).all() and torch.equal(want, got)
+    close_to_plain(got, first, nh, nk, hd)
     second = case(2, [300, 129], nh, nk, hd, seed=2)
     want2, got2 = run_both(lib, second, nh, nk, hd, n_splits=3)
     assert torch.isfinite(want2.float()).all() and torch.equal(want2, got2)
-    # against plain attention in 64 bits, so that "equal" is not "equally wrong"
-    q, kc, vt, table, pos, seq = [t.cpu() for t in second]
-    for b in range(2):
-        n = int(pos[b]) + 1
-        pages = table[b, :(n + PAGE - 1) // PAGE].long()
-        k = kc[pages].double().permute(1, 0, 2, 3).reshape(nk, -1, hd)[:, :n]                 # [nk][keys][hd]
-        v = vt[pages].double().permute(1, 0, 2, 4, 3).reshape(nk, -1, hd)[:, :n]              # [pages][nk][2][hd][32] -> keys
-        qh = q[b].double().view(nh, hd)
-        for h in range(nh):
-            s = (k[h // (nh // nk)] @ qh[h]) * 0.11
-            o = torch.softmax(s, 0) @ v[h // (nh // nk)]
-            assert (got2[b].float().cpu().view(nh, hd)[h].double() - o).abs().max() < 2e-2
+    close_to_plain(got2, second, nh, nk, hd)
     # one split: no scratch at all
     want3, got3 = run_both(lib, second, nh, nk, hd, n_splits=1)
     assert torch.equal(want3, got3)
+    close_to_plain(got3, second, nh, nk, hd)
     # other head sizes and groups go through the same kernels
     third = case(3, [500, 31, 260], 9, 3, 48, seed=3)
     want4, got4 = run_both(lib, third, 9, 3, 48, n_splits=4)
     assert torch.equal(want4, got4)
+    close_to_plain(got4, third, 9, 3, 48)
 
 
 def test_noalloc_entry_point_refuses_what_its_array_cannot_hold():

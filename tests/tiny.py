@@ -28,6 +28,13 @@ TINY_C = dict(
 
 TINIES = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 
+# for long prompts: room for 4,096 positions, two layers, three heads to a kv head
+TINY_LONG = dict(
+    architectures=["Qwen2ForCausalLM"], model_type="qwen2", hidden_act="silu",
+    num_hidden_layers=2, hidden_size=192, num_attention_heads=6, num_key_value_heads=2,
+    intermediate_size=272, vocab_size=600, rope_theta=1000000.0, rms_norm_eps=1e-6,
+    max_position_embeddings=4096, tie_word_embeddings=False, use_sliding_window=False)
+
 
 def write_tiny(tmp_path, name: str, seed: int = 0) -> str:
     from minfer_amd import config_from_dict, write_random_model
