@@ -270,9 +270,13 @@ __global__ __launch_bounds__(256, NKS <= 8 ? 2 : 1) void attn_prefill_kernel(
     __syncthreads();
     int* last = reinterpret_cast<int*>(smem);            // (the page buffers are free behind the loop's last barrier)
     if (tid == 0) {
+      // Counting in releases this block's part and, for the block that arrives last, acquires the
+      // others': the block's stores are ordered before the increment by the barrier above (and are
+      // atomic stores themselves), the increments on one counter form a release sequence, and the
+      // last arriver's loads below are ordered behind its increment by the barrier that follows.
       int* count = arrived + share_slot * nh + h;
-      const int before = __hip_atomic_fetch_add(count, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      if (before == n_shares - 1) __hip_atomic_store(count, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);   // as it was found
+      const int before = __hip_atomic_fetch_add(count, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      if (before == n_shares - 1) __hip_atomic_store(count, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as it was found
       *last = before == n_shares - 1;
     }
     __syncthreads();

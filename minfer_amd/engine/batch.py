@@ -57,14 +57,20 @@ class StepContext:
             self._memo[key] = (both[0], both[1])
         return self._memo[key]
 
-    def shared_query_tiles(self, block: int, page: int, window: int, load_of, max_shares: int):
+    def shared_query_tiles(self, block: int, page: int, window: int, n_heads: int, n_cu: int, per_cu: int,
+                           min_pages: int, max_shares: int, min_imbalance: float = 1.5):
         """(tile_seq, tile_q0, tile_share, n_slots, most shares): as `query_tiles`, but a block of queries with
         many pages of keys is listed several times, once for each of the workgroups that are to
-        take its pages in turn.  `load_of(total_pages)` gives the number of pages one workgroup
-        should get at most; entry i of tile_share is share + 256 * shares + 65536 * slot (0 for a
+        take its pages in turn.  A workgroup should get at most its even share of the step's pages
+        (all blocks x `n_heads` heads over the `n_cu` x `per_cu` workgroups that run at once), and at
+        least `min_pages`; entry i of tile_share is share + 256 * shares + 65536 * slot (0 for a
         block listed once), slots numbering the blocks that are shared.  None where no block needs
-        sharing."""
-        key = ("shared_query_tiles", block, page, window, max_shares)
+        sharing, or where sharing cannot gain: the step takes at least as long as a CU's even
+        share of all pages and as its longest block, and only where the longest block is
+        `min_imbalance` times that share is there time to win by cutting it (putting the parts
+        together has a price).  Kept per set of arguments: layers with other head counts plan for
+        themselves."""
+        key = ("shared_query_tiles", block, page, window, n_heads, n_cu, per_cu, min_pages, max_shares, min_imbalance)
         if key not in self._memo:
             tiles = []
             for b, n in enumerate(self.host_new):
@@ -73,7 +79,12 @@ class StepContext:
                     last_key = first + min(q0 + block, n) - 1
                     first_key = max(0, first + q0 - window + 1) if window > 0 else 0
                     tiles.append((last_key // page - first_key // page + 1, b, q0))
-            target = max(1, int(load_of(sum(t[0] for t in tiles))))
+            total = sum(t[0] for t in tiles)
+            longest = max(t[0] for t in tiles)
+            if longest * max(1, n_cu) < min_imbalance * total * n_heads:
+                self._memo[key] = None
+                return None
+            target = max(1, int(min_pages), -(-total * n_heads // max(1, n_cu * per_cu)))
             entries, n_slots, most = [], 0, 1
             for pages, b, q0 in tiles:
                 shares = min(max_shares, (pages + target - 1) // target)

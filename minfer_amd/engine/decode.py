@@ -64,8 +64,9 @@ class DecodeSession:
         self._launched = self._collected = 0
         self.last_logits: Optional[torch.Tensor] = None
         self.graph: Optional[torch.cuda.CUDAGraph] = None
-        self._graph_generation = -1          # ops.workspace_generation() the graph was captured under
+        self._lease = None                   # ops.GraphLease of the captured graph
         self.warm = False
+        self._finalizer = None
         self.slots: List[int] = []
         self._host_tables: Dict[int, List[List[int]]] = {}
         engine.model.prepare(max_len)
@@ -89,6 +90,9 @@ class DecodeSession:
         """Gives up the captured graph and with it the memory pool it holds."""
         self.graph = None
         self.warm = False
+        if self._finalizer is not None:
+            self._finalizer()                # gives the lease back (once)
+        self._lease = self._finalizer = None
 
     def bind(self, slots: Sequence[int], next_tokens: Sequence[int], keys: Sequence[int],
              steps: Sequence[int], sampler=None) -> None:
@@ -166,8 +170,8 @@ class DecodeSession:
                 if self._host_tables.get(id(g)) != rows:
                     self.tables[id(g)].copy_(torch.tensor(rows, dtype=torch.int32))
                     self._host_tables[id(g)] = rows
-        if self.graph is not None and self._graph_generation != ops.workspace_generation():
-            self.release()                   # a buffer the graph points at was replaced: capture again
+        if self.graph is not None and self._lease.stale():
+            self.release()                   # a buffer the graph points at was replaced: capture again, let the old one go
         if not self.use_graph:
             self._run()
         elif self.graph is not None:
@@ -186,7 +190,8 @@ class DecodeSession:
                 if collecting:
                     gc.enable()
             self.graph = graph
-            self._graph_generation = ops.workspace_generation()
+            self._lease = ops.lease_graph()
+            self._finalizer = weakref.finalize(self, ops.release_graph, self._lease)
             graph.replay()
         k = self._launched % 2
         if self._pinned is not None:

@@ -149,10 +149,14 @@ class Engine:
 
     def decode_session(self, n_seqs: int, max_len: int, sampler, use_graph: bool = True):
         """A `DecodeSession` for this batch size, reused (with its captured graph) while the
-        size, the reach and the sampling options other than the seed stay the same.  At most
+        size, the reach (`max_len` rounded up to a power of two, at least 256, at most the model's
+        positions) and the sampling options other than the seed stay the same.  At most
         MAX_SESSIONS are kept; the one unused for longest gives up its graph and buffers."""
         from .decode import DecodeSession
-        max_len = min(self.max_positions, (max_len + 255) // 256 * 256)
+        reach = 256                          # in powers of two: prompts of many lengths share few captures
+        while reach < max_len:
+            reach *= 2
+        max_len = min(self.max_positions, reach)
         key = (n_seqs, max_len, sampler.structure, use_graph)
         session = self._sessions.get(key)
         if session is None:

@@ -20,13 +20,24 @@ from ..weights.loader import TensorSpec
 
 
 def _build_block(bs: BlockSpec, rt: Runtime):
+    """The block's arrangement and the parts its spec names; the arrangement says which it needs."""
     if bs.kind not in BLOCKS:
         raise KeyError(f"unknown block arrangement {bs.kind!r}; registered: {', '.join(sorted(BLOCKS))}")
-    return BLOCKS[bs.kind](
-        make_part(MIXERS, bs.mixer, rt, "mixer"),
-        make_part(FEED_FORWARDS, bs.feed_forward, rt, "feed-forward"),
-        make_part(NORMS, bs.mixer_norm, rt, "norm"),
-        make_part(NORMS, bs.feed_forward_norm, rt, "norm"), rt)
+    cls = BLOCKS[bs.kind]
+    where = f"block {bs.prefix!r} ({bs.kind})"
+    if cls.needs_mixer and bs.mixer is None:
+        raise ValueError(f"{where}: this arrangement needs a mixer")
+    if cls.needs_feed_forward and bs.feed_forward is None:
+        raise ValueError(f"{where}: this arrangement needs a feed-forward")
+    known = tuple(cls.norm_names) + tuple(cls.optional_norms)
+    missing = [n for n in cls.norm_names if n not in bs.norms]
+    unknown = [n for n in bs.norms if n not in known]
+    if missing or unknown:
+        raise ValueError(f"{where}: norms missing {missing}, not known to the arrangement {unknown}; "
+                         f"it takes {list(known)}")
+    return cls(None if bs.mixer is None else make_part(MIXERS, bs.mixer, rt, "mixer"),
+               None if bs.feed_forward is None else make_part(FEED_FORWARDS, bs.feed_forward, rt, "feed-forward"),
+               {name: make_part(NORMS, spec, rt, "norm") for name, spec in bs.norms.items()}, rt)
 
 
 class DecoderModel:
@@ -98,7 +109,7 @@ class DecoderModel:
     # ------------------------------------------------------------ cache needs
     def cache_requests(self) -> Dict[int, object]:
         """cache entry -> what the mixer that writes it asks for."""
-        return {e.cache: self.blocks[e.block].mixer.cache_request()
+        return {e.cache: None if self.blocks[e.block].mixer is None else self.blocks[e.block].mixer.cache_request()
                 for e in self.spec.schedule if e.writes_cache}
 
     def prepare(self, max_len: int) -> None:
@@ -115,7 +126,7 @@ class DecoderModel:
             raise RuntimeError("model has no weights yet")
         s = self.spec
         h = torch.empty((ctx.n_tokens, s.hidden_size), dtype=torch.float32, device=self.rt.device)
-        self.embedding.forward(ctx.token_ids, h)
+        self.embedding.forward(ctx.token_ids, h, ctx)
         rows = ctx.logit_rows
         last = len(s.schedule) - 1
         for n, e in enumerate(s.schedule):
@@ -125,7 +136,7 @@ class DecoderModel:
             kept = torch.empty((rows.numel(), s.hidden_size), dtype=torch.float32, device=h.device)
             ops.gather_rows(h, rows, kept)
             h = kept
-        return self.head.forward(normed_input(self.final_norm, self.head, h))
+        return self.head.forward(normed_input(self.final_norm, self.head, h), ctx)
 
 
 def expected_tensors(spec: ModelSpec) -> Dict[str, TensorSpec]:

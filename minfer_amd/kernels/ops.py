@@ -171,42 +171,93 @@ def _is_bf16(t: torch.Tensor) -> int:
 _FLOATS = (torch.float32, torch.bfloat16)
 
 # ------------------------------------------------------------------ workspaces
+# Scratch buffers are shared by all callers and replaced by larger ones on demand.  A captured
+# graph holds the addresses of the buffers that were current when it was captured, so an outgrown
+# buffer must stay allocated while such a graph may still be replayed.  One rule, kept here: whoever
+# captures ops calls takes a `GraphLease` right after the capture and gives it back when the
+# graph is dropped (`lease_graph`, `release_graph`); a buffer that is replaced is kept while any
+# lease is older than its replacement, and freed otherwise.  `lease.stale()` tells an owner that
+# a buffer was replaced since its capture: it may capture again (and so let the old one go), or go
+# on replaying, which stays safe.
 _workspaces: Dict[Tuple[str, int], torch.Tensor] = {}
+_counters: Dict[Tuple[str, int], torch.Tensor] = {}
 _workspace_generation = 0
+_retired: list = []                  # (generation in which the buffer was last current, buffer)
+_leases: Dict[int, "GraphLease"] = {}
+_next_lease = 0
+
+
+def _device_index(device) -> int:
+    dev = torch.device(device)
+    if dev.type != "cuda":
+        return -1
+    return dev.index if dev.index is not None else torch.cuda.current_device()
+
+
+class GraphLease:
+    """Held by the owner of a captured graph for as long as the graph may be replayed."""
+
+    def __init__(self, token: int, generation: int):
+        self.token, self.generation = token, generation
+
+    def stale(self) -> bool:
+        """A buffer whose address the graph may hold has been replaced since the capture."""
+        return self.generation != _workspace_generation
+
+
+def lease_graph() -> GraphLease:
+    """To be called right after a capture that recorded ops calls."""
+    global _next_lease
+    _next_lease += 1
+    lease = _leases[_next_lease] = GraphLease(_next_lease, _workspace_generation)
+    return lease
+
+
+def release_graph(lease: Optional[GraphLease]) -> None:
+    """The graph is gone: buffers that only it could still address are freed."""
+    if lease is not None and _leases.pop(lease.token, None) is not None:
+        _drop_unreachable()
+
+
+def _drop_unreachable() -> None:
+    oldest = min((l.generation for l in _leases.values()), default=None)
+    _retired[:] = [(g, b) for g, b in _retired if oldest is not None and oldest <= g]
+
+
+def _retire(buffer: torch.Tensor) -> None:
+    """`buffer` is being replaced: the generation moves on, and the buffer stays allocated if a
+    leased graph was captured while it was current."""
+    global _workspace_generation
+    _retired.append((_workspace_generation, buffer))
+    _workspace_generation += 1
+    _drop_unreachable()
 
 
 def workspace(tag: str, n_floats: int, device) -> torch.Tensor:
-    """A float32 scratch tensor of at least n_floats, kept per (tag, device) and grown when
-    needed.  Kernels that use one run in stream order, so sharing it is safe.  When one grows,
-    the old tensor is given up and `workspace_generation()` moves on: a captured graph holds the
-    old address, so whoever keeps a graph compares the generation it captured under with the
-    current one and captures again when they differ (`DecodeSession` does)."""
-    global _workspace_generation
-    key = (tag, torch.device(device).index or 0)
+    """A float32 scratch tensor of at least n_floats, kept per (tag, device) and replaced by one at
+    least twice as large when it is outgrown.  Kernels that use one run in stream order, so sharing
+    it is safe."""
+    key = (tag, _device_index(device))
     w = _workspaces.get(key)
     if w is None or w.numel() < n_floats:
         if w is not None:
-            _workspace_generation += 1
+            _retire(w)
+            n_floats = max(n_floats, 2 * w.numel())
         w = torch.empty(max(n_floats, 1 << 16), dtype=torch.float32, device=device)
         _workspaces[key] = w
     return w
 
 
-_counters: Dict[Tuple[str, int], torch.Tensor] = {}
-
-
 def _zeroed_counters(tag: str, n: int, device) -> torch.Tensor:
     """int32 counters for kernels whose workgroups count themselves in and leave the counters at
-    zero again: zero when made, kept per (tag, device), made anew (and the generation moved on)
-    when more are needed."""
-    global _workspace_generation
-    dev = torch.device(device)
-    key = (tag, dev.index if dev.index is not None else torch.cuda.current_device())
+    zero again: zero when made, kept per (tag, device), replaced (see above) when more are needed."""
+    key = (tag, _device_index(device))
     c = _counters.get(key)
     if c is None or c.numel() < n:
         if c is not None:
-            _workspace_generation += 1
-        c = torch.zeros(max(n, 1024), dtype=torch.int32, device=dev)
+            _retire(c)
+            n = max(n, 2 * c.numel())
+        c = torch.zeros(max(n, 1024), dtype=torch.int32, device=torch.device(device))
         _counters[key] = c
     return c
 
@@ -215,11 +266,10 @@ def workspace_generation() -> int:
     return _workspace_generation
 
 
-def note_replaced_buffer() -> None:
+def note_replaced_buffer(old: Optional[torch.Tensor] = None) -> None:
     """For any other buffer whose address a captured graph may hold (a rotation table that was
-    rebuilt longer): moves the generation on, so that graphs are captured again."""
-    global _workspace_generation
-    _workspace_generation += 1
+    rebuilt longer): `old` is treated like an outgrown workspace."""
+    _retire(old if old is not None else torch.empty(0))
 
 
 # ------------------------------------------------------------------ element-wise
@@ -635,12 +685,13 @@ def _need_caches(what: str, kcache: torch.Tensor, vcache: torch.Tensor, dtype, n
 
 
 # Sequences that can be this long share their step's key splits by length: working the shares out
-# costs a block about a microsecond, which shorter ones do not gain back.
+# costs a block about a microsecond, which shorter ones do not gain back.  (This threshold, the cap
+# of four times the even share and the 32 places were tuned on an MI355X: 256 CUs in 8 dies.)
 SHARED_SPLITS_FROM = 8192
 
 
 def decode_split_plan(n_tok: int, n_kv_heads: int, group: int, max_len: int,
-                      target_blocks: int = 256) -> Tuple[int, int]:
+                      target_blocks: Optional[int] = None) -> Tuple[int, int]:
     """(places, splits) of the bfloat16 decode attention's key splits.  `splits`: about one block
     per CU, at least 256 keys of the longest possible sequence per split, at most 32.  A step of
     one token, of more than 64, of sequences that cannot be long, or without splits, gives every
@@ -649,6 +700,8 @@ def decode_split_plan(n_tok: int, n_kv_heads: int, group: int, max_len: int,
     at most `places` = 4 x splits (at most 32), so that a long sequence among short ones is cut
     finer and the blocks have about equal work.  The kernel divides a token's keys in rounds of
     128; a place without keys is marked empty and the merge passes it over."""
+    if target_blocks is None:
+        target_blocks = cu_count()
     blocks = n_tok * n_kv_heads * ((group + 15) // 16)
     splits = tuning.ATTN_SPLITS or max(1, min(target_blocks // max(1, blocks), (max_len + 255) // 256, 32))
     if n_tok == 1 or n_tok > 64 or splits == 1 or max_len < SHARED_SPLITS_FROM or tuning.ATTN_EQUAL_SPLITS:
@@ -746,14 +799,13 @@ def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pa
     if ctx.max_len > page_table.shape[1] * PAGE or page_table.shape[0] != ctx.n_seqs:
         raise KernelError(f"attention: page table {tuple(page_table.shape)} does not cover "
                           f"{ctx.n_seqs} sequences of up to {ctx.max_len} positions")
-    # The kernel's time is that of the block with the most pages (the last queries of the longest
-    # prompt): blocks of queries with more pages than a workgroup's even share of all of them (two
-    # workgroups fit a CU) are given to several workgroups, which take the pages in turn.
+    # Where the kernel's time is that of the block with the most pages (a few new tokens on a long
+    # context, few short prompts), blocks of queries with more pages than a workgroup's even share
+    # of all of them (two workgroups fit a CU) are given to several workgroups, which take the
+    # pages in turn.
     window = int(window or 0)
-    slots = 2 * cu_count()
     shared = None if tuning.NO_SHARED_PAGES else ctx.shared_query_tiles(
-        PREFILL_BLOCK, PAGE, window, lambda pages: max(PREFILL_MIN_PAGES, -(-pages * n_heads // slots)),
-        PREFILL_MAX_SHARES)
+        PREFILL_BLOCK, PAGE, window, n_heads, cu_count(), 2, PREFILL_MIN_PAGES, PREFILL_MAX_SHARES)
     if shared is None:
         tile_seq, tile_q0 = ctx.query_tiles(PREFILL_BLOCK)
         tile_share = parts = arrived = None
@@ -762,11 +814,14 @@ def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pa
         part = _fn("attn_prefill_bf16", "mf_attn_prefill_part_floats")(head_dim)
         parts = workspace("prefill_parts", n_slots * n_heads * most_shares * part, q.device)
         arrived = _zeroed_counters("prefill_arrived", n_slots * n_heads, q.device)
-    _check(_fn("attn_prefill_bf16", "mf_attn_prefill_bf16")(
+    rc = _fn("attn_prefill_bf16", "mf_attn_prefill_bf16")(
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(ctx.cu_seqlens),
         _ptr(ctx.start_pos), _ptr(tile_seq), _ptr(tile_q0), _ptr(tile_share), _ptr(parts), _ptr(arrived),
         most_shares if shared is not None else 1, _ptr(out), tile_seq.numel(), n_heads, n_kv_heads, head_dim, float(scale), window,
-        _stream()), "attn_prefill_bf16")
+        _stream())
+    if rc != 0 and arrived is not None:
+        arrived.zero_()                  # a launch that failed may have left workgroups counted in
+    _check(rc, "attn_prefill_bf16")
 
 
 # ------------------------------------------------------------------ sampling

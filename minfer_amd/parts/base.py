@@ -140,8 +140,10 @@ class FeedForward(Part):
 class Embedding(Part):
     """Token ids in, rows of the 32-bit residual stream out."""
 
-    def forward(self, token_ids: torch.Tensor, out: torch.Tensor) -> None:
-        """Writes the row of every id (int32 on the device) into `out` (float32 `[tokens][hidden]`)."""
+    def forward(self, token_ids: torch.Tensor, out: torch.Tensor, ctx) -> None:
+        """Writes the row of every id (int32 on the device) into `out` (float32 `[tokens][hidden]`).
+        `ctx` is the step (positions, sequences), for an embedding that depends on where a token
+        stands."""
         raise NotImplementedError
 
     def table(self) -> Optional[torch.Tensor]:
@@ -155,26 +157,44 @@ class Head(Part):
     def tie(self, embedding: "Embedding") -> None:
         """Called once after loading when the head shares the embedding's storage."""
 
-    def forward(self, x) -> torch.Tensor:
-        """`x`: the final norm's rows, as a tensor or (when `takes_normed`) a `Normed`.
-        Returns float32 `[rows][vocab]`."""
+    def forward(self, x, ctx) -> torch.Tensor:
+        """`x`: the final norm's rows, as a tensor or (when `takes_normed`) a `Normed`: the step's
+        rows `ctx.logit_rows` (all of them when that is None), in that order.  Returns float32
+        `[rows][vocab]`."""
         raise NotImplementedError
 
     takes_normed = False
 
 
 class Block:
-    """An arrangement of parts.  `forward` returns the residual stream, reduced to the rows
+    """An arrangement of parts: a mixer and a feed-forward (either may be None where the
+    arrangement allows it) and norms under the names the arrangement gives them (`norm_names`;
+    `optional_norms` may be left out).  `forward` returns the residual stream, reduced to the rows
     `keep_rows` (int32 indices on the device) when given."""
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
-                 feed_forward_norm: Norm, rt: Runtime):
+    norm_names = ("mixer", "feed_forward")
+    optional_norms = ()
+    needs_mixer = True
+    needs_feed_forward = True
+
+    def __init__(self, mixer: Optional[Mixer], feed_forward: Optional[FeedForward], norms: Dict[str, Norm],
+                 rt: Runtime):
         self.mixer, self.feed_forward = mixer, feed_forward
-        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+        self.norms = dict(norms)
         self.rt = rt
 
+    @property
+    def mixer_norm(self) -> Optional[Norm]:
+        return self.norms.get("mixer")
+
+    @property
+    def feed_forward_norm(self) -> Optional[Norm]:
+        return self.norms.get("feed_forward")
+
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
+        """Every part of the block that exists, norms in the order of `norm_names`."""
+        named = [self.norms[n] for n in self.norm_names + self.optional_norms if n in self.norms]
+        return tuple(p for p in [self.mixer, self.feed_forward] + named if p is not None)
 
     def forward(self, h, ctx, entry: int, writes_cache: bool, keep_rows=None):
         raise NotImplementedError

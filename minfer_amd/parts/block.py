@@ -13,13 +13,29 @@ from .base import Block, normed_input, register_block
 
 @register_block("prenorm")
 class PreNormBlock(Block):
+    """norms: "mixer" before the mixer, "feed_forward" before the feed-forward.  A block without a
+    mixer or without a feed-forward (and then without that branch's norm) is that branch left out."""
+
+    needs_mixer = False
+    needs_feed_forward = False
+    norm_names = ()
+    optional_norms = ("mixer", "feed_forward")
+
+    def __init__(self, mixer, feed_forward, norms, rt):
+        super().__init__(mixer, feed_forward, norms, rt)
+        for part, name in ((mixer, "mixer"), (feed_forward, "feed_forward")):
+            if (part is None) != (name not in self.norms):
+                raise ValueError(f"prenorm block: the {name} and the norm before it come together or not at all")
+
     def forward(self, h, ctx, entry: int, writes_cache: bool, keep_rows=None):
-        x = normed_input(self.mixer_norm, self.mixer, h)
-        self.mixer.forward(x, h, ctx, entry, writes_cache)
+        if self.mixer is not None:
+            x = normed_input(self.mixer_norm, self.mixer, h)
+            self.mixer.forward(x, h, ctx, entry, writes_cache)
         if keep_rows is not None:
             kept = torch.empty((keep_rows.numel(), h.shape[1]), dtype=h.dtype, device=h.device)
             ops.gather_rows(h, keep_rows, kept)
             h = kept
-        x = normed_input(self.feed_forward_norm, self.feed_forward, h)
-        self.feed_forward.forward(x, h, ctx)
+        if self.feed_forward is not None:
+            x = normed_input(self.feed_forward_norm, self.feed_forward, h)
+            self.feed_forward.forward(x, h, ctx)
         return h

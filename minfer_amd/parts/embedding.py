@@ -32,7 +32,7 @@ class TokenEmbedding(Embedding):
     def table(self):
         return self.weight
 
-    def forward(self, token_ids, out) -> None:
+    def forward(self, token_ids, out, ctx=None) -> None:
         ops.embed(self.weight, token_ids, out)
 
 
@@ -69,5 +69,5 @@ class LinearHead(Head):
     def decode_copies(self, make: bool, min_row_length: int = 0) -> int:
         return self.linear.decode_copy(make, min_row_length)
 
-    def forward(self, x) -> torch.Tensor:
+    def forward(self, x, ctx=None) -> torch.Tensor:
         return self.linear(x, out_dtype=torch.float32)

@@ -37,7 +37,8 @@ class RotaryNeoX(PositionEncoding):
             n = min(self.max_positions, max(FIRST_TABLE, 1 << (max_len - 1).bit_length()))
             if self.cos is not None:
                 self.generation += 1
-                ops.note_replaced_buffer()
+                ops.note_replaced_buffer(self.cos)
+                ops.note_replaced_buffer(self.sin)
             self.cos, self.sin = ops.rope_table(n, self.head_dim // 2, self.theta, self.freq_scale,
                                                 self.rt.device)
 

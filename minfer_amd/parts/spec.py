@@ -13,7 +13,7 @@ src/graph/builder.rs:79-286 of yusiwen/minfer) inside one loop over layers
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, Optional, Tuple
+from typing import Any, Dict, Mapping, Optional, Tuple
 
 
 @dataclass(frozen=True)
@@ -28,14 +28,30 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class BlockSpec:
-    """One block: the arrangement (`kind`, e.g. pre-norm residual) and its four parts.
-    `prefix` is put before every tensor name of the block's parts."""
+    """One block: the arrangement (`kind`, e.g. pre-norm residual), its mixer and feed-forward
+    (either may be absent) and its norms by the names the arrangement gives them.  `prefix` is
+    put before every tensor name of the block's parts.  `mixer_norm` and `feed_forward_norm` are
+    short for the norms named "mixer" and "feed_forward", the two that a pre-norm block has; an
+    arrangement with others (a norm after each branch as well, one norm shared by two parallel
+    branches) names them in `norms`."""
     kind: str
     prefix: str
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    mixer: Optional[PartSpec] = None
+    feed_forward: Optional[PartSpec] = None
+    mixer_norm: Optional[PartSpec] = None
+    feed_forward_norm: Optional[PartSpec] = None
+    norms: Mapping[str, PartSpec] = field(default_factory=dict)
+
+    def __post_init__(self):
+        norms = dict(self.norms)
+        for name, short in (("mixer", self.mixer_norm), ("feed_forward", self.feed_forward_norm)):
+            if short is not None:
+                if name in norms and norms[name] != short:
+                    raise ValueError(f"block {self.prefix!r}: the norm {name!r} is given twice")
+                norms[name] = short
+        object.__setattr__(self, "norms", norms)
+        object.__setattr__(self, "mixer_norm", norms.get("mixer"))
+        object.__setattr__(self, "feed_forward_norm", norms.get("feed_forward"))
 
 
 @dataclass(frozen=True)

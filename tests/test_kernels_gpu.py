@@ -549,8 +549,7 @@ def test_attn_prefill_shared_pages(ops, nh, nk, hd, window):
     one adds up (one sequence continues from 600 cached tokens; the short one stays whole)."""
     new, start = [1500, 260, 40], [600, 0, 0]
     q, kc, vc, table, ctx_on = prefill_case(nh, nk, hd, new, start, 23)
-    shared = ctx_on("cpu").shared_query_tiles(ops.PREFILL_BLOCK, ops.PAGE, window,
-                                              lambda pages: max(ops.PREFILL_MIN_PAGES, -(-pages * nh // 512)),
+    shared = ctx_on("cpu").shared_query_tiles(ops.PREFILL_BLOCK, ops.PAGE, window, nh, 256, 2, ops.PREFILL_MIN_PAGES,
                                               ops.PREFILL_MAX_SHARES)
     assert shared is not None
     words = shared[2].tolist()

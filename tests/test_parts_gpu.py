@@ -471,7 +471,7 @@ class ToyScaledEmbedding(Embedding):
     def table(self):
         return self.weight
 
-    def forward(self, token_ids, out):
+    def forward(self, token_ids, out, ctx):
         out.copy_(self.weight[token_ids.long()] * self.scale)
 
 
@@ -492,7 +492,7 @@ class ToyCappedHead(Head):
     def tie(self, embedding):
         self.w = embedding.table()
 
-    def forward(self, x):
+    def forward(self, x, ctx):
         return (self.cap * torch.tanh((x.float() @ self.w.t() + self.bias) / self.cap)).contiguous()
 
 
@@ -539,3 +539,158 @@ def test_other_embedding_and_head_parts_without_touching_the_model(tmp_path):
     ref = {r: plain(t) for r, t in requests.items()}
     compare(run_steps(eng, whole_steps(requests)), ref, "float32", "toy ends whole")
     compare(run_steps(eng, tail_steps(requests, tail=5)), ref, "float32", "toy ends one by one")
+
+
+# ------------------------------------------------------------------ other arrangements, and ends that know the positions
+@register_block("toy_sandwich")
+class ToySandwichBlock(Block):
+    """Four norms: h += post(mixer(pre(h))); h += post(feed_forward(pre(h))).  The branch's output
+    is collected in a buffer of its own, normed, and only then added to the stream."""
+
+    norm_names = ("mixer", "mixer_post", "feed_forward", "feed_forward_post")
+
+    def forward(self, h, ctx, entry, writes_cache, keep_rows=None):
+        branch = torch.zeros_like(h)
+        self.mixer.forward(self.norms["mixer"].forward(h), branch, ctx, entry, writes_cache)
+        h += self.norms["mixer_post"].forward(branch).float()
+        if keep_rows is not None:
+            h = h[keep_rows.long()].contiguous()
+        branch = torch.zeros_like(h)
+        self.feed_forward.forward(self.norms["feed_forward"].forward(h), branch, ctx)
+        h += self.norms["feed_forward_post"].forward(branch).float()
+        return h
+
+
+@register_embedding("toy_positional_embedding")
+class ToyPositionalEmbedding(Embedding):
+    """Learned absolute positions: row of the token table plus row of a position table, which
+    only the step's context can tell."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.vocab, self.hidden, self.n_pos = (int(spec.params[k]) for k in ("vocab_size", "hidden_size", "positions"))
+
+    def tensor_specs(self):
+        return {"emb": TensorSpec((self.vocab, self.hidden)), "pos_emb": TensorSpec((self.n_pos, self.hidden))}
+
+    def load(self, get):
+        self.weight, self.pos = get("emb").float(), get("pos_emb").float()
+
+    def forward(self, token_ids, out, ctx):
+        out.copy_(self.weight[token_ids.long()] + self.pos[ctx.positions.long()])
+
+
+@register_head("toy_position_head")
+class ToyPositionHead(Head):
+    """logits = W x + slope * (position of the row): the head asks the context which rows it got."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.vocab, self.hidden, self.slope = int(spec.params["vocab_size"]), int(spec.params["hidden_size"]), float(spec.params["slope"])
+
+    def tensor_specs(self):
+        return {"head": TensorSpec((self.vocab, self.hidden))}
+
+    def load(self, get):
+        self.w = get("head").float()
+
+    def forward(self, x, ctx):
+        pos = ctx.positions if ctx.logit_rows is None else ctx.positions[ctx.logit_rows.long()]
+        return (x.float() @ self.w.t() + self.slope * pos.float()[:, None]).contiguous()
+
+
+class ToySandwichConfig(ToyConfig):
+    """Block 0: four norms around attention and SwiGLU.  Block 1: a pre-norm block that has a mixer
+    and no feed-forward.  Block 2: a pre-norm block that has a feed-forward and no mixer."""
+
+    def model_spec(self):
+        hid = self.hidden
+        norm = lambda n: PartSpec("rmsnorm", dict(size=hid, eps=1e-5, weight=n))
+        pos = PartSpec("rope_neox", dict(head_dim=16, theta=1e4, max_positions=256))
+        attn = PartSpec("gqa_attention", dict(hidden_size=hid, n_heads=4, n_kv_heads=2, head_dim=16, scale=0.25, window=None,
+                                              qkv_bias=True, out_bias=False, position=pos, q="a.q", k="a.k", v="a.v", o="a.o"))
+        ffn = PartSpec("swiglu", dict(hidden_size=hid, intermediate_size=72, gate="f.g", up="f.u", down="f.d"))
+        sizes = dict(vocab_size=self.vocab, hidden_size=hid)
+        blocks = (BlockSpec("toy_sandwich", "l0.", attn, ffn, norms={"mixer": norm("n1"), "mixer_post": norm("n2"),
+                                                                     "feed_forward": norm("n3"), "feed_forward_post": norm("n4")}),
+                  BlockSpec("prenorm", "l1.", mixer=attn, mixer_norm=norm("n1")),
+                  BlockSpec("prenorm", "l2.", feed_forward=ffn, feed_forward_norm=norm("n2")))
+        return ModelSpec(hidden_size=hid, vocab_size=self.vocab, final_norm=norm("nf"), blocks=blocks,
+                         schedule=(RunEntry(0, 0), RunEntry(1, 1), RunEntry(2, 2)), max_positions=256,
+                         embedding=PartSpec("toy_positional_embedding", dict(sizes, positions=256)),
+                         head=PartSpec("toy_position_head", dict(sizes, slope=0.002)))
+
+    def random_init_std(self, name):
+        return 0.3 if name in ("emb", "pos_emb") else 0.08
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_four_norm_block_blocks_without_a_branch_and_ends_that_see_positions(tmp_path, dtype):
+    """Registered from here alone: a block of four norms, pre-norm blocks that lack a feed-forward
+    or a mixer, an embedding with learned absolute positions and a head that adds a term of the
+    row's position (both get the step's context).  Whole, one by one and in unequal batches
+    against a plain version written out below."""
+    from minfer_amd import Engine, load_model, register_architecture, write_random_model
+    from safetensors.torch import load_file
+    register_architecture("ToySandwichLM", ToySandwichConfig)
+    cfg = ToySandwichConfig(dict(architectures=["ToySandwichLM"], hidden_size=64, vocab_size=190))
+    folder = write_random_model(str(tmp_path / "sandwich"), cfg, seed=13)
+    model = load_model(folder, dtype=dtype)
+    names = set(model.expected_tensors())
+    assert {"l0.n4", "l1.n1", "l2.n2", "pos_emb", "head"} <= names and "l1.n2" not in names and "l1.f.g.weight" not in names
+    assert "l2.a.q.weight" not in names
+    assert model.blocks[1].feed_forward is None and model.blocks[2].mixer is None
+    assert model.cache_requests()[2] is None and isinstance(model.cache_requests()[1], KVRequest)
+    w = {k: v.double().numpy() for k, v in load_file(folder + "/model.safetensors").items()}
+
+    def attention(p, x, pos):
+        q = pq.rope_neox(pq.linear(x, w[p + "a.q.weight"], w[p + "a.q.bias"]), pos, 4, 16, 1e4)
+        k = pq.rope_neox(pq.linear(x, w[p + "a.k.weight"], w[p + "a.k.bias"]), pos, 2, 16, 1e4)
+        a = pq.gqa_attention(q, k, pq.linear(x, w[p + "a.v.weight"], w[p + "a.v.bias"]), pos, pos, 4, 2, 16, 0.25)
+        return pq.linear(a, w[p + "a.o.weight"])
+
+    def ffn(p, x):
+        return pq.swiglu_ffn(x, w[p + "f.g.weight"], w[p + "f.u.weight"], w[p + "f.d.weight"])
+
+    def plain(tokens):
+        pos = np.arange(len(tokens))
+        n = lambda x, name: pq.rms_norm(x, w[name], 1e-5)
+        h = w["emb"][tokens] + w["pos_emb"][pos]
+        h = h + n(attention("l0.", n(h, "l0.n1"), pos), "l0.n2")
+        h = h + n(ffn("l0.", n(h, "l0.n3")), "l0.n4")
+        h = h + attention("l1.", n(h, "l1.n1"), pos)
+        h = h + ffn("l2.", n(h, "l2.n2"))
+        return n(h, "nf") @ w["head"].T + 0.002 * pos[:, None]
+    eng = Engine(model, max_tokens=64 * 6, max_seqs=3, poison_cache=True)
+    requests = requests_for(190, (9, 70, 3, 31), seed=4)
+    ref = {r: plain(t) for r, t in requests.items()}
+    ids = list(requests)
+    compare(run_steps(eng, whole_steps(requests)), ref, dtype, "sandwich whole", layers=3)
+    compare(run_steps(eng, tail_steps(requests, tail=6)), ref, dtype, "sandwich one by one", layers=3)
+    compare(run_steps(eng, batch_steps(requests, [ids[:3], ids[3:]])), ref, dtype, "sandwich batches", layers=3)
+    # "last" rows only: the head is told which rows it got
+    s = eng.new_sequence()
+    last = eng.step([s], [requests["r1"]], "last").cpu().numpy()
+    eng.end_sequence(s)
+    tol = 1e-4 if dtype == "float32" else 0.055 * 2 * float(ref["r1"][-1].std())
+    assert np.abs(last[0] - ref["r1"][-1]).max() < tol
+
+
+def test_block_specs_are_checked_against_their_arrangement():
+    """A spec that leaves out a norm its arrangement needs, names one it does not know, or lacks
+    the mixer of an arrangement that needs one is refused with the block's name."""
+    from minfer_amd.engine.model import _build_block
+    rt = Runtime(torch.float32, torch.device("cpu"))
+    norm = lambda n: PartSpec("rmsnorm", dict(size=8, eps=1e-5, weight=n))
+    ffn = PartSpec("swiglu", dict(hidden_size=8, intermediate_size=8, gate="g", up="u", down="d"))
+    with pytest.raises(ValueError, match="l7.*norms missing.*mixer_post"):
+        _build_block(BlockSpec("toy_sandwich", "l7.", ffn, ffn, norms={"mixer": norm("a"), "feed_forward": norm("b"),
+                                                                      "feed_forward_post": norm("c")}), rt)
+    with pytest.raises(ValueError, match="not known to the arrangement \\['extra'\\]"):
+        _build_block(BlockSpec("prenorm", "l0.", feed_forward=ffn, feed_forward_norm=norm("b"), norms={"extra": norm("x")}), rt)
+    with pytest.raises(ValueError, match="needs a mixer"):
+        _build_block(BlockSpec("toy_sandwich", "l1.", None, ffn), rt)
+    with pytest.raises(ValueError, match="come together"):
+        _build_block(BlockSpec("prenorm", "l2.", feed_forward=ffn), rt)
+    with pytest.raises(ValueError, match="given twice"):
+        BlockSpec("prenorm", "l3.", feed_forward=ffn, feed_forward_norm=norm("a"), norms={"feed_forward": norm("b")})

@@ -70,13 +70,15 @@ def test_split_plan_of_the_32_bit_attention():
 
 def test_decode_split_plan_bounds():
     for n_tok, nk, group, max_len in itertools.product((1, 8, 64, 300), (1, 2, 4), (1, 5, 7, 17), (1, 64, 4096, 32768)):
-        places, n = ops.decode_split_plan(n_tok, nk, group, max_len)
+        places, n = ops.decode_split_plan(n_tok, nk, group, max_len, target_blocks=256)
         assert 1 <= n <= places <= 32
         assert n == 1 or n * 256 <= max_len + 255
         assert places == n or (1 < n_tok <= 64 and n > 1 and max_len >= 8192 and places == min(4 * n, 32))
-    assert ops.decode_split_plan(1, 4, 7, 32768) == (32, 32) and ops.decode_split_plan(64, 4, 7, 32768) == (1, 1)
-    assert ops.decode_split_plan(8, 4, 7, 32768) == (32, 8)          # shares in proportion to the keys
-    assert ops.decode_split_plan(8, 4, 7, 4096) == (8, 8)
+    plan = lambda *a: ops.decode_split_plan(*a, target_blocks=256)
+    assert plan(1, 4, 7, 32768) == (32, 32) and plan(64, 4, 7, 32768) == (1, 1)
+    assert plan(8, 4, 7, 32768) == (32, 8)          # shares in proportion to the keys
+    assert plan(8, 4, 7, 4096) == (8, 8)
+    assert ops.decode_split_plan(8, 4, 7, 4096, target_blocks=64) == (2, 2)        # a chip of 64 CUs splits less
 
 
 def test_plan_linear_names_the_kernels_of_the_model_shapes():
@@ -136,7 +138,7 @@ def test_shared_query_tiles_cover_every_page_once():
 
     for new, start, window, load, cap in (([1500, 260, 40], [600, 0, 0], 0, 4, 8), ([64], [30000], 0, 26, 8),
                                           ([2048], [0], 0, 15, 8), ([300, 17], [900, 5000], 700, 4, 3)):
-        got = ctx(new, start).shared_query_tiles(128, 64, window, lambda pages: load, cap)
+        got = ctx(new, start).shared_query_tiles(128, 64, window, 1, 1 << 19, 2, load, cap)      # the least load binds
         assert got is not None
         seqs, q0s, words, n_slots, most = (x.tolist() if hasattr(x, "tolist") else x for x in got)
         tiles = {}
@@ -157,4 +159,18 @@ def test_shared_query_tiles_cover_every_page_once():
             assert n == cap or -(-pages // n) <= load
             slots.add(ws[0] >> 16)
         assert slots == set(range(n_slots))
-    assert ctx([100, 30], [0, 0]).shared_query_tiles(128, 64, 0, lambda pages: 4, 8) is None
+    assert ctx([100, 30], [0, 0]).shared_query_tiles(128, 64, 0, 1, 1 << 19, 2, 4, 8) is None
+    # the even share binds: 64 tokens on 30,000 are 470 pages; 28 heads over 512 workgroups at once
+    # give each at most 26 of them, 4 heads give each at most 4: layers with other head counts get
+    # plans of their own from the same step
+    c = ctx([64], [30000])
+    a = c.shared_query_tiles(128, 64, 0, 28, 256, 2, 4, 64)
+    b = c.shared_query_tiles(128, 64, 0, 4, 256, 2, 4, 64)
+    assert a[4] == -(-470 // 26) and b[4] == 64 and c.shared_query_tiles(128, 64, 0, 28, 256, 2, 4, 64) is a
+    # no sharing where it cannot gain: a whole prompt of 2,048 tokens with 28 heads keeps every CU
+    # busy for as long as its longest block takes (32 pages against an even 30 a CU); with 2 heads
+    # the CUs would idle behind the longest blocks
+    assert ctx([2048], [0]).shared_query_tiles(128, 64, 0, 28, 256, 2, 4, 8) is None
+    assert ctx([2048], [0]).shared_query_tiles(128, 64, 0, 2, 256, 2, 4, 8) is not None
+    assert ctx([128] * 8, [2000] * 8).shared_query_tiles(128, 64, 0, 28, 256, 2, 4, 8) is None
+    assert ctx([512], [4096]).shared_query_tiles(128, 64, 0, 28, 256, 2, 4, 8) is not None
