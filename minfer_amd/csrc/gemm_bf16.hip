@@ -1324,6 +1324,53 @@ int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const fl
   return mf_launch_status();
 }
 
+// The RMS norm folded around the products of 17 to 64 rows, across two kernels (y = x /
+// sqrt(mean(x^2) + eps) * g, src/vec_ops.rs:500-522):
+//  * a product that adds into the residual stream x and knows the weight g of the norm that reads
+//    the stream next leaves, beside the stream's new rows, xg = bf16(x g) and for every row the
+//    sums of x^2 over runs of 256 columns (`out_*`; the kernel that adds the parts of a K split
+//    does it: it has every new value of x in its hands);
+//  * the product that follows takes xg as its activations and multiplies its own sums by the
+//    row's 1 / sqrt(sum / K + eps) in its epilogue (`in_*`), the partial sums of squares added up
+//    in their order.
+// No norm kernel, no pass over the stream between the two products.  The same arithmetic as the
+// fold of the register-resident kernel above (bf16(x g) to the matrix cores, the row's factor in
+// the epilogue).
+constexpr int MF_NOT_BUILT = -2;     // an entry point's answer for a shape it has no kernel for; nothing was launched
+
+struct FusedNorm {
+  const float* in_ssq;     // [M][in_parts] partial sums of squares of the rows this product reads (null: none)
+  int in_parts;
+  float in_eps;
+  const float* out_g;      // [N] weight of the norm that reads the output next (null: none)
+  bf16* out_xg;            // [M][N]
+  float* out_ssq;          // [M][ceil(N / 256)]
+};
+
+// 1 / sqrt(mean(x^2) + eps) of NR rows from their partial sums, K the rows' length, in two steps
+// so that a kernel can ask for the sums early and use them late; all lanes of a wave call both with
+// the same rows (a row outside [0, M) gives 1).  The lanes take the partial sums between them, all
+// rows' loads in flight together, and add up in a fixed tree.
+template <int NR>
+__device__ __forceinline__ void row_sums_ask(const FusedNorm& f, const int (&rows)[NR], int M, int lane, float (&t)[NR]) {
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    t[i] = 0.f;
+    if (rows[i] >= 0 && rows[i] < M)
+      for (int p = lane; p < f.in_parts; p += 64) t[i] += f.in_ssq[(size_t)rows[i] * f.in_parts + p];
+  }
+}
+
+template <int NR>
+__device__ __forceinline__ void row_factors_of(const FusedNorm& f, const int (&rows)[NR], int M, int K, float (&t)[NR]) {
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) t[i] += __shfl_xor(t[i], o, MF_WAVE);
+    t[i] = (rows[i] >= 0 && rows[i] < M) ? 1.0f / sqrtf(t[i] / (float)K + f.in_eps) : 1.f;
+  }
+}
+
 // 17 to 64 rows against a wide matrix (at least 8 tiles of 16 weight rows for every CU): one block
 // per CU with an equal share of the matrix, the whole of K, no partial sums between blocks and no
 // second kernel.  The share is cut into passes of at most 16 tiles; wave w multiplies tiles w and
@@ -1346,12 +1393,15 @@ template <int MT, bool TILED>
 __global__ __launch_bounds__(512) void panel_kernel(const bf16* __restrict__ A, int lda,
                                                     const bf16* __restrict__ W, int ldw,
                                                     const float* __restrict__ bias, void* __restrict__ C,
-                                                    int ldc, int M, int N, int K, int units_total, int epi) {
+                                                    int ldc, int M, int N, int K, int units_total, int epi,
+                                                    FusedNorm fused) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   constexpr int ROWS = MT * 16;
   bf16* As = reinterpret_cast<bf16*>(smem);                                            // [2][ROWS][SK_LD]
   float* ot = reinterpret_cast<float*>(smem + 2 * ROWS * SK_LD * sizeof(bf16));        // [ROWS][OT_LD]
+  __shared__ float rfac[ROWS];                 // the rows' norm factors (1 where no norm is folded in)
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+
   const int r16 = lane & 15, kq = (lane >> 4) * 8;
   constexpr int WSTEP = TILED ? 512 : 32;
   const bool pair = epi == EPI_SWIGLU;
@@ -1392,12 +1442,26 @@ __global__ __launch_bounds__(512) void panel_kernel(const bf16* __restrict__ A, 
   const bf16* wp[2] = {slot_ptr(0, 0), slot_ptr(0, 1)};
   bf16x8 wr[2][KC / 32];
   load_stage(0);
+  // the rows' norm factors: wave w has rows w, w + 8, ...  Their partial sums are asked for between
+  // the first activations and the first weights and used behind the activations' staging, so that
+  // nothing the weight stream needs waits for them.
+  int frow[2 * MT];
+  float ffac[2 * MT];
+#pragma unroll
+  for (int i = 0; i < 2 * MT; ++i) frow[i] = fused.in_ssq ? wid + 8 * i : -1;
+  row_sums_ask<2 * MT>(fused, frow, M, lane, ffac);
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int s = 0; s < KC / 32; ++s) {
     wr[0][s] = *reinterpret_cast<const bf16x8*>(wp[0] + s * WSTEP);
     wr[1][s] = *reinterpret_cast<const bf16x8*>(wp[1] + s * WSTEP);
   }
+  __builtin_amdgcn_sched_barrier(0);
   store_stage(0);
+  row_factors_of<2 * MT>(fused, frow, M, K, ffac);
+  if (lane == 0)
+#pragma unroll
+    for (int i = 0; i < 2 * MT; ++i) rfac[wid + 8 * i] = ffac[i];
   __syncthreads();
   floatx4 acc[2][MT];
 #pragma unroll
@@ -1463,13 +1527,13 @@ __global__ __launch_bounds__(512) void panel_kernel(const bf16* __restrict__ A, 
         if (c < cnt * 8 && col < ldc) {
           const int o = (c >> 4) * 32 + (c & 15);
           for (int m = tid >> 8; m < M; m += 2)
-            ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(ot[m * OT_LD + o], ot[m * OT_LD + o + 16]);
+            ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(ot[m * OT_LD + o] * rfac[m], ot[m * OT_LD + o + 16] * rfac[m]);
         }
       } else {
         const int col = u0 * 32 + c;
         if (c < cnt * 16 && col < N) {
           const float b = bias ? bias[col] : 0.f;
-          for (int m = tid >> 8; m < M; m += 2) store_out(C, ldc, m, col, ot[m * OT_LD + c] + b, epi);
+          for (int m = tid >> 8; m < M; m += 2) store_out(C, ldc, m, col, ot[m * OT_LD + c] * rfac[m] + b, epi);
         }
       }
     }
@@ -1513,27 +1577,52 @@ __device__ __forceinline__ float sum_of_parts(const float* __restrict__ part, si
 
 __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restrict__ part,
                                                             const float* __restrict__ bias,
-                                                            void* __restrict__ C, int ldc, int M, int N,
-                                                            int splits, int epi) {
+                                                            void* __restrict__ C, int ldc, int M, int N, int K,
+                                                            int splits, int epi, FusedNorm fused) {
   const int n = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
   const size_t stride = (size_t)M * N;
+  const int frow[1] = {fused.in_ssq ? m : -1};
+  float ffac[1];
+  row_sums_ask<1>(fused, frow, M, threadIdx.x & 63, ffac);
+  row_factors_of<1>(fused, frow, M, K, ffac);
+  const float rf = ffac[0];
   if (epi == EPI_SWIGLU) {       // n runs over the ldc outputs
     if (n >= ldc) return;
     const int ng = (n >> 5) * 64 + (n & 31);
     const float g = sum_of_parts(part, stride, (size_t)m * N + ng, splits);
     const float u = sum_of_parts(part, stride, (size_t)m * N + ng + 32, splits);
-    ((bf16*)C)[(size_t)m * ldc + n] = (bf16)swiglu_f(g, u);
+    ((bf16*)C)[(size_t)m * ldc + n] = (bf16)swiglu_f(g * rf, u * rf);
     return;
   }
-  if (n >= N) return;
-  const float v = sum_of_parts(part, stride, (size_t)m * N + n, splits);
-  store_out(C, ldc, m, n, v + (bias ? bias[n] : 0.f), epi);
+  float v = 0.f;                 // the output's new value (0 beyond the row's end)
+  if (n < N) {
+    v = sum_of_parts(part, stride, (size_t)m * N + n, splits) * rf + (bias ? bias[n] : 0.f);
+    if (epi == EPI_BF16) {
+      ((bf16*)C)[(size_t)m * ldc + n] = (bf16)v;
+    } else {
+      float* c = (float*)C + (size_t)m * ldc + n;
+      if (epi == EPI_ACC_F32) v += *c;
+      *c = v;
+    }
+  }
+  if (fused.out_g) {
+    // for the norm that reads these rows next: bf16(x g), and this block's sum of x^2, the waves'
+    // sums added in their order
+    if (n < N) fused.out_xg[(size_t)m * N + n] = (bf16)(v * fused.out_g[n]);
+    __shared__ float wsum[4];
+    float sq = v * v;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, MF_WAVE);
+    if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = sq;
+    __syncthreads();
+    if (threadIdx.x == 0) fused.out_ssq[(size_t)m * gridDim.x + blockIdx.x] = ((wsum[0] + wsum[1]) + wsum[2]) + wsum[3];
+  }
 }
 
 template <int MT, bool VEC>
 int launch_skinny_v(const bf16* A, int lda, const bf16* W, const bf16* Wt, int ldw, const float* bias, void* C,
                     int ldc, float* part, int M, int N, int K, int splits, int k_per_split, int epi,
-                    hipStream_t stream) {
+                    const FusedNorm& fused, hipStream_t stream) {
   constexpr int smem = 2 * MT * 16 * SK_LD * (int)sizeof(bf16);
   static bool configured = false;
   const bool tiled = VEC && Wt != nullptr;
@@ -1549,6 +1638,7 @@ int launch_skinny_v(const bf16* A, int lda, const bf16* W, const bf16* Wt, int l
   }
   dim3 grid((N + 127) / 128, splits);
   const bool two_pass = splits > 1 || epi == EPI_SWIGLU;   // gate and up columns sit in different waves
+  if (!two_pass && (fused.in_ssq || fused.out_g)) return MF_NOT_BUILT;     // the second kernel is what folds the norm in
   if (ring_takes(VEC, K, splits, k_per_split)) {
     constexpr int smem_ring = smem + MT * 16 * SR_LD * (int)sizeof(float);
     static bool ring_configured = false;
@@ -1574,7 +1664,7 @@ int launch_skinny_v(const bf16* A, int lda, const bf16* W, const bf16* Wt, int l
   int rc = mf_launch_status();
   if (rc == 0 && two_pass) {
     dim3 g2(((epi == EPI_SWIGLU ? ldc : N) + 255) / 256, M);
-    skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, splits, epi);
+    skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, K, splits, epi, fused);
     rc = mf_launch_status();
   }
   return rc;
@@ -1583,19 +1673,18 @@ int launch_skinny_v(const bf16* A, int lda, const bf16* W, const bf16* Wt, int l
 template <int MT>
 int launch_skinny(const bf16* A, int lda, const bf16* W, const bf16* Wt, int ldw, const float* bias, void* C,
                   int ldc, float* part, int M, int N, int K, int splits, int k_per_split, int epi, int vec_ok,
-                  hipStream_t stream) {
+                  const FusedNorm& fused, hipStream_t stream) {
   return vec_ok ? launch_skinny_v<MT, true>(A, lda, W, Wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split,
-                                            epi, stream)
+                                            epi, fused, stream)
                 : launch_skinny_v<MT, false>(A, lda, W, nullptr, ldw, bias, C, ldc, part, M, N, K, splits,
-                                             k_per_split, epi, stream);
+                                             k_per_split, epi, fused, stream);
 }
 
 // The whole-K kernel for 17 to 64 rows, where the matrix is wide enough to give every CU at least
 // 8 tiles; MF_NOT_BUILT (nothing launched) for any other shape.
-constexpr int MF_NOT_BUILT = -2;
 template <int MT, bool TILED>
 int launch_panel_mt(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc, int M,
-                    int N, int K, int epi, int grid, int units, hipStream_t stream) {
+                    int N, int K, int epi, int grid, int units, const FusedNorm& fused, hipStream_t stream) {
   constexpr int smem = 2 * MT * 16 * SK_LD * (int)sizeof(bf16) + MT * 16 * OT_LD * (int)sizeof(float);
   static bool configured = false;
   if (!configured) {
@@ -1604,27 +1693,27 @@ int launch_panel_mt(const bf16* A, int lda, const bf16* W, int ldw, const float*
     if (e != hipSuccess) return (int)e;
     configured = true;
   }
-  panel_kernel<MT, TILED><<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, units, epi);
+  panel_kernel<MT, TILED><<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, units, epi, fused);
   return mf_launch_status();
 }
 
 int launch_panel(const bf16* A, int lda, const bf16* W, const bf16* Wt, int ldw, const float* bias, void* C, int ldc,
-                 int M, int N, int K, int epi, hipStream_t stream) {
+                 int M, int N, int K, int epi, const FusedNorm& fused, hipStream_t stream) {
   const int n_cu = cu_count();
   if (n_cu <= 0) return (int)hipErrorUnknown;
   const bool aligned = ldw % 8 == 0 && (uintptr_t)W % 16 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0;
-  if (!panel_takes(M, N, K, aligned, epi, n_cu)) return MF_NOT_BUILT;
+  if (!panel_takes(M, N, K, aligned, epi, n_cu) || fused.out_g) return MF_NOT_BUILT;
   const int units = (N + 31) / 32;
   switch ((M + 15) / 16) {
     case 2:
-      return Wt ? launch_panel_mt<2, true>(A, lda, Wt, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream)
-                : launch_panel_mt<2, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
+      return Wt ? launch_panel_mt<2, true>(A, lda, Wt, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, fused, stream)
+                : launch_panel_mt<2, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, fused, stream);
     case 3:
-      return Wt ? launch_panel_mt<3, true>(A, lda, Wt, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream)
-                : launch_panel_mt<3, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
+      return Wt ? launch_panel_mt<3, true>(A, lda, Wt, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, fused, stream)
+                : launch_panel_mt<3, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, fused, stream);
     case 4:
-      return Wt ? launch_panel_mt<4, true>(A, lda, Wt, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream)
-                : launch_panel_mt<4, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, stream);
+      return Wt ? launch_panel_mt<4, true>(A, lda, Wt, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, fused, stream)
+                : launch_panel_mt<4, false>(A, lda, W, ldw, bias, C, ldc, M, N, K, epi, n_cu, units, fused, stream);
   }
   return MF_NOT_BUILT;
 }
@@ -1791,7 +1880,7 @@ MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, c
                                                      N, K, EPI_F32, vec_ok, stream, splits, k_per_split);
   if (rc) return rc;
   dim3 g2(((epi == EPI_SWIGLU ? ldc : N) + 255) / 256, M);
-  skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, splits, epi);
+  skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, K, splits, epi, FusedNorm{});
   return mf_launch_status();
 }
 
@@ -1816,12 +1905,9 @@ static int stationary16(const void* a, int lda, const bf16* w, const bf16* wt, i
   return MF_NOT_BUILT;
 }
 
-// M <= 64.  `part` holds splits*M*N floats when splits > 1; k_per_split is a multiple of 256.
-// `Wt`: the tiled copy of W (see w_operand), or null; the kernels that have a form for it read it
-// instead of W.
-MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, const void* Wt, int ldw, const float* bias,
-                               void* C, int ldc, float* part, int M, int N, int K, int splits,
-                               int k_per_split, int epi, hipStream_t stream) {
+static int skinny_product(const void* A, int lda, const void* W, const void* Wt, int ldw, const float* bias,
+                          void* C, int ldc, float* part, int M, int N, int K, int splits, int k_per_split, int epi,
+                          const FusedNorm& fused, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || lda < K || ldw < K || epi < 0 || epi > 3 || splits < 1 ||
       k_per_split % KC != 0 || (long)splits * k_per_split < K || (splits > 1 && !part))
@@ -1834,7 +1920,9 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, const void
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   const bf16* wt = (K % 32 == 0 && (uintptr_t)Wt % 16 == 0) ? (const bf16*)Wt : nullptr;
+  const bool folds = fused.in_ssq || fused.out_g;
   const SkinnyChoice choice = skinny_choice(M, N, K, vec_ok, epi, splits, k_per_split, cu_count());
+  if (folds && M <= 16 && choice != SK_RING && choice != SK_STAGED) return MF_NOT_BUILT;
   switch (choice) {
     case SK_STATIONARY: return stationary16(a, lda, w, wt, ldw, bias, C, ldc, M, N, K, epi, nullptr, stream);
     case SK_ROLLING:
@@ -1844,16 +1932,43 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, const void
     case SK_GUARDED_4X2: return launch_skinny16<4, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case SK_GUARDED_8X2: return launch_skinny16<8, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case SK_GUARDED_8X1: return launch_skinny16<8, 1, 8>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
-    case SK_PANEL: return launch_panel(a, lda, w, wt, ldw, bias, C, ldc, M, N, K, epi, stream);
+    case SK_PANEL: return launch_panel(a, lda, w, wt, ldw, bias, C, ldc, M, N, K, epi, fused, stream);
     default: break;
   }
   switch ((M + 15) / 16) {
-    case 1: return launch_skinny<1>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
-    case 2: return launch_skinny<2>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
-    case 3: return launch_skinny<3>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
-    case 4: return launch_skinny<4>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, stream);
+    case 1: return launch_skinny<1>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, fused, stream);
+    case 2: return launch_skinny<2>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, fused, stream);
+    case 3: return launch_skinny<3>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, fused, stream);
+    case 4: return launch_skinny<4>(a, lda, w, wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, vec_ok, fused, stream);
   }
   return (int)hipErrorInvalidValue;
+}
+
+// M <= 64.  `part` holds splits*M*N floats when splits > 1; k_per_split is a multiple of 256.
+// `Wt`: the tiled copy of W (see w_operand), or null; the kernels that have a form for it read it
+// instead of W.
+MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, const void* Wt, int ldw, const float* bias,
+                               void* C, int ldc, float* part, int M, int N, int K, int splits,
+                               int k_per_split, int epi, hipStream_t stream) {
+  return skinny_product(A, lda, W, Wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, FusedNorm{}, stream);
+}
+
+// The same with an RMS norm folded in on either side (see FusedNorm), for the shapes whose kernels
+// have a place for it (17 to 64 rows: the whole-K kernel on the reading side, the K-split kernels
+// with more than one split on both); MF_NOT_BUILT (-2), having launched nothing, for any other.
+//  * in_ssq [M][in_parts], in_eps: A holds bf16(x g) of rows x whose sums of squares these are; the
+//    product's sums are multiplied by the row's 1 / sqrt(sum / K + eps) before bias and epilogue.
+//  * out_g [N], out_xg [M][N] bf16, out_ssq [M][ceil(N / 256)]: beside C (32-bit, stored or added
+//    to), bf16(C g) and the sums of C^2 over runs of 256 columns are written.
+MF_API int mf_gemm_bf16_skinny_fused(const void* A, int lda, const void* W, const void* Wt, int ldw,
+                                     const float* bias, void* C, int ldc, float* part, int M, int N, int K,
+                                     int splits, int k_per_split, int epi, const float* in_ssq, int in_parts,
+                                     float in_eps, const float* out_g, void* out_xg, float* out_ssq,
+                                     hipStream_t stream) {
+  if (in_ssq && in_parts < 1) return (int)hipErrorInvalidValue;
+  if (out_g && (!out_xg || !out_ssq || (epi != EPI_F32 && epi != EPI_ACC_F32))) return (int)hipErrorInvalidValue;
+  const FusedNorm fused{in_ssq, in_parts, in_eps, out_g, (bf16*)out_xg, out_ssq};
+  return skinny_product(A, lda, W, Wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, fused, stream);
 }
 
 // RMS norm of rows of the 32-bit residual stream x (row m of the product is x[row_idx[m]]), then

@@ -35,6 +35,12 @@ class StepContext:
     host_new: List[int] = field(default_factory=list)        # new tokens of each sequence
     host_start: Optional[List[int]] = None                   # tokens each held before (None in a decode step)
     new_lengths: Dict[int, int] = field(default_factory=dict)   # slot -> tokens held after the step
+    # between a product that adds into the residual stream and the norm that reads it next (see
+    # `parts.base.announce_norm`): the norm the running part's output meets, the norm that follows
+    # the running block, and what a product prepared for the next norm
+    norm_next: object = None
+    norm_after_block: object = None
+    norm_ahead: object = None
     _memo: Dict = field(default_factory=dict, repr=False)
 
     def page_table(self, group) -> torch.Tensor:

@@ -129,14 +129,21 @@ class DecoderModel:
         self.embedding.forward(ctx.token_ids, h, ctx)
         rows = ctx.logit_rows
         last = len(s.schedule) - 1
+        ctx.norm_ahead = None
         for n, e in enumerate(s.schedule):
             keep = rows if (n == last and rows is not None) else None
+            # the norm that reads the stream behind this block: the next block's first one, or the final one
+            ctx.norm_after_block = (self.final_norm if n == last else self.blocks[s.schedule[n + 1].block].first_norm())
             h = self.blocks[e.block].forward(h, ctx, e.cache, e.writes_cache, keep_rows=keep)
+            ahead = ctx.norm_ahead
+            if ahead is not None and (ahead.norm is not ctx.norm_after_block or ahead.h is not h):
+                ctx.norm_ahead = None            # prepared for someone who will not come
+        ctx.norm_after_block = None
         if not s.schedule and rows is not None:
             kept = torch.empty((rows.numel(), s.hidden_size), dtype=torch.float32, device=h.device)
             ops.gather_rows(h, rows, kept)
             h = kept
-        return self.head.forward(normed_input(self.final_norm, self.head, h), ctx)
+        return self.head.forward(normed_input(self.final_norm, self.head, h, ctx=ctx), ctx)
 
 
 def expected_tensors(spec: ModelSpec) -> Dict[str, TensorSpec]:

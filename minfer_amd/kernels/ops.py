@@ -59,6 +59,8 @@ _PROTOTYPES = {
                                 c_int, c_int, _P],
         "mf_gemm_bf16_normed": [_P, c_int, _P, _P, c_float, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int,
                                 c_int, _P],
+        "mf_gemm_bf16_skinny_fused": [_P, c_int, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int,
+                                      c_int, c_int, _P, c_int, c_float, _P, _P, _P, _P],
         "mf_gemm_bf16_plan": [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_char_p, c_int],
         "mf_gemm_bf16_tile_plan": [c_int, c_int, c_int, c_int, c_int, c_int, _P],
     },
@@ -655,6 +657,79 @@ def linear_normed(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, row_id
     if rc == NOT_BUILT:
         return False
     _check(rc, f"gemm_bf16_normed{'(swiglu)' if swiglu else ''} {m}x{n}x{k}")
+    return True
+
+
+NORM_SUM_RUN = 256       # columns a partial sum of squares covers (a block of the kernel that adds a K split's parts)
+
+
+def norm_sum_parts(n: int) -> int:
+    """Partial sums of squares a row of `n` values comes with (see `linear_fused`)."""
+    return (n + NORM_SUM_RUN - 1) // NORM_SUM_RUN
+
+
+def linear_fused(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                 accumulate: bool = False, tiled: Optional[torch.Tensor] = None, swiglu: bool = False,
+                 scale_in=None, norm_out=None) -> bool:
+    """A bfloat16 product of at most 64 rows with an RMS norm folded in on either side, for steps of
+    17 to 64 tokens, where the norm would otherwise be a kernel of its own between two products:
+
+    * `norm_out` = (g `[n]`, xg `[m][n]` bfloat16, sums `[m][norm_sum_parts(n)]`): the product stores
+      or adds into the 32-bit `out` as `linear` does and leaves, beside it, bf16(out g) and the sums
+      of out^2 over runs of 256 columns, for the norm with weight g that reads `out` next;
+    * `scale_in` = (sums `[m][parts]`, eps): `x` is such an xg, and the product's sums are multiplied
+      by the row's 1 / sqrt(sum / k + eps) before the bias and the epilogue; with `swiglu`, `weight`
+      is `interleave_gate_up(Wg, Wu)` and out = silu(gate) * up, bfloat16.
+
+    Returns False, having launched nothing, where the kernels the shape takes have no place for it
+    (the caller then runs norm and product one after the other)."""
+    _need(x, "linear_fused.x", torch.bfloat16)
+    _need(weight, "linear_fused.weight", torch.bfloat16)
+    m, k = x.shape
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"linear_fused: x is [{m},{k}], weight is {tuple(weight.shape)}")
+    if m == 0 or m > 64 or (scale_in is None and norm_out is None):
+        return False
+    if swiglu:
+        nf = out.shape[1]
+        if n % 64 or not n // 2 - 32 < nf <= n // 2 or bias is not None or accumulate or norm_out is not None:
+            raise KernelError(f"linear_fused(swiglu): weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+        _need(out, "linear_fused.out", torch.bfloat16, (m, nf))
+        epi, ldc = EPI_SWIGLU, nf
+    else:
+        _need(out, "linear_fused.out", _FLOATS, (m, n))
+        if accumulate and out.dtype != torch.float32:
+            raise KernelError("linear_fused: accumulation needs a float32 output")
+        epi = EPI_BF16 if out.dtype == torch.bfloat16 else (EPI_ACC_F32 if accumulate else EPI_F32)
+        ldc = n
+    if bias is not None:
+        _need(bias, "linear_fused.bias", torch.float32, (n,))
+    in_ssq, in_parts, in_eps = None, 0, 0.0
+    if scale_in is not None:
+        in_ssq, in_eps = scale_in
+        _need(in_ssq, "linear_fused.scale_in", torch.float32)
+        if in_ssq.dim() != 2 or in_ssq.shape[0] != m or in_ssq.shape[1] < 1:
+            raise KernelError(f"linear_fused.scale_in: sums {tuple(in_ssq.shape)} for {m} rows")
+        in_parts = in_ssq.shape[1]
+    out_g = out_xg = out_ssq = None
+    if norm_out is not None:
+        out_g, out_xg, out_ssq = norm_out
+        if out.dtype != torch.float32:
+            raise KernelError("linear_fused.norm_out: the product's own output must be float32")
+        _need(out_g, "linear_fused.norm_out.g", torch.float32, (n,))
+        _need(out_xg, "linear_fused.norm_out.xg", torch.bfloat16, (m, n))
+        _need(out_ssq, "linear_fused.norm_out.sums", torch.float32, (m, norm_sum_parts(n)))
+    aligned = not (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8)
+    splits, per = _k_split(m, n, k, swiglu, aligned, tiled=tiled is not None)
+    part = workspace("skinny", splits * m * n, x.device) if (splits > 1 or (swiglu and m > 16)) else None
+    _need_tiled(tiled, "linear_fused.tiled", n, k)
+    rc = _fn("gemm_bf16", "mf_gemm_bf16_skinny_fused")(
+        _ptr(x), k, _ptr(weight), _ptr(tiled), k, _ptr(bias), _ptr(out), ldc, _ptr(part), m, n, k, splits, per, epi,
+        _ptr(in_ssq), in_parts, float(in_eps), _ptr(out_g), _ptr(out_xg), _ptr(out_ssq), _stream())
+    if rc == NOT_BUILT:
+        return False
+    _check(rc, f"gemm_bf16_skinny_fused{'(swiglu)' if swiglu else ''} {m}x{n}x{k}")
     return True
 
 

@@ -20,7 +20,9 @@ Kernel choice, for measurements (each overrides what `ops` would pick by shape):
 * MF_NO_SHARED_PAGES=1  a block of queries of the prompt attention keeps all its pages to itself
 * MF_NO_DECODE_COPIES=1 a model keeps no second, tiled copy of its matrices for the steps of few tokens
 * MF_NO_FOLD=1          the RMS norm is a kernel of its own instead of being folded into the
-                        product that follows it
+                        product that follows it (steps of at most 16 rows)
+* MF_NO_NORM_AHEAD=1    in steps of 17 to 64 rows, a product that adds into the residual stream does
+                        not prepare the next norm's input: the norm is a kernel of its own
 """
 from __future__ import annotations
 
@@ -44,5 +46,6 @@ ATTN_SPLITS = _int("MF_ATTN_SPLITS")
 ATTN_EQUAL_SPLITS = _flag("MF_ATTN_EQUAL_SPLITS")
 SKINNY_TARGET = _int("MF_SKINNY_TARGET")
 NO_FOLD = _flag("MF_NO_FOLD")
+NO_NORM_AHEAD = _flag("MF_NO_NORM_AHEAD")
 NO_SHARED_PAGES = _flag("MF_NO_SHARED_PAGES")
 NO_DECODE_COPIES = _flag("MF_NO_DECODE_COPIES")

@@ -81,7 +81,7 @@ class GQAttention(Mixer):
             # decode: rotation, cache write and attention in one kernel
             ops.attn_decode_rope(qkv, tables[0], tables[1], kc, vc, table, ctx.positions, ctx.seq_of_tok, o,
                                  self.nh, self.nk, self.hd, self.scale, window, ctx.max_len, writes_cache)
-            self.o(o, out=h, accumulate=True)
+            self.o(o, out=h, accumulate=True, ctx=ctx)
             return
         q = torch.empty_like(o)
         if tables is not None:         # rotation and cache write in one kernel
@@ -99,4 +99,4 @@ class GQAttention(Mixer):
         else:
             ops.attn_tokens(q, kc, vc, table, ctx.positions, ctx.seq_of_tok, o, self.nh, self.nk,
                             self.hd, self.scale, window, ctx.max_len)
-        self.o(o, out=h, accumulate=True)
+        self.o(o, out=h, accumulate=True, ctx=ctx)

@@ -68,14 +68,28 @@ class Norm(Part):
         return None
 
 
+@dataclass
+class NormAhead:
+    """What a product that added into the residual stream `h` left for `norm`, the norm that reads
+    the stream next: bf16(h g) and, per row, partial sums of h^2 (`ops.linear_fused`).  The product
+    that follows the norm may take these instead of the normed rows."""
+    norm: "Norm"
+    h: torch.Tensor
+    xg: torch.Tensor
+    sums: torch.Tensor
+
+
 class Normed:
     """The rows `norm(h[row_idx])` before anyone has computed them.  A block hands this to a
     mixer or feed-forward that declares `takes_normed = True`; such a part passes it to its
     first `Linear`, which folds the norm into the product where a kernel for that exists, or
-    calls `tensor()` (computed once, then kept) like any part that needs the rows themselves."""
+    calls `tensor()` (computed once, then kept) like any part that needs the rows themselves.
+    `ahead`: what the product before the norm prepared for it, if it did."""
 
-    def __init__(self, norm: "Norm", h: torch.Tensor, row_idx: Optional[torch.Tensor] = None):
+    def __init__(self, norm: "Norm", h: torch.Tensor, row_idx: Optional[torch.Tensor] = None,
+                 ahead: Optional[NormAhead] = None):
         self.norm, self.h, self.row_idx = norm, h, row_idx
+        self.ahead = ahead
         self._rows: Optional[torch.Tensor] = None
 
     @property
@@ -92,11 +106,26 @@ class Normed:
         return self._rows
 
 
-def normed_input(norm: "Norm", part, h: torch.Tensor, row_idx: Optional[torch.Tensor] = None):
-    """What a block gives `part` as its input: the lazy form if the part takes it."""
+def normed_input(norm: "Norm", part, h: torch.Tensor, row_idx: Optional[torch.Tensor] = None, ctx=None):
+    """What a block gives `part` as its input: the lazy form if the part takes it.  With `ctx`,
+    whatever the product before left for this norm over these rows (`ctx.norm_ahead`) goes along,
+    and is taken off the context either way: it describes the stream as it is now."""
+    ahead = None
+    if ctx is not None:
+        ahead, ctx.norm_ahead = getattr(ctx, "norm_ahead", None), None
+        if ahead is not None and (ahead.norm is not norm or ahead.h is not h or row_idx is not None):
+            ahead = None
     if getattr(part, "takes_normed", False):
-        return Normed(norm, h, row_idx)
+        return Normed(norm, h, row_idx, ahead)
     return norm.forward(h, row_idx=row_idx)
+
+
+def announce_norm(ctx, norm: Optional["Norm"]) -> None:
+    """A block says which norm reads the residual stream after the part it is about to run (None:
+    nobody it knows of).  A part whose last product adds into the stream may pass `ctx` on to it
+    (`Linear(..., ctx=ctx)`), and the product may then prepare that norm's input (`NormAhead`)."""
+    ctx.norm_next = norm
+    ctx.norm_ahead = None
 
 
 class PositionEncoding(Part):
@@ -195,6 +224,11 @@ class Block:
         """Every part of the block that exists, norms in the order of `norm_names`."""
         named = [self.norms[n] for n in self.norm_names + self.optional_norms if n in self.norms]
         return tuple(p for p in [self.mixer, self.feed_forward] + named if p is not None)
+
+    def first_norm(self) -> Optional[Norm]:
+        """The norm that reads the residual stream first when this block runs, if it starts with
+        one (the block before may then prepare its input, see `announce_norm`)."""
+        return None
 
     def forward(self, h, ctx, entry: int, writes_cache: bool, keep_rows=None):
         raise NotImplementedError

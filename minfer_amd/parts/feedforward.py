@@ -56,9 +56,15 @@ class SwiGLU(FeedForward):
         y = torch.empty((x.shape[0], self.inter), dtype=self.rt.dtype, device=x.device)
         if self.fused is not None:
             fold = x.norm.rms_scale() if isinstance(x, Normed) else None
-            if fold is None or not ops.linear_normed(x.h, fold[0], fold[1], x.row_idx, self.fused, None, y,
-                                                     swiglu=True, tiled=self.fused_tiled):
+            done = False
+            if fold is not None and x.ahead is not None:      # the product before prepared this norm's input
+                done = ops.linear_fused(x.ahead.xg, self.fused, None, y, tiled=self.fused_tiled, swiglu=True,
+                                        scale_in=(x.ahead.sums, fold[1]))
+            if not done and fold is not None:
+                done = ops.linear_normed(x.h, fold[0], fold[1], x.row_idx, self.fused, None, y, swiglu=True,
+                                         tiled=self.fused_tiled)
+            if not done:
                 ops.linear_swiglu(x.tensor() if isinstance(x, Normed) else x, self.fused, y, tiled=self.fused_tiled)
         else:
             ops.swiglu(self.gate_up(x, out_dtype=torch.float32), y)
-        self.down(y, out=h, accumulate=True)
+        self.down(y, out=h, accumulate=True, ctx=ctx)

@@ -11,8 +11,8 @@ from typing import List, Optional
 
 import torch
 
-from ..kernels import ops
-from .base import Normed
+from ..kernels import ops, tuning
+from .base import NormAhead, Normed
 
 
 def common_matrix_dtype(tensors: List[torch.Tensor]) -> torch.dtype:
@@ -52,15 +52,22 @@ class Linear:
         return cls(w, b)
 
     def __call__(self, x, out: Optional[torch.Tensor] = None,
-                 out_dtype: torch.dtype = torch.float32, accumulate: bool = False) -> torch.Tensor:
+                 out_dtype: torch.dtype = torch.float32, accumulate: bool = False, ctx=None) -> torch.Tensor:
+        """`ctx`: the step's context, from a part whose output this product adds into the residual
+        stream: where the block has announced the norm that reads the stream next, the product
+        may prepare that norm's input on its way out (`_prepare_norm`)."""
         rows = x.shape[0]
         if out is None:
             out = torch.empty((rows, self.out_features), dtype=out_dtype, device=x.device)
         if isinstance(x, Normed):
-            fold = x.norm.rms_scale() if self.weight.dtype == torch.bfloat16 else None
-            if fold is not None and ops.linear_normed(x.h, fold[0], fold[1], x.row_idx, self.weight, self.bias,
-                                                      out, accumulate=accumulate, tiled=self.tiled):
-                return out
+            if self.weight.dtype == torch.bfloat16:
+                if x.ahead is not None and ops.linear_fused(x.ahead.xg, self.weight, self.bias, out, accumulate=accumulate,
+                                                            tiled=self.tiled, scale_in=(x.ahead.sums, x.norm.rms_scale()[1])):
+                    return out
+                fold = x.norm.rms_scale()
+                if fold is not None and ops.linear_normed(x.h, fold[0], fold[1], x.row_idx, self.weight, self.bias,
+                                                          out, accumulate=accumulate, tiled=self.tiled):
+                    return out
             x = x.tensor()
         if self.weight.dtype == torch.float32 and x.dtype != torch.float32:
             wide = torch.empty(x.shape, dtype=torch.float32, device=x.device)
@@ -71,5 +78,28 @@ class Linear:
             ops.linear(x, self.weight, self.bias, tmp)
             ops.convert(tmp, out)
             return out
+        if ctx is not None and self._prepare_norm(x, out, accumulate, ctx):
+            return out
         ops.linear(x, self.weight, self.bias, out, accumulate=accumulate, tiled=self.tiled)
         return out
+
+    def _prepare_norm(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool, ctx) -> bool:
+        """Runs the product with the next norm's input prepared beside it (bf16(out g) and the rows'
+        partial sums of squares, left in `ctx.norm_ahead`) where the block has said which norm
+        that is, the norm is of the RMS form and the product's kernels have a place for it (steps of
+        17 to 64 rows whose K is split over blocks).  False: nothing ran."""
+        norm = getattr(ctx, "norm_next", None)
+        if norm is None or not 16 < x.shape[0] <= 64 or x.dtype != torch.bfloat16 or out.dtype != torch.float32:
+            return False
+        if tuning.NO_NORM_AHEAD:
+            return False
+        fold = norm.rms_scale()
+        if fold is None or fold[0].numel() != self.out_features:
+            return False
+        xg = torch.empty(out.shape, dtype=torch.bfloat16, device=out.device)
+        sums = torch.empty((out.shape[0], ops.norm_sum_parts(self.out_features)), dtype=torch.float32, device=out.device)
+        if not ops.linear_fused(x, self.weight, self.bias, out, accumulate=accumulate, tiled=self.tiled,
+                                norm_out=(fold[0], xg, sums)):
+            return False
+        ctx.norm_ahead = NormAhead(norm, out, xg, sums)
+        return True

@@ -132,6 +132,11 @@ def linear_normed(x, norm_weight, eps, row_idx, weight, bias, out, accumulate=Fa
     return False
 
 
+def linear_fused(x, weight, bias, out, accumulate=False, tiled=None, swiglu=False, scale_in=None, norm_out=None):
+    """The stand-in folds no norm around a product: the caller runs the norm as a step of its own."""
+    return False
+
+
 def linear_normed_reference(x, norm_weight, eps, row_idx, weight, bias, swiglu=False):
     """What the folded kernel computes, in float64, with its one rounding of the activations:
     bf16(x * g) goes to the matrix cores and 1 / sqrt(mean(x^2) + eps) is applied to the sums."""
@@ -266,7 +271,7 @@ def advance(next_ids, sampled, positions, steps, prev=None, n_prev=None, cursor=
 
 NAMES = ["embed", "rmsnorm", "gather_rows", "swiglu", "convert", "fill_normal", "rope_table",
          "rope_kvwrite", "rope_inplace", "linear", "attn_tokens", "attn_prefill", "argmax", "sample", "penalties",
-         "top_k", "top_p", "sample_filtered", "sample_filtered_takes", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed", "attn_decode_rope"]
+         "top_k", "top_p", "sample_filtered", "sample_filtered_takes", "advance", "interleave_gate_up", "linear_swiglu", "linear_normed", "linear_fused", "attn_decode_rope"]
 
 
 def install(monkeypatch):

@@ -107,6 +107,32 @@ def test_four_layers_untied_head_at_7b_widths(folder4, reference4, dtype):
     print(f"{dtype}: worst abs err {worst:.3e} (logit std {float(ref['r1'].std()):.3f})")
 
 
+def test_batch_of_forty_through_four_layers(folder4):
+    """Forty short requests through four layers: steps of 17 to 64 rows, where the norms are folded
+    around the products (the product that adds into the stream prepares the next norm's input, the
+    product behind the norm applies the rows' factors), from one layer to the next and into the
+    final norm; then the batch thins out into the steps of at most 16 rows."""
+    from minfer_amd import Engine, load_model
+    from minfer_amd.kernels import ops
+    plain = PlainQwen2.from_folder(folder4, dtype=np.float64)
+    reqs = requests_for(152064, [2 + (i * 3) % 5 for i in range(40)], seed=18)
+    ref = plain_logits(plain, reqs)
+    del plain
+    eng = Engine(load_model(folder4, dtype="bfloat16"), max_tokens=64 * 40, poison_cache=True)
+    steps = batch_steps(reqs, [list(reqs)], prompt_frac=0.4)
+    assert 17 <= len(steps[1]["entries"]) <= 64
+    calls = []
+    real = ops.linear_fused
+    ops.linear_fused = lambda *a, **k: calls.append((a[0].shape[0], "scale_in" in k and k["scale_in"] is not None, real(*a, **k))) or calls[-1][2]
+    try:
+        worst = compare(run_steps(eng, steps), ref, "bfloat16", "7B widths, 4 layers, batch of 40", layers=4)
+    finally:
+        ops.linear_fused = real
+    took = [c for c in calls if c[2]]
+    assert any(c[1] for c in took) and any(not c[1] for c in took), "both sides of the fold ran"
+    print(f"worst abs err {worst:.3e}; {len(took)} of {len(calls)} fused calls ran")
+
+
 # ------------------------------------------------------------------ the whole depth: all 28 layers
 SHAPE_7B_FULL = dict(WIDTHS_7B, num_hidden_layers=28, tie_word_embeddings=False)
 
