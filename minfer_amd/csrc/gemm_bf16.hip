@@ -435,11 +435,20 @@ __global__ __launch_bounds__(512) void tile_dma_kernel(const bf16* __restrict__ 
     __builtin_amdgcn_sched_barrier(0);
     dma_wait<LOADS>(issued - kt - 2);          // tile kt + 1 has landed when only the later ones are in flight
     __syncthreads();
-    if (issued < nkt) { issue(issued, stage); ++issued; }         // into the stage of tile kt
+    // Tile kt + STAGES goes into the stage of tile kt: waves 0..3 set their copies out here, waves
+    // 4..7 (the other wave of each SIMD) behind the tile's last products, a quarter of a k tile
+    // later.  All eight at once measured 2 to 11 % slower (the down product of a prompt most):
+    // the copies' requests reach the L2 in one burst from every CU of the XCD, which walk K in
+    // step, and meet the fragment reads of the new tile in LDS.  (Four groups a quarter apart,
+    // or every wave's copies in two halves, measured worse than two groups: the last ones land late.)
+    const int freed = stage;
+    if (wid < 4 && issued < nkt) { issue(issued, freed); ++issued; }
     stage = stage + 1 == STAGES ? 0 : stage + 1;
     read_frags(stage, S0{});
     __builtin_amdgcn_sched_barrier(0);
     multiply(1, S1{});
+    __builtin_amdgcn_sched_barrier(0);
+    if (wid >= 4 && issued < nkt) { issue(issued, freed); ++issued; }
     __builtin_amdgcn_sched_barrier(0);
   }
   multiply(0, S0{});
