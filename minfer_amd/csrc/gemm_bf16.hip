@@ -9,7 +9,7 @@
 //  * `tile_dma_kernel`: tiles of 256 x 256, 256 x 192 or 256 x 128 with their k tiles copied
 //    straight into LDS; the choice for large aligned products (the width by how the tiles fill
 //    the chip's rounds).
-//  * `stationary16_kernel`: at most 16 rows and K of 1536, 2048, 3584, 4096, 5120 or 8192 (decode):
+//  * `stationary16_kernel`: at most 16 rows and K of 896, 1536, 2048, 3584, 4096, 5120 or 8192 (decode):
 //    one block per CU keeps the activations in registers and walks over weight tiles.
 //  * `rolling16_kernel`, `skinny16_kernel`: at most 16 rows, any K (decode).  The time is the
 //    weight stream: the waves of a block split K, each reads weights and activations straight
@@ -846,9 +846,15 @@ constexpr int stationary_ring(int NS, int NT) {
   return 1;
 }
 
+constexpr int STATIONARY_K7 = 896;       // the one K that runs as 7 waves of 4 steps
+
 bool stationary_takes(int M, int N, int K, int epi, bool normed) {
-  if (M > 16 || K % 256 != 0 || (N + 15) / 16 < 128) return false;
   if (epi == EPI_SWIGLU && N % 64 != 0) return false;
+  // (a model that narrow has few weight rows as well, and its steps are their kernels' starts, not
+  // the stream: there the fold of the norm is what this kernel is taken for, from 64 tiles on)
+  if (K == STATIONARY_K7) return M <= 16 && (N + 15) / 16 >= 64;
+  if (M > 16 || (N + 15) / 16 < 128) return false;
+  if (K % 256 != 0) return false;
   // a K above 5120 without a norm or SwiGLU to fold in (the o product of the widest models): the
   // rolling kernel is the faster one there
   if (K > 5120 && !normed && epi != EPI_SWIGLU) return false;
@@ -1060,14 +1066,15 @@ struct NormArgs {
 // RING = NS the registers hold a whole item; for a long K (5120, 8192) the activations alone take
 // up to half the registers, so the weights go through a shorter ring, and a register is refilled
 // with the step RING further on, of this item or of the next one.
-template <int NS, int RING, int NT, bool PAIR, bool NORM, bool TILED>
-__global__ __launch_bounds__(512) void stationary16_kernel(const void* __restrict__ Av, int lda,
-                                                           const bf16* __restrict__ W, int ldw,
-                                                           const float* __restrict__ bias,
-                                                           void* __restrict__ C, int ldc, int M, int N,
-                                                           int cols_total, int unit, int share, int extra, int epi,
-                                                           NormArgs norm) {
-  constexpr int NW = 8;
+// NW: waves of a block, each with a slice of NS steps of K: 8, K = 256 NS; or 7 with NS = 4 for a K
+// of 896 (14 heads of 64, the narrowest model of the family), which is no multiple of 256.
+template <int NS, int RING, int NT, bool PAIR, bool NORM, bool TILED, int NW = 8>
+__global__ __launch_bounds__(NW * 64) void stationary16_kernel(const void* __restrict__ Av, int lda,
+                                                               const bf16* __restrict__ W, int ldw,
+                                                               const float* __restrict__ bias,
+                                                               void* __restrict__ C, int ldc, int M, int N,
+                                                               int cols_total, int unit, int share, int extra, int epi,
+                                                               NormArgs norm) {
   constexpr int KK = NW * NS * 32;         // K
   constexpr int WSTEP = TILED ? 512 : 32;  // elements from one step's weights to the next's
   constexpr int COLS = 16 * NT;            // weight rows (output columns) of an item
@@ -1076,7 +1083,7 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
   __shared__ float ssq[NW][16];            // NORM: sum of x^2 over a wave's slice, per activation row
   extern __shared__ __attribute__((aligned(16))) float gs[];   // NORM: the norm's weight, K floats
   static_assert(NS % RING == 0, "the ring divides a slice");
-  static_assert(NW * (64 / COLS) >= 16, "an epilogue pass for every activation row");
+  static_assert(PAIR ? NW * 4 >= 16 : NW * (64 / COLS) >= 16, "an epilogue pass for every activation row");
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int r16 = lane & 15;
   const int k0 = wid * NS * 32 + (lane >> 4) * 8;         // this lane's k in step 0 of its slice
@@ -1297,7 +1304,7 @@ __global__ __launch_bounds__(512) void stationary16_kernel(const void* __restric
 }
 
 // true when the shape is one the register-resident kernel is built for
-template <int NS, int NT, bool PAIR, bool TILED>
+template <int NS, int NT, bool PAIR, bool TILED, int NW = 8>
 int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
                         int M, int N, int epi, const NormArgs* norm, hipStream_t stream) {
   const int n_cu = cu_count();
@@ -1313,8 +1320,8 @@ int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const fl
   constexpr int RING = stationary_ring(NS, NT);
   static_assert(NS % RING == 0 && 4 * NS + 4 * NT * RING <= 200, "activations and weight ring fit the registers");
   if (norm) {
-    constexpr int smem = 8 * NS * 32 * (int)sizeof(float);       // the norm's weight
-    auto kern = stationary16_kernel<NS, RING, NT, PAIR, true, TILED>;
+    constexpr int smem = NW * NS * 32 * (int)sizeof(float);      // the norm's weight
+    auto kern = stationary16_kernel<NS, RING, NT, PAIR, true, TILED, NW>;
     static bool configured = false;
     if (!configured) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1322,10 +1329,10 @@ int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const fl
       if (e != hipSuccess) return (int)e;
       configured = true;
     }
-    kern<<<grid, 512, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, cols_total, unit, units / grid, units % grid,
+    kern<<<grid, NW * 64, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, cols_total, unit, units / grid, units % grid,
                                       epi, *norm);
   } else {
-    stationary16_kernel<NS, RING, NT, PAIR, false, TILED><<<grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
+    stationary16_kernel<NS, RING, NT, PAIR, false, TILED, NW><<<grid, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
                                                                              cols_total, unit, units / grid,
                                                                              units % grid, epi,
                                                                              NormArgs{nullptr, nullptr, 0.f});
@@ -1908,6 +1915,14 @@ static int stationary16(const void* a, int lda, const bf16* w, const bf16* wt, i
                      : launch_stationary16<NS_, 1, false, T_>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, stream))
 #define MF_STATIONARY(NS_) \
   case NS_: return wt ? MF_STATIONARY_T(NS_, true, wt) : MF_STATIONARY_T(NS_, false, w);
+  if (K == STATIONARY_K7) {
+    // seven waves: one tile an item outside SwiGLU (the epilogue gives every wave 64 / (16 NT) rows)
+#define MF_STATIONARY_7(T_, W_)                                                                                  \
+  (epi == EPI_SWIGLU ? launch_stationary16<4, 2, true, T_, 7>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, stream) \
+                     : launch_stationary16<4, 1, false, T_, 7>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, stream))
+    return wt ? MF_STATIONARY_7(true, wt) : MF_STATIONARY_7(false, w);
+#undef MF_STATIONARY_7
+  }
   switch (K / 256) { MF_STATIONARY_NS(MF_STATIONARY) }
 #undef MF_STATIONARY
 #undef MF_STATIONARY_T

@@ -419,12 +419,15 @@ def cu_count() -> int:
 # K = 256 NS for which the register-resident decode product is instantiated
 # (MF_STATIONARY_NS in csrc/gemm_bf16.hip; `plan_linear` asks the library itself)
 STATIONARY_NS = (4, 6, 8, 10, 12, 14, 16, 20, 24, 28, 32)
+STATIONARY_K7 = 896      # and this K, which runs as seven waves of four steps (the narrowest model of the family)
 
 
 def stationary_shape(n: int, k: int, folded: bool = False) -> bool:
     """True where the register-resident decode product is built for [n][k] weights (aligned
-    operands given): K = 256 NS for one of the NS above and at least 128 tiles of 16 weight rows;
+    operands given): K = 256 NS for one of the NS above, or 896, and at least 128 tiles of 16 weight rows;
     a K above 5120 only with a norm or SwiGLU folded in (`folded`)."""
+    if k == STATIONARY_K7:
+        return (n + 15) // 16 >= 64
     return k % 256 == 0 and k // 256 in STATIONARY_NS and (n + 15) // 16 >= 128 and (k <= 5120 or folded)
 
 

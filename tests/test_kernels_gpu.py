@@ -634,6 +634,7 @@ def test_tile_weight_layout(ops):
 
 @pytest.mark.parametrize("m,n,k", [(8, 3584, 18944), (1, 1000, 8224), (16, 4608, 3584), (5, 152064, 1536),
                                    (3, 2100, 8192), (16, 8192, 8192), (8, 90, 4096), (2, 2048, 96),
+                                   (8, 2100, 896), (16, 4864, 896),
                                    # 17 to 64 rows: K split over blocks, and the whole-K kernel of a wide matrix
                                    (64, 3584, 3584), (40, 3584, 18944), (17, 1000, 2048), (33, 40001, 768),
                                    (64, 33000, 512),
@@ -730,7 +731,8 @@ def test_gemm_bf16_swiglu(ops, variant, m, nf, k):
 @pytest.mark.parametrize("m,n,k,idx", [(1, 2100, 1536, False), (5, 4608, 2048, True), (8, 4001, 3584, False),
                                        (16, 2048, 4096, True), (3, 152064, 3584, True),
                                        (2, 2100, 5120, True), (9, 5000, 5120, False), (7, 5000, 8192, True),
-                                       (16, 2048, 8192, False)])
+                                       (16, 2048, 8192, False), (1, 2100, 896, False), (8, 1152, 896, True),
+                                       (16, 151936, 896, False)])
 def test_gemm_bf16_normed(ops, m, n, k, idx):
     """RMS norm folded into the few-row product: against the same formula in float64 with the
     kernel's one rounding (tight), and against norm-then-product as the two kernels do it."""
@@ -763,7 +765,7 @@ def test_gemm_bf16_normed(ops, m, n, k, idx):
 
 
 @pytest.mark.parametrize("m,nf,k", [(8, 1100, 1536), (3, 2100, 3584), (16, 1030, 4096), (1, 18944, 3584),
-                                    (4, 2100, 5120), (16, 1100, 8192), (1, 2500, 8192)])
+                                    (4, 2100, 5120), (16, 1100, 8192), (1, 2500, 8192), (8, 4864, 896), (16, 1100, 896)])
 def test_gemm_bf16_normed_swiglu(ops, m, nf, k):
     h = rnd((m, k), seed=50, scale=2.0)
     g = 1.0 + rnd((k,), seed=51, scale=0.2)
