@@ -1635,6 +1635,77 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
   }
 }
 
+// The same for rows whose length is a multiple of 4 (16-byte aligned parts, bias and output): a
+// thread adds up four neighbouring outputs, a wave a run of 256 columns (so that a run's sum of
+// squares is one wave's and needs no barrier), a block four runs.  A quarter of the blocks and of
+// the loads of the kernel above, which is what its time is made of.
+__global__ __launch_bounds__(256) void skinny_reduce4_kernel(const float* __restrict__ part,
+                                                             const float* __restrict__ bias,
+                                                             void* __restrict__ C, int ldc, int M, int N, int K,
+                                                             int splits, int epi, FusedNorm fused) {
+  const int run = blockIdx.x * 4 + (threadIdx.x >> 6);       // of 256 columns
+  const int n = run * 256 + (threadIdx.x & 63) * 4, m = blockIdx.y;
+  if (run * 256 >= N) return;                                // (whole waves leave: the shuffles below stay among those that stay)
+  const size_t stride = (size_t)M * N;
+  const int frow[1] = {fused.in_ssq ? m : -1};
+  float ffac[1];
+  row_sums_ask<1>(fused, frow, M, threadIdx.x & 63, ffac);
+  float4 v = float4{0.f, 0.f, 0.f, 0.f};
+  const bool in = n < N;                                     // N in fours: all four inside, or none
+  if (in) {
+    const float* p = part + (size_t)m * N + n;
+    for (int s0 = 0; s0 < splits; s0 += 8) {                 // eight parts' loads in flight together, added in their order
+      float4 x[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        x[j] = s0 + j < splits ? *reinterpret_cast<const float4*>(p + (size_t)(s0 + j) * stride) : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) { v.x += x[j].x; v.y += x[j].y; v.z += x[j].z; v.w += x[j].w; }
+    }
+  }
+  row_factors_of<1>(fused, frow, M, K, ffac);
+  if (in) {
+    const float rf = ffac[0];
+    const float4 b = bias ? *reinterpret_cast<const float4*>(bias + n) : float4{0.f, 0.f, 0.f, 0.f};
+    v = float4{v.x * rf + b.x, v.y * rf + b.y, v.z * rf + b.z, v.w * rf + b.w};
+    if (epi == EPI_BF16) {
+      bf16* c = (bf16*)C + (size_t)m * ldc + n;
+      c[0] = (bf16)v.x; c[1] = (bf16)v.y; c[2] = (bf16)v.z; c[3] = (bf16)v.w;
+    } else {
+      float4* c = reinterpret_cast<float4*>((float*)C + (size_t)m * ldc + n);
+      if (epi == EPI_ACC_F32) { const float4 o = *c; v = float4{v.x + o.x, v.y + o.y, v.z + o.z, v.w + o.w}; }
+      *c = v;
+    }
+  }
+  if (fused.out_g) {
+    if (in) {
+      const float4 g = *reinterpret_cast<const float4*>(fused.out_g + n);
+      bf16* xg = fused.out_xg + (size_t)m * N + n;
+      xg[0] = (bf16)(v.x * g.x); xg[1] = (bf16)(v.y * g.y); xg[2] = (bf16)(v.z * g.z); xg[3] = (bf16)(v.w * g.w);
+    }
+    float sq = ((v.x * v.x + v.y * v.y) + v.z * v.z) + v.w * v.w;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, MF_WAVE);
+    if ((threadIdx.x & 63) == 0) fused.out_ssq[(size_t)m * ((N + 255) / 256) + run] = sq;
+  }
+}
+
+// adds the parts of a K split and runs the epilogue: the kernel in fours where the operands allow it
+int launch_reduce(const float* part, const float* bias, void* C, int ldc, int M, int N, int K, int splits, int epi,
+                  const FusedNorm& fused, hipStream_t stream) {
+  const bool fours = epi != EPI_SWIGLU && N % 4 == 0 && ldc % 4 == 0 && (uintptr_t)part % 16 == 0 &&
+                     (uintptr_t)bias % 16 == 0 && (uintptr_t)C % 16 == 0 && (uintptr_t)fused.out_g % 16 == 0 &&
+                     (uintptr_t)fused.out_xg % 8 == 0;
+  if (fours) {
+    dim3 g4((N + 1023) / 1024, M);
+    skinny_reduce4_kernel<<<g4, 256, 0, stream>>>(part, bias, C, ldc, M, N, K, splits, epi, fused);
+  } else {
+    dim3 g2(((epi == EPI_SWIGLU ? ldc : N) + 255) / 256, M);
+    skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, K, splits, epi, fused);
+  }
+  return mf_launch_status();
+}
+
 template <int MT, bool VEC>
 int launch_skinny_v(const bf16* A, int lda, const bf16* W, const bf16* Wt, int ldw, const float* bias, void* C,
                     int ldc, float* part, int M, int N, int K, int splits, int k_per_split, int epi,
@@ -1678,11 +1749,7 @@ int launch_skinny_v(const bf16* A, int lda, const bf16* W, const bf16* Wt, int l
                                       k_per_split, epi);
   }
   int rc = mf_launch_status();
-  if (rc == 0 && two_pass) {
-    dim3 g2(((epi == EPI_SWIGLU ? ldc : N) + 255) / 256, M);
-    skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, K, splits, epi, fused);
-    rc = mf_launch_status();
-  }
+  if (rc == 0 && two_pass) rc = launch_reduce(part, bias, C, ldc, M, N, K, splits, epi, fused, stream);
   return rc;
 }
 
@@ -1895,9 +1962,7 @@ MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, c
                      : launch_tile<128, 128, 64, 64>((const bf16*)A, lda, (const bf16*)W, ldw, nullptr, part, N, M,
                                                      N, K, EPI_F32, vec_ok, stream, splits, k_per_split);
   if (rc) return rc;
-  dim3 g2(((epi == EPI_SWIGLU ? ldc : N) + 255) / 256, M);
-  skinny_reduce_kernel<<<g2, 256, 0, stream>>>(part, bias, C, ldc, M, N, K, splits, epi, FusedNorm{});
-  return mf_launch_status();
+  return launch_reduce(part, bias, C, ldc, M, N, K, splits, epi, FusedNorm{}, stream);
 }
 
 // The register-resident kernel for the shapes it is built for (K = 256 NS with enough tiles to
