@@ -17,8 +17,7 @@ from ..cache.paged import v_page_shape
 
 PAGE = 64          # tokens per cache page (MF_PAGE in csrc/common.h)
 HAVE_PREFILL_ATTENTION = True
-PREFILL_BLOCK = 128     # query tokens per workgroup of the prompt attention kernel
-PREFILL_MAX_SHARES = 8  # workgroups that may take the pages of one such block of queries in turn
+PREFILL_MAX_SHARES = 8  # workgroups that may take the pages of one block of queries of the prompt attention in turn
 PREFILL_MIN_PAGES = 4   # ... each with at least this many pages
 EPI_F32, EPI_ACC_F32, EPI_BF16, EPI_SWIGLU = 0, 1, 2, 3
 
@@ -76,8 +75,10 @@ _PROTOTYPES = {
     },
     "attn_prefill_bf16": {
         "mf_attn_prefill_bf16": [_P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, c_int,
-                                 c_int, c_float, c_int, _P],
+                                 c_int, c_int, c_int, c_float, c_int, _P],
         "mf_attn_prefill_part_floats": [c_int],
+        "mf_attn_prefill_rows": [c_int],
+        "mf_attn_prefill_per_cu": [c_int],
     },
     "sampling": {
         "mf_argmax": [_P, c_int, c_int, c_int, _P, _P, c_int, _P],
@@ -855,6 +856,16 @@ def attn_decode_rope(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, kc
         float(scale), int(window or 0), n_splits, base, 1 if write_kv else 0, _stream()), "attn_decode_rope_bf16")
 
 
+def prefill_tile(n_heads: int, n_kv_heads: int, head_dim: int):
+    """(tq, gh, workgroups per block of queries): a workgroup of the prompt attention takes `gh` heads
+    of a kv head's group (all of them, unless there are more than it has rows) times `tq` consecutive
+    new tokens, so that a page of keys it brings in serves every head that reads it."""
+    rows = _fn("attn_prefill_bf16", "mf_attn_prefill_rows")(head_dim)
+    group = n_heads // n_kv_heads
+    gh = min(group, rows)
+    return rows // gh, gh, n_kv_heads * (-(-group // gh))
+
+
 def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, page_table: torch.Tensor,
                  ctx, out: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  window: int) -> None:
@@ -879,24 +890,26 @@ def attn_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, pa
                           f"{ctx.n_seqs} sequences of up to {ctx.max_len} positions")
     # Where the kernel's time is that of the block with the most pages (a few new tokens on a long
     # context, few short prompts), blocks of queries with more pages than a workgroup's even share
-    # of all of them (two workgroups fit a CU) are given to several workgroups, which take the
-    # pages in turn.
+    # of all of them (two workgroups fit a CU up to a head size of 128) are given to several
+    # workgroups, which take the pages in turn.
     window = int(window or 0)
+    tq, gh, per_tile = prefill_tile(n_heads, n_kv_heads, head_dim)
+    per_cu = _fn("attn_prefill_bf16", "mf_attn_prefill_per_cu")(head_dim)
     shared = None if tuning.NO_SHARED_PAGES else ctx.shared_query_tiles(
-        PREFILL_BLOCK, PAGE, window, n_heads, cu_count(), 2, PREFILL_MIN_PAGES, PREFILL_MAX_SHARES)
+        tq, PAGE, window, per_tile, cu_count(), per_cu, PREFILL_MIN_PAGES, PREFILL_MAX_SHARES)
     if shared is None:
-        tile_seq, tile_q0 = ctx.query_tiles(PREFILL_BLOCK)
+        tile_seq, tile_q0 = ctx.query_tiles(tq)
         tile_share = parts = arrived = None
     else:
         tile_seq, tile_q0, tile_share, n_slots, most_shares = shared
         part = _fn("attn_prefill_bf16", "mf_attn_prefill_part_floats")(head_dim)
-        parts = workspace("prefill_parts", n_slots * n_heads * most_shares * part, q.device)
-        arrived = _zeroed_counters("prefill_arrived", n_slots * n_heads, q.device)
+        parts = workspace("prefill_parts", n_slots * per_tile * most_shares * part, q.device)
+        arrived = _zeroed_counters("prefill_arrived", n_slots * per_tile, q.device)
     rc = _fn("attn_prefill_bf16", "mf_attn_prefill_bf16")(
         _ptr(q), _ptr(kcache), _ptr(vcache), _ptr(page_table), page_table.shape[1], _ptr(ctx.cu_seqlens),
         _ptr(ctx.start_pos), _ptr(tile_seq), _ptr(tile_q0), _ptr(tile_share), _ptr(parts), _ptr(arrived),
-        most_shares if shared is not None else 1, _ptr(out), tile_seq.numel(), n_heads, n_kv_heads, head_dim, float(scale), window,
-        _stream())
+        most_shares if shared is not None else 1, _ptr(out), tile_seq.numel(), n_heads, n_kv_heads, head_dim,
+        gh, tq, float(scale), window, _stream())
     if rc != 0 and arrived is not None:
         arrived.zero_()                  # a launch that failed may have left workgroups counted in
     _check(rc, "attn_prefill_bf16")

@@ -518,10 +518,11 @@ def prefill_case(nh, nk, hd, new, start, seed):
 
 @pytest.mark.parametrize("nh,nk,hd,window", [(4, 2, 16, 0), (4, 1, 32, 0), (9, 3, 48, 0), (28, 4, 128, 0),
                                              (6, 6, 64, 0), (10, 2, 80, 0), (4, 2, 256, 0), (4, 2, 64, 40),
-                                             (7, 1, 128, 200), (4, 4, 112, 0)])
+                                             (7, 1, 128, 200), (4, 4, 112, 0), (12, 1, 64, 0), (130, 1, 16, 0)])
 def test_attn_prefill(ops, nh, nk, hd, window):
-    # new tokens per sequence straddle the 32/128 tiles and the 64-key pages; two sequences
-    # continue from a cache that already holds tokens
+    # new tokens per sequence straddle the blocks of queries (128 rows of (token, head of the group):
+    # 128, 64, 42, 32, 25, 18 or 10 tokens; a group of 130 heads takes two workgroups a token) and the
+    # 64-key pages; two sequences continue from a cache that already holds tokens
     new = [1, 5, 31, 33, 64, 65, 127, 129, 300, 70]
     start = [0, 0, 0, 0, 0, 0, 0, 0, 0, 150]
     q, kc, vc, table, ctx_on = prefill_case(nh, nk, hd, new, start, 21)
@@ -549,11 +550,12 @@ def test_attn_prefill_shared_pages(ops, nh, nk, hd, window):
     one adds up (one sequence continues from 600 cached tokens; the short one stays whole)."""
     new, start = [1500, 260, 40], [600, 0, 0]
     q, kc, vc, table, ctx_on = prefill_case(nh, nk, hd, new, start, 23)
-    shared = ctx_on("cpu").shared_query_tiles(ops.PREFILL_BLOCK, ops.PAGE, window, nh, 256, 2, ops.PREFILL_MIN_PAGES,
+    tq, gh, per_tile = ops.prefill_tile(nh, nk, hd)
+    shared = ctx_on("cpu").shared_query_tiles(tq, ops.PAGE, window, per_tile, 256, 2, ops.PREFILL_MIN_PAGES,
                                               ops.PREFILL_MAX_SHARES)
     assert shared is not None
     words = shared[2].tolist()
-    assert max((w >> 8) & 255 for w in words) == (8 if window == 0 else 5)     # 33 pages, or the window's 16
+    assert max((w >> 8) & 255 for w in words) == (8 if window == 0 else 4)     # 33 pages, or the 16 a window and a block of queries span
     by_slot = {}
     for w in words:
         if w:
