@@ -442,13 +442,16 @@ def skinny_plan(m: int, n: int, k: int, target_blocks: Optional[int] = None,
     register-resident kernel does not hold, where it does badly from 9 rows on (every block reads
     its own copy of the activations from L2; from 13 rows on where it reads the tiled copy of the
     weights: the down product of the 7B shape at 12 rows 28.9 us against 29.9, at 16 rows 32.4
-    against 30.4) and where a CU's share of the weight rows fills its 16-row tiles poorly."""
+    against 30.4) and where a CU's share of the weight rows fills its 16-row tiles poorly, unless
+    the matrix is small (the down product of the 3B shape, 2048 x 11008, at 8 rows: 13.5 us in one
+    kernel, half-filled tiles and all, against 15.0 in two; at 16 rows 17.1 against 15.4)."""
     if target_blocks is None:
         target_blocks = tuning.SKINNY_TARGET or cu_count()
     if m <= 16:
         share = (n + target_blocks - 1) // target_blocks          # weight rows of a block in the one-kernel form
         fill = share / float((share + 15) // 16 * 16)
-        if k < 8192 or (m <= (12 if tiled else 8) and fill >= 0.8) or stationary_shape(n, k, swiglu):
+        small = m <= 8 and n * k <= 24 << 20          # up to 48 MB of weights: the second kernel's few microseconds count
+        if k < 8192 or (m <= (12 if tiled else 8) and fill >= 0.8) or small or stationary_shape(n, k, swiglu):
             return 1, (k + 255) // 256 * 256
     n_blocks = (n + 127) // 128
     chunks = (k + 255) // 256
