@@ -60,7 +60,11 @@ struct Shape {
   static constexpr bool POW2 = (CPR & (CPR - 1)) == 0;
   static constexpr int KDIV = 16 / CPR > 1 ? 16 / CPR : 1;   // rows that share a swizzle (power-of-two CPR)
   static constexpr int KBYTES = KT * HD * 2;
-  static constexpr int VBYTES = 2 * HDP * KT;        // [2][HDP][32 keys], rows from HD on never written nor used
+  // V in LDS: [2][HDP][32 keys] in groups of 16 rows (a kilobyte, one copy instruction), every other
+  // group 8 bytes further on: the lanes of a fragment read take 8 bytes at the same place of rows d and
+  // d + 16, which would meet in one bank.  Rows from HD on are never written nor used.
+  static constexpr int VGROUP = 1024 + 16;
+  static constexpr int VBYTES = 2 * (HDP / 16) * VGROUP + 16;
   static constexpr int STAGE = KBYTES + VBYTES;
   static constexpr int NI = (CPR + NW - 1) / NW;     // copies per wave and page, of K and of V each
   static constexpr bool SURPLUS = CPR % NW != 0;     // some waves' last copy has no chunk: it goes to a dump
@@ -162,7 +166,8 @@ __global__ __launch_bounds__(Shape<NKS>::NW * 64, Shape<NKS>::PER_CU) void attn_
     // V: rows (half, d) of 64 bytes, 16 an instruction; chunk position lane % 4 holds chunk (lane % 4) ^ ((d >> 2) & 3)
     const int R = 16 * ii + (lane >> 2), half = R / HD, d = R - half * HD;
     voff[n] = (unsigned)((half * HD + d) * 4 + ((lane & 3) ^ ((d >> 2) & 3))) * 16u;
-    vdst[n] = real[n] ? KBYTES + (half * HDP + (16 * ii - half * HD)) * 64 : NST * STAGE + wid * 1024;
+    const int group = half * (HDP / 16) + (16 * ii - half * HD) / 16;
+    vdst[n] = real[n] ? KBYTES + group * S::VGROUP + (group & 1) * 8 : NST * STAGE + wid * 1024;
   }
   auto issue = [&](int page, int stage) {
     const bf16* kp = kc + ((size_t)page * nk + hk) * KT * HD;
@@ -183,7 +188,8 @@ __global__ __launch_bounds__(Shape<NKS>::NW * 64, Shape<NKS>::PER_CU) void attn_
   // V^T: row d = 32 dt + ql of a half, the four keys 4 hf .. of chunk cl at position cl ^ ((ql >> 2) & 3)
   unsigned vaddr[4];
 #pragma unroll
-  for (int cl = 0; cl < 4; ++cl) vaddr[cl] = (unsigned)(KBYTES + (ql * 4 + (cl ^ ((ql >> 2) & 3))) * 16 + hf * 8);
+  for (int cl = 0; cl < 4; ++cl)
+    vaddr[cl] = (unsigned)(KBYTES + (ql >> 4) * (S::VGROUP + 8) + ((ql & 15) * 4 + (cl ^ ((ql >> 2) & 3))) * 16 + hf * 8);
 
   // this block's pages: first + share, first + share + n_shares, ...
   const int page_first = key_lo / KT + share, page_last = blk_p_hi / KT;
@@ -220,12 +226,16 @@ __global__ __launch_bounds__(Shape<NKS>::NW * 64, Shape<NKS>::PER_CU) void attn_
         const int cs = x & 3, R = x >> 2, half = R / HD, d = R - half * HD;
         const int k0 = half * 32 + (cs ^ ((d >> 2) & 3)) * 8;
         if (k0 + 8 > n_written) {
-          bf16x8* at = reinterpret_cast<bf16x8*>(st + KBYTES + ((half * HDP + d) * 4 + cs) * 16);
-          bf16x8 v = *at;
+          const int group = half * (HDP / 16) + d / 16;
+          bf16x4* at = reinterpret_cast<bf16x4*>(st + KBYTES + group * S::VGROUP + (group & 1) * 8 + ((d & 15) * 4 + cs) * 16);
+          bf16x4 v0 = at[0], v1 = at[1];
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (k0 + e >= n_written) v[e] = (bf16)0.f;
-          *at = v;
+          for (int e = 0; e < 4; ++e) {
+            if (k0 + e >= n_written) v0[e] = (bf16)0.f;
+            if (k0 + 4 + e >= n_written) v1[e] = (bf16)0.f;
+          }
+          at[0] = v0;
+          at[1] = v1;
         }
       }
       __syncthreads();
@@ -315,7 +325,7 @@ __global__ __launch_bounds__(Shape<NKS>::NW * 64, Shape<NKS>::PER_CU) void attn_
     bf16x4 v[VAHEAD + 1][2];
     auto read_v = [&](int i, int slot) {
       const int kg = i / NDT, dt = i % NDT;
-      const unsigned char* vrow = st + ((kg >> 1) * HDP + dt * 32) * 64;
+      const unsigned char* vrow = st + ((kg >> 1) * (HDP / 16) + dt * 2) * S::VGROUP;
       v[slot][0] = *reinterpret_cast<const bf16x4*>(vrow + vaddr[2 * (kg & 1)]);
       v[slot][1] = *reinterpret_cast<const bf16x4*>(vrow + vaddr[2 * (kg & 1) + 1]);
     };
