@@ -176,3 +176,26 @@ def test_shared_query_tiles_cover_every_page_once():
     assert ctx([2048], [0]).shared_query_tiles(128, 64, 0, 2, 256, 2, 4, 8) is not None
     assert ctx([128] * 8, [2000] * 8).shared_query_tiles(128, 64, 0, 28, 256, 2, 4, 8) is None
     assert ctx([512], [4096]).shared_query_tiles(128, 64, 0, 28, 256, 2, 4, 8) is not None
+
+
+def test_prefill_tile_takes_a_group_of_heads_together():
+    """Rows of the prompt attention are (token, head of the kv group) pairs, 128 a workgroup: as many
+    whole tokens as fit beside all heads of the group; a group with more heads than rows goes in chunks."""
+    assert ops.prefill_tile(28, 4, 128) == (18, 7, 4)          # the 7B shape: 126 of 128 rows in use
+    assert ops.prefill_tile(6, 6, 64) == (128, 1, 6)           # one head a group: 128 tokens
+    assert ops.prefill_tile(64, 8, 128) == (16, 8, 8)
+    assert ops.prefill_tile(40, 8, 256) == (25, 5, 8)
+    assert ops.prefill_tile(130, 1, 16) == (1, 128, 2)         # 130 heads: a token's heads in two workgroups
+    for nh, nk, hd in itertools.product((1, 3, 12, 28, 64, 300), (1, 2, 4), (16, 48, 128, 256)):
+        if nh % nk:
+            continue
+        tq, gh, per_tile = ops.prefill_tile(nh, nk, hd)
+        group = nh // nk
+        assert 1 <= gh <= group and tq >= 1 and tq * gh <= 128
+        assert per_tile == nk * -(-group // gh)
+
+
+def test_skinny_plan_keeps_a_small_matrix_in_one_kernel():
+    assert ops.skinny_plan(8, 2048, 11008, target_blocks=256, tiled=True)[0] == 1      # the 3B shape's down product
+    assert ops.skinny_plan(16, 2048, 11008, target_blocks=256, tiled=True)[0] > 1
+    assert ops.skinny_plan(8, 5120, 13824, target_blocks=256, tiled=True)[0] > 1       # the 14B shape's: 141 MB
