@@ -10,10 +10,10 @@ the pool is sized in tokens (each sequence rounded up to whole pages), not in sl
 context.  The same rule makes reuse safe: a page's old rows are never read, because a
 sequence reads positions below its own length only and writes each before reading it.
 
-Layers with the same needs (kv heads, head size, window) form a group with storage of its
-own: one K tensor `[entries][pages][kv_heads][64][head_dim]`, one V tensor (the same shape in
-32-bit, `[entries][pages][kv_heads][2][head_dim][32]` in bfloat16, see `v_page_shape`) and one
-page pool.
+Layers with the same needs (kv heads, head size, window, value width) form a group with storage
+of its own: one K tensor `[entries][pages][kv_heads][64][head_dim]`, one V tensor (the same shape
+in 32-bit, `[entries][pages][kv_heads][2][head_dim][32]` in bfloat16, see `v_page_shape`; with the
+request's own value width where it names one) and one page pool.
 A group with a window gives pages back as soon as every position in them has left the
 window of all later queries.
 """
@@ -54,6 +54,11 @@ class KVRequest:
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None      # None: all earlier positions
+    v_head_dim: Optional[int] = None  # width of a value row where it is not that of a key row
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
 @dataclass(frozen=True)
@@ -104,7 +109,7 @@ class KVGroup:
         self.pool = PagePool(n_pages)
         self.k = torch.empty((len(entries), n_pages, request.n_kv_heads, PAGE, request.head_dim),
                              dtype=dtype, device=device)
-        self.v = torch.empty((len(entries), n_pages) + v_page_shape(request.n_kv_heads, request.head_dim, dtype),
+        self.v = torch.empty((len(entries), n_pages) + v_page_shape(request.n_kv_heads, request.value_dim, dtype),
                              dtype=dtype, device=device)
         if poison:
             self.k.fill_(float("nan"))
@@ -268,6 +273,10 @@ class Cache:
         from ..kernels import ops
         k, v, group = self.kv(entry)
         req = group.request
+        if req.value_dim != req.head_dim:
+            raise CacheError(f"store_kv writes keys and values of one width; entry {entry} asks for keys of "
+                             f"{req.head_dim} and values of {req.value_dim}: a mixer with a value width of its own "
+                             "writes its rows into the pages of `kv(entry)` with a kernel of its own")
         ops.rope_kvwrite(qkv, None, None, ctx.positions, ctx.seq_of_tok, ctx.page_table(group), q_out, k, v,
                          n_heads, req.n_kv_heads, req.head_dim, True)
 

@@ -41,7 +41,7 @@ def cache_bytes_per_token(requests: Dict[int, object], dtype: torch.dtype) -> in
     """Bytes one token of one sequence takes in the cache: K and V of every entry."""
     from ..cache.paged import KVRequest
     elem = torch.empty((), dtype=dtype).element_size()
-    return sum(2 * r.n_kv_heads * r.head_dim * elem for r in requests.values() if isinstance(r, KVRequest))
+    return sum(r.n_kv_heads * (r.head_dim + r.value_dim) * elem for r in requests.values() if isinstance(r, KVRequest))
 
 
 def state_bytes_per_sequence(requests: Dict[int, object]) -> int:

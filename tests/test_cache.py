@@ -41,6 +41,24 @@ def test_groups_have_storage_of_their_own():
     assert k0.shape == (8, 2, PAGE, 16) and k0.data_ptr() != k1.data_ptr() and g is full
 
 
+def test_values_may_have_a_width_of_their_own():
+    """An entry may ask for value rows of another width than its key rows: its group's V pages have
+    that width (in both layouts), sizing counts it, and the built-in write, which takes one width,
+    refuses the entry instead of writing rows of the wrong size."""
+    from minfer_amd.engine.engine import cache_bytes_per_token
+    reqs = {0: KVRequest(2, 16), 1: KVRequest(2, 16, v_head_dim=24), 2: KVRequest(2, 16, v_head_dim=16)}
+    assert reqs[0] != reqs[1] and reqs[1].value_dim == 24 and reqs[0].value_dim == 16
+    c = Cache(reqs, 64 * 4, 2, torch.float32, "cpu")
+    assert len(c.groups) == 3 or c.group_of[0] is not c.group_of[1]
+    k, v, g = c.kv(1)
+    assert k.shape == (4, 2, PAGE, 16) and v.shape == (4, 2, PAGE, 24)
+    b = Cache(reqs, 64 * 4, 2, torch.bfloat16, "cpu")
+    assert b.kv(1)[1].shape == (4, 2, 2, 24, PAGE // 2) and b.kv(0)[1].shape == (4, 2, 2, 16, PAGE // 2)
+    assert cache_bytes_per_token(reqs, torch.float32) == (2 * 32 + 2 * 40 + 2 * 32) * 4
+    with pytest.raises(CacheError, match="value width of its own"):
+        c.store_kv(1, torch.zeros(1, 4 * 16), None, 2, torch.zeros(1, 2 * 16))
+
+
 def test_slots_are_given_back_and_used_again():
     c = make(max_seqs=2)
     a, b = c.alloc_slot(), c.alloc_slot()
