@@ -518,7 +518,8 @@ def prefill_case(nh, nk, hd, new, start, seed):
 
 @pytest.mark.parametrize("nh,nk,hd,window", [(4, 2, 16, 0), (4, 1, 32, 0), (9, 3, 48, 0), (28, 4, 128, 0),
                                              (6, 6, 64, 0), (10, 2, 80, 0), (4, 2, 256, 0), (4, 2, 64, 40),
-                                             (7, 1, 128, 200), (4, 4, 112, 0), (12, 1, 64, 0), (130, 1, 16, 0)])
+                                             (7, 1, 128, 200), (4, 4, 112, 0), (12, 1, 64, 0), (130, 1, 16, 0),
+                                             (2, 1, 96, 0), (2, 2, 160, 0), (3, 1, 192, 70), (2, 1, 240, 0)])
 def test_attn_prefill(ops, nh, nk, hd, window):
     # new tokens per sequence straddle the blocks of queries (128 rows of (token, head of the group):
     # 128, 64, 42, 32, 25, 18 or 10 tokens; a group of 130 heads takes two workgroups a token) and the
