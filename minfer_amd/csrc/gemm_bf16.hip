@@ -880,6 +880,73 @@ bool ring_takes(bool aligned, int K, int splits, int k_per_split) {
   return aligned && K % 256 == 0 && (long)(splits - 1) * k_per_split < K;
 }
 
+// The RMS norm folded around the products of at most 64 rows, across two kernels (y = x /
+// sqrt(mean(x^2) + eps) * g, src/vec_ops.rs:500-522):
+//  * a product that adds into the residual stream x and knows the weight g of the norm that reads
+//    the stream next leaves, beside the stream's new rows, xg = bf16(x g) and for every row the
+//    sums of x^2 in parts (`out_*`): over runs of 256 columns where the kernel that adds the parts
+//    of a K split does it (17 to 64 rows: it has every new value of x in its hands), one part per
+//    block where a one-kernel product of at most 16 rows does it in its epilogue (every block
+//    owns some columns; `out_parts` places a row, the ones past the grid set to zero);
+//  * the product that follows takes xg as its activations and multiplies its own sums by the
+//    row's 1 / sqrt(sum / K + eps) in its epilogue (`in_*`), the partial sums of squares added up
+//    in their order.
+// No norm kernel, no pass over the stream between the two products.  The same arithmetic as the
+// fold of the register-resident kernel above (bf16(x g) to the matrix cores, the row's factor in
+// the epilogue).
+constexpr int MF_NOT_BUILT = -2;     // an entry point's answer for a shape it has no kernel for; nothing was launched
+
+struct FusedNorm {
+  const float* in_ssq;     // [M][in_parts] partial sums of squares of the rows this product reads (null: none)
+  int in_parts;
+  float in_eps;
+  const float* out_g;      // [N] weight of the norm that reads the output next (null: none)
+  bf16* out_xg;            // [M][N]
+  float* out_ssq;          // [M][ceil(N / 256)], or [M][out_parts] from a one-kernel product of at most 16 rows
+  int out_parts;
+};
+
+// 1 / sqrt(mean(x^2) + eps) of NR rows from their partial sums, K the rows' length, in two steps
+// so that a kernel can ask for the sums early and use them late; all lanes of a wave call both with
+// the same rows (a row outside [0, M) gives 1).  The lanes take the partial sums between them, all
+// rows' loads in flight together, and add up in a fixed tree.
+template <int NR>
+__device__ __forceinline__ void row_sums_ask(const FusedNorm& f, const int (&rows)[NR], int M, int lane, float (&t)[NR]) {
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    t[i] = 0.f;
+    if (rows[i] >= 0 && rows[i] < M)
+      for (int p = lane; p < f.in_parts; p += 64) t[i] += f.in_ssq[(size_t)rows[i] * f.in_parts + p];
+  }
+}
+
+template <int NR>
+__device__ __forceinline__ void row_factors_of(const FusedNorm& f, const int (&rows)[NR], int M, int K, float (&t)[NR]) {
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) t[i] += __shfl_xor(t[i], o, MF_WAVE);
+    t[i] = (rows[i] >= 0 && rows[i] < M) ? 1.0f / sqrtf(t[i] / (float)K + f.in_eps) : 1.f;
+  }
+}
+
+
+// End of a one-kernel product of at most 16 rows that prepares the next norm (FusedNorm::out_*):
+// every lane has the squares of its own outputs of row e_m in `sq` (0 where it has none), the
+// COLS lanes of a row sit side by side; their sum is this block's part of the row.  Block 0 also
+// sets the places past the grid to zero.
+template <int COLS>
+__device__ __forceinline__ void norm_part_out(const FusedNorm& f, float sq, int e_m, int e_c, int M) {
+#pragma unroll
+  for (int o = COLS / 2; o > 0; o >>= 1) sq += __shfl_xor(sq, o, MF_WAVE);
+  if (e_c == 0 && e_m < M) f.out_ssq[(size_t)e_m * f.out_parts + blockIdx.x] = sq;
+  if (blockIdx.x == 0) {
+    const int spare = f.out_parts - (int)gridDim.x;
+    for (int i = threadIdx.x; i < M * spare; i += blockDim.x)
+      f.out_ssq[(size_t)(i / spare) * f.out_parts + gridDim.x + i % spare] = 0.f;
+  }
+}
+
 // The same split of the work as skinny16_kernel (a block owns 16 NT weight rows, its waves split
 // K), for aligned operands and K a multiple of 32, with the loads rolling: a wave holds S steps
 // of weights and activations in registers, and the refill of a register is issued right behind
@@ -892,7 +959,8 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
                                                             const bf16* __restrict__ W, int ldw,
                                                             const float* __restrict__ bias,
                                                             void* __restrict__ C, int ldc, int M, int N,
-                                                            int K, int steps_per_wave, int epi, int rpb) {
+                                                            int K, int steps_per_wave, int epi, int rpb,
+                                                            FusedNorm fused) {
   constexpr int COLS = 16 * NT;
   constexpr int RS = COLS + 4;
   constexpr int WSTEP = TILED ? 512 : 32;
@@ -930,8 +998,9 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
   const int e_n = tile_row(e_c >> 4) + (e_c & 15);
   const int e_m = wid * ROWS_PER_PASS + lane / COLS;
   const bool e_mine = e_m < M && e_n < N && (PAIR || e_c < rpb);
-  float c_old = 0.f;
+  float c_old = 0.f, e_g = 0.f;
   if (epi == EPI_ACC_F32 && e_mine) c_old = ((const float*)C)[(size_t)e_m * ldc + e_n];
+  if (fused.out_g && e_mine) e_g = fused.out_g[e_n];       // the next norm's weight, where this product prepares it
   const int R = T / S, rem = T % S;
   if (R == 0) {       // a slice shorter than the registers hold: step by step
     for (int s = 0; s < T; ++s) {
@@ -1001,17 +1070,25 @@ __global__ __launch_bounds__(NW * 64) void rolling16_kernel(const bf16* __restri
     }
     return;
   }
-  if (!e_mine) return;
-  float v = bias ? bias[e_n] : 0.f;
+  float sq = 0.f;
+  if (e_mine) {
+    float v = bias ? bias[e_n] : 0.f;
 #pragma unroll
-  for (int ww = 0; ww < NW; ++ww) v += red[ww][e_m][e_c];
-  if (epi == EPI_ACC_F32) ((float*)C)[(size_t)e_m * ldc + e_n] = c_old + v;
-  else store_out(C, ldc, e_m, e_n, v, epi);
+    for (int ww = 0; ww < NW; ++ww) v += red[ww][e_m][e_c];
+    if (epi == EPI_ACC_F32) v += c_old;
+    if (epi == EPI_ACC_F32) ((float*)C)[(size_t)e_m * ldc + e_n] = v;
+    else store_out(C, ldc, e_m, e_n, v, epi);
+    if (fused.out_g) {
+      fused.out_xg[(size_t)e_m * ldc + e_n] = (bf16)(v * e_g);
+      sq = v * v;
+    }
+  }
+  if (fused.out_g) norm_part_out<COLS>(fused, sq, e_m, e_c, M);
 }
 
 template <int NW, int NT, int S, bool PAIR = false, bool TILED = false>
 int launch_rolling16(const bf16* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
-                     int M, int N, int K, int epi, hipStream_t stream) {
+                     int M, int N, int K, int epi, hipStream_t stream, const FusedNorm& fused = FusedNorm{}) {
   const int steps_per_wave = (K / 32 + NW - 1) / NW;
   int rpb = 16 * NT, blocks = N / 32;
   if (!PAIR) {
@@ -1021,8 +1098,9 @@ int launch_rolling16(const bf16* A, int lda, const bf16* W, int ldw, const float
     rpb = rpb < 1 ? 1 : (rpb > 16 * NT ? 16 * NT : rpb);
     blocks = (N + rpb - 1) / rpb;
   }
+  if (fused.out_g && (PAIR || blocks > fused.out_parts)) return MF_NOT_BUILT;
   rolling16_kernel<NW, NT, S, PAIR, TILED><<<blocks, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K,
-                                                                           steps_per_wave, epi, rpb);
+                                                                           steps_per_wave, epi, rpb, fused);
   return mf_launch_status();
 }
 
@@ -1074,13 +1152,14 @@ __global__ __launch_bounds__(NW * 64) void stationary16_kernel(const void* __res
                                                                const float* __restrict__ bias,
                                                                void* __restrict__ C, int ldc, int M, int N,
                                                                int cols_total, int unit, int share, int extra, int epi,
-                                                               NormArgs norm) {
+                                                               NormArgs norm, FusedNorm fused) {
   constexpr int KK = NW * NS * 32;         // K
   constexpr int WSTEP = TILED ? 512 : 32;  // elements from one step's weights to the next's
   constexpr int COLS = 16 * NT;            // weight rows (output columns) of an item
   constexpr int RS = COLS + 4;             // row stride of the sums in LDS: conflict-free writes
   __shared__ float red[2][NW][16][RS];     // [buffer][wave][activation row][weight row of the item]
   __shared__ float ssq[NW][16];            // NORM: sum of x^2 over a wave's slice, per activation row
+  __shared__ float rfac[16];               // not NORM: the rows' factors of a norm prepared by the product before (1 where none)
   extern __shared__ __attribute__((aligned(16))) float gs[];   // NORM: the norm's weight, K floats
   static_assert(NS % RING == 0, "the ring divides a slice");
   static_assert(PAIR ? NW * 4 >= 16 : NW * (64 / COLS) >= 16, "an epilogue pass for every activation row");
@@ -1207,10 +1286,30 @@ __global__ __launch_bounds__(NW * 64) void stationary16_kernel(const void* __res
     const bf16* arow = (const bf16*)Av + (size_t)min(r16, M - 1) * lda + k0;
 #pragma unroll
     for (int s = 0; s < NS; ++s) afr[s] = *reinterpret_cast<const bf16x8*>(arow + s * 32);
+  }
+  // Not NORM: the activations may be bf16(x g) of rows whose sums of squares the product before has
+  // left in parts (FusedNorm::in_*): wave w adds up rows w, w + NW, ..., asked for here, between the
+  // activations and the first weights, and used behind them; the epilogue multiplies by the factors.
+  constexpr int FR = (16 + NW - 1) / NW;
+  int frow[FR];
+  float ffac[FR];
+#pragma unroll
+  for (int i = 0; i < FR; ++i) frow[i] = (!NORM && fused.in_ssq && wid + NW * i < 16) ? wid + NW * i : -1;
+  if constexpr (!NORM) {
+    row_sums_ask<FR>(fused, frow, M, lane, ffac);
+    __builtin_amdgcn_sched_barrier(0);
     first_loads(0);
   }
 #pragma unroll
   for (int j = 1; j < NT; ++j) first_loads(j);
+  if constexpr (!NORM) {
+    row_factors_of<FR>(fused, frow, M, KK, ffac);
+    if (lane == 0)
+#pragma unroll
+      for (int i = 0; i < FR; ++i)
+        if (wid + NW * i < 16) rfac[wid + NW * i] = ffac[i];       // read behind the first item's barrier
+  }
+  float sq = 0.f;                      // a product that prepares the next norm: squares of this lane's outputs
   for (int it = 0; it < n_items; ++it) {
     // The loop body has no branch, so that the compiler can count the loads in flight and wait
     // for the oldest one only: behind the last item the loads go to the head of the matrix,
@@ -1233,11 +1332,12 @@ __global__ __launch_bounds__(NW * 64) void stationary16_kernel(const void* __res
     const int e_n = c0 + e_c;
     const int e_m = wid * (64 / COLS) + lane / COLS;
     const bool e_mine = !PAIR && e_n < c_end && e_m < M;
-    float c_old = 0.f, e_bias = 0.f;
+    float c_old = 0.f, e_bias = 0.f, e_g = 0.f;
     if constexpr (!PAIR) {
       const float* dummy = reinterpret_cast<const float*>(W);
       c_old = *((e_mine && epi == EPI_ACC_F32) ? (const float*)C + (size_t)e_m * ldc + e_n : dummy);
       e_bias = *((e_mine && bias) ? bias + e_n : dummy);
+      e_g = *((e_mine && fused.out_g) ? fused.out_g + e_n : dummy);
     }
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -1255,7 +1355,7 @@ __global__ __launch_bounds__(NW * 64) void stationary16_kernel(const void* __res
         __builtin_amdgcn_sched_barrier(0);      // keep "use a register, then refill it" in this order
       }
       // (held here, or the compiler moves the two loads to where they are used)
-      if (s == 0) asm volatile("" : "+v"(c_old), "+v"(e_bias));
+      if (s == 0) asm volatile("" : "+v"(c_old), "+v"(e_bias), "+v"(e_g));
     }
 #pragma unroll
     for (int j = 0; j < NT; ++j) wcur[j] = wrow[j];
@@ -1282,11 +1382,9 @@ __global__ __launch_bounds__(NW * 64) void stationary16_kernel(const void* __res
         float g = 0.f, u = 0.f;
 #pragma unroll
         for (int ww = 0; ww < NW; ++ww) { g += red[buf][ww][m][r16]; u += red[buf][ww][m][16 + r16]; }
-        if constexpr (NORM) {
-          const float sc = row_scale(m);
-          g *= sc;
-          u *= sc;
-        }
+        const float sc = NORM ? row_scale(m) : rfac[m];
+        g *= sc;
+        u *= sc;
         ((bf16*)C)[(size_t)m * ldc + col] = (bf16)swiglu_f(g, u);
       }
     } else {
@@ -1294,19 +1392,26 @@ __global__ __launch_bounds__(NW * 64) void stationary16_kernel(const void* __res
         float v = 0.f;
 #pragma unroll
         for (int ww = 0; ww < NW; ++ww) v += red[buf][ww][e_m][e_c];
-        if constexpr (NORM) v *= row_scale(e_m);
+        v *= NORM ? row_scale(e_m) : rfac[e_m];
         v += (bias ? e_bias : 0.f);
-        if (epi == EPI_ACC_F32) ((float*)C)[(size_t)e_m * ldc + e_n] = c_old + v;
+        if (epi == EPI_ACC_F32) v += c_old;
+        if (epi == EPI_ACC_F32) ((float*)C)[(size_t)e_m * ldc + e_n] = v;
         else store_out(C, ldc, e_m, e_n, v, epi);
+        if (fused.out_g) {
+          fused.out_xg[(size_t)e_m * ldc + e_n] = (bf16)(v * e_g);
+          sq = fmaf(v, v, sq);
+        }
       }
     }
   }
+  if constexpr (!PAIR)
+    if (fused.out_g) norm_part_out<COLS>(fused, sq, wid * (64 / COLS) + lane / COLS, lane % COLS, M);
 }
 
 // true when the shape is one the register-resident kernel is built for
 template <int NS, int NT, bool PAIR, bool TILED, int NW = 8>
 int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const float* bias, void* C, int ldc,
-                        int M, int N, int epi, const NormArgs* norm, hipStream_t stream) {
+                        int M, int N, int epi, const NormArgs* norm, const FusedNorm& fused, hipStream_t stream) {
   const int n_cu = cu_count();
   if (n_cu <= 0) return (int)hipErrorUnknown;
   const int cols_total = PAIR ? N / 2 : N;
@@ -1329,62 +1434,17 @@ int launch_stationary16(const void* A, int lda, const bf16* W, int ldw, const fl
       if (e != hipSuccess) return (int)e;
       configured = true;
     }
+    if (fused.in_ssq || fused.out_g) return MF_NOT_BUILT;
     kern<<<grid, NW * 64, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, cols_total, unit, units / grid, units % grid,
-                                      epi, *norm);
+                                      epi, *norm, FusedNorm{});
   } else {
+    if (fused.out_g && (PAIR || grid > fused.out_parts)) return MF_NOT_BUILT;
     stationary16_kernel<NS, RING, NT, PAIR, false, TILED, NW><<<grid, NW * 64, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N,
                                                                              cols_total, unit, units / grid,
                                                                              units % grid, epi,
-                                                                             NormArgs{nullptr, nullptr, 0.f});
+                                                                             NormArgs{nullptr, nullptr, 0.f}, fused);
   }
   return mf_launch_status();
-}
-
-// The RMS norm folded around the products of 17 to 64 rows, across two kernels (y = x /
-// sqrt(mean(x^2) + eps) * g, src/vec_ops.rs:500-522):
-//  * a product that adds into the residual stream x and knows the weight g of the norm that reads
-//    the stream next leaves, beside the stream's new rows, xg = bf16(x g) and for every row the
-//    sums of x^2 over runs of 256 columns (`out_*`; the kernel that adds the parts of a K split
-//    does it: it has every new value of x in its hands);
-//  * the product that follows takes xg as its activations and multiplies its own sums by the
-//    row's 1 / sqrt(sum / K + eps) in its epilogue (`in_*`), the partial sums of squares added up
-//    in their order.
-// No norm kernel, no pass over the stream between the two products.  The same arithmetic as the
-// fold of the register-resident kernel above (bf16(x g) to the matrix cores, the row's factor in
-// the epilogue).
-constexpr int MF_NOT_BUILT = -2;     // an entry point's answer for a shape it has no kernel for; nothing was launched
-
-struct FusedNorm {
-  const float* in_ssq;     // [M][in_parts] partial sums of squares of the rows this product reads (null: none)
-  int in_parts;
-  float in_eps;
-  const float* out_g;      // [N] weight of the norm that reads the output next (null: none)
-  bf16* out_xg;            // [M][N]
-  float* out_ssq;          // [M][ceil(N / 256)]
-};
-
-// 1 / sqrt(mean(x^2) + eps) of NR rows from their partial sums, K the rows' length, in two steps
-// so that a kernel can ask for the sums early and use them late; all lanes of a wave call both with
-// the same rows (a row outside [0, M) gives 1).  The lanes take the partial sums between them, all
-// rows' loads in flight together, and add up in a fixed tree.
-template <int NR>
-__device__ __forceinline__ void row_sums_ask(const FusedNorm& f, const int (&rows)[NR], int M, int lane, float (&t)[NR]) {
-#pragma unroll
-  for (int i = 0; i < NR; ++i) {
-    t[i] = 0.f;
-    if (rows[i] >= 0 && rows[i] < M)
-      for (int p = lane; p < f.in_parts; p += 64) t[i] += f.in_ssq[(size_t)rows[i] * f.in_parts + p];
-  }
-}
-
-template <int NR>
-__device__ __forceinline__ void row_factors_of(const FusedNorm& f, const int (&rows)[NR], int M, int K, float (&t)[NR]) {
-#pragma unroll
-  for (int i = 0; i < NR; ++i) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) t[i] += __shfl_xor(t[i], o, MF_WAVE);
-    t[i] = (rows[i] >= 0 && rows[i] < M) ? 1.0f / sqrtf(t[i] / (float)K + f.in_eps) : 1.f;
-  }
 }
 
 // 17 to 64 rows against a wide matrix (at least 8 tiles of 16 weight rows for every CU): one block
@@ -1631,7 +1691,10 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
     for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, MF_WAVE);
     if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = sq;
     __syncthreads();
-    if (threadIdx.x == 0) fused.out_ssq[(size_t)m * gridDim.x + blockIdx.x] = ((wsum[0] + wsum[1]) + wsum[2]) + wsum[3];
+    if (threadIdx.x == 0) fused.out_ssq[(size_t)m * fused.out_parts + blockIdx.x] = ((wsum[0] + wsum[1]) + wsum[2]) + wsum[3];
+    // (a row's places past the runs, where it has more of them: zero)
+    if (blockIdx.x == 0)
+      for (int p = gridDim.x + threadIdx.x; p < fused.out_parts; p += blockDim.x) fused.out_ssq[(size_t)m * fused.out_parts + p] = 0.f;
   }
 }
 
@@ -1686,7 +1749,9 @@ __global__ __launch_bounds__(256) void skinny_reduce4_kernel(const float* __rest
     float sq = ((v.x * v.x + v.y * v.y) + v.z * v.z) + v.w * v.w;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, MF_WAVE);
-    if ((threadIdx.x & 63) == 0) fused.out_ssq[(size_t)m * ((N + 255) / 256) + run] = sq;
+    if ((threadIdx.x & 63) == 0 && run < (N + 255) / 256) fused.out_ssq[(size_t)m * fused.out_parts + run] = sq;
+    if (blockIdx.x == 0 && threadIdx.x < 64)                 // (a row's places past its runs, where it has more of them: zero)
+      for (int p = (N + 255) / 256 + threadIdx.x; p < fused.out_parts; p += 64) fused.out_ssq[(size_t)m * fused.out_parts + p] = 0.f;
   }
 }
 
@@ -1968,23 +2033,24 @@ MF_API int mf_gemm_bf16_splitk(const void* A, int lda, const void* W, int ldw, c
 // The register-resident kernel for the shapes it is built for (K = 256 NS with enough tiles to
 // go round); MF_NOT_BUILT for any other, and nothing is launched.
 static int stationary16(const void* a, int lda, const bf16* w, const bf16* wt, int ldw, const float* bias, void* C,
-                        int ldc, int M, int N, int K, int epi, const NormArgs* norm, hipStream_t stream) {
+                        int ldc, int M, int N, int K, int epi, const NormArgs* norm, hipStream_t stream,
+                        const FusedNorm& fused = FusedNorm{}) {
   if (!stationary_takes(M, N, K, epi, norm != nullptr)) return MF_NOT_BUILT;
   // two tiles an item where a block's share is more than one: 128-byte rows of 32-bit output
   const int n_cu = cu_count();
   if (n_cu <= 0) return (int)hipErrorUnknown;
   const bool two = (N + n_cu - 1) / n_cu > 16;
 #define MF_STATIONARY_T(NS_, T_, W_)                                                                          \
-  (epi == EPI_SWIGLU ? launch_stationary16<NS_, 2, true, T_>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, stream) \
-   : two             ? launch_stationary16<NS_, 2, false, T_>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, stream) \
-                     : launch_stationary16<NS_, 1, false, T_>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, stream))
+  (epi == EPI_SWIGLU ? launch_stationary16<NS_, 2, true, T_>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, fused, stream) \
+   : two             ? launch_stationary16<NS_, 2, false, T_>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, fused, stream) \
+                     : launch_stationary16<NS_, 1, false, T_>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, fused, stream))
 #define MF_STATIONARY(NS_) \
   case NS_: return wt ? MF_STATIONARY_T(NS_, true, wt) : MF_STATIONARY_T(NS_, false, w);
   if (K == STATIONARY_K7) {
     // seven waves: one tile an item outside SwiGLU (the epilogue gives every wave 64 / (16 NT) rows)
 #define MF_STATIONARY_7(T_, W_)                                                                                  \
-  (epi == EPI_SWIGLU ? launch_stationary16<4, 2, true, T_, 7>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, stream) \
-                     : launch_stationary16<4, 1, false, T_, 7>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, stream))
+  (epi == EPI_SWIGLU ? launch_stationary16<4, 2, true, T_, 7>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, fused, stream) \
+                     : launch_stationary16<4, 1, false, T_, 7>(a, lda, W_, ldw, bias, C, ldc, M, N, epi, norm, fused, stream))
     return wt ? MF_STATIONARY_7(true, wt) : MF_STATIONARY_7(false, w);
 #undef MF_STATIONARY_7
   }
@@ -2011,12 +2077,16 @@ static int skinny_product(const void* A, int lda, const void* W, const void* Wt,
   const bf16* wt = (K % 32 == 0 && (uintptr_t)Wt % 16 == 0) ? (const bf16*)Wt : nullptr;
   const bool folds = fused.in_ssq || fused.out_g;
   const SkinnyChoice choice = skinny_choice(M, N, K, vec_ok, epi, splits, k_per_split, cu_count());
-  if (folds && M <= 16 && choice != SK_RING && choice != SK_STAGED) return MF_NOT_BUILT;
+  // at most 16 rows: the register-resident kernel takes a prepared norm and prepares the next one, the
+  // rolling kernel prepares the next one; the K-split kernels' second kernel counts its parts otherwise
+  if (folds && M <= 16 && choice != SK_STATIONARY && choice != SK_RING && choice != SK_STAGED &&
+      !(choice == SK_ROLLING && !fused.in_ssq))
+    return MF_NOT_BUILT;
   switch (choice) {
-    case SK_STATIONARY: return stationary16(a, lda, w, wt, ldw, bias, C, ldc, M, N, K, epi, nullptr, stream);
+    case SK_STATIONARY: return stationary16(a, lda, w, wt, ldw, bias, C, ldc, M, N, K, epi, nullptr, stream, fused);
     case SK_ROLLING:
-      return wt ? launch_rolling16<8, 1, 16, false, true>(a, lda, wt, ldw, bias, C, ldc, M, N, K, epi, stream)
-                : launch_rolling16<8, 1, 16>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream);
+      return wt ? launch_rolling16<8, 1, 16, false, true>(a, lda, wt, ldw, bias, C, ldc, M, N, K, epi, stream, fused)
+                : launch_rolling16<8, 1, 16>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, stream, fused);
     case SK_GUARDED_PAIR: return launch_skinny16<4, 2, 4, true>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case SK_GUARDED_4X2: return launch_skinny16<4, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
     case SK_GUARDED_8X2: return launch_skinny16<8, 2, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, epi, vec_ok, stream);
@@ -2044,19 +2114,24 @@ MF_API int mf_gemm_bf16_skinny(const void* A, int lda, const void* W, const void
 
 // The same with an RMS norm folded in on either side (see FusedNorm), for the shapes whose kernels
 // have a place for it (17 to 64 rows: the whole-K kernel on the reading side, the K-split kernels
-// with more than one split on both); MF_NOT_BUILT (-2), having launched nothing, for any other.
+// with more than one split on both; at most 16 rows: the register-resident kernel on both sides,
+// the rolling kernel on the writing side); MF_NOT_BUILT (-2), having launched nothing, for any other.
 //  * in_ssq [M][in_parts], in_eps: A holds bf16(x g) of rows x whose sums of squares these are; the
 //    product's sums are multiplied by the row's 1 / sqrt(sum / K + eps) before bias and epilogue.
-//  * out_g [N], out_xg [M][N] bf16, out_ssq [M][ceil(N / 256)]: beside C (32-bit, stored or added
-//    to), bf16(C g) and the sums of C^2 over runs of 256 columns are written.
+//  * out_g [N], out_xg [M][N] bf16, out_ssq [M][out_parts]: beside C (32-bit, stored or added
+//    to), bf16(C g) and the sums of C^2 in parts are written: over runs of 256 columns (out_parts =
+//    ceil(N / 256)) for 17 to 64 rows; for at most 16 rows one part per block of the product's one
+//    kernel, out_parts at least the number of CUs (the places past the grid are set to zero).
 MF_API int mf_gemm_bf16_skinny_fused(const void* A, int lda, const void* W, const void* Wt, int ldw,
                                      const float* bias, void* C, int ldc, float* part, int M, int N, int K,
                                      int splits, int k_per_split, int epi, const float* in_ssq, int in_parts,
                                      float in_eps, const float* out_g, void* out_xg, float* out_ssq,
-                                     hipStream_t stream) {
+                                     int out_parts, hipStream_t stream) {
   if (in_ssq && in_parts < 1) return (int)hipErrorInvalidValue;
-  if (out_g && (!out_xg || !out_ssq || (epi != EPI_F32 && epi != EPI_ACC_F32))) return (int)hipErrorInvalidValue;
-  const FusedNorm fused{in_ssq, in_parts, in_eps, out_g, (bf16*)out_xg, out_ssq};
+  if (out_g && (!out_xg || !out_ssq || out_parts < 1 || ldc != N || (epi != EPI_F32 && epi != EPI_ACC_F32)))
+    return (int)hipErrorInvalidValue;
+  if (out_g && out_parts < (N + 255) / 256) return (int)hipErrorInvalidValue;
+  const FusedNorm fused{in_ssq, in_parts, in_eps, out_g, (bf16*)out_xg, out_ssq, out_parts};
   return skinny_product(A, lda, W, Wt, ldw, bias, C, ldc, part, M, N, K, splits, k_per_split, epi, fused, stream);
 }
 

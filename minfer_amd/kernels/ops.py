@@ -59,7 +59,7 @@ _PROTOTYPES = {
         "mf_gemm_bf16_normed": [_P, c_int, _P, _P, c_float, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int,
                                 c_int, _P],
         "mf_gemm_bf16_skinny_fused": [_P, c_int, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int,
-                                      c_int, c_int, _P, c_int, c_float, _P, _P, _P, _P],
+                                      c_int, c_int, _P, c_int, c_float, _P, _P, _P, c_int, _P],
         "mf_gemm_bf16_plan": [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_char_p, c_int],
         "mf_gemm_bf16_tile_plan": [c_int, c_int, c_int, c_int, c_int, c_int, _P],
     },
@@ -670,20 +670,24 @@ def linear_normed(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, row_id
 NORM_SUM_RUN = 256       # columns a partial sum of squares covers (a block of the kernel that adds a K split's parts)
 
 
-def norm_sum_parts(n: int) -> int:
-    """Partial sums of squares a row of `n` values comes with (see `linear_fused`)."""
-    return (n + NORM_SUM_RUN - 1) // NORM_SUM_RUN
+def norm_sum_parts(n: int, m: int = 64) -> int:
+    """Partial sums of squares a row of `n` values comes with from a product of `m` rows (see
+    `linear_fused`): one per run of 256 columns from 17 rows on (the kernel that adds the parts of a K
+    split writes them), one per workgroup of the product's one kernel for at most 16 rows."""
+    return cu_count() if m <= 16 else (n + NORM_SUM_RUN - 1) // NORM_SUM_RUN
 
 
 def linear_fused(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                  accumulate: bool = False, tiled: Optional[torch.Tensor] = None, swiglu: bool = False,
                  scale_in=None, norm_out=None) -> bool:
-    """A bfloat16 product of at most 64 rows with an RMS norm folded in on either side, for steps of
-    17 to 64 tokens, where the norm would otherwise be a kernel of its own between two products:
+    """A bfloat16 product of at most 64 rows with an RMS norm folded in on either side, across two
+    products: the norm is no kernel of its own between them (17 to 64 rows), and the product behind
+    it reads its activations in bfloat16, half the bytes, with nothing to convert (at most 16 rows,
+    where the norm is otherwise folded into that product's prologue):
 
-    * `norm_out` = (g `[n]`, xg `[m][n]` bfloat16, sums `[m][norm_sum_parts(n)]`): the product stores
+    * `norm_out` = (g `[n]`, xg `[m][n]` bfloat16, sums `[m][norm_sum_parts(n, m)]`): the product stores
       or adds into the 32-bit `out` as `linear` does and leaves, beside it, bf16(out g) and the sums
-      of out^2 over runs of 256 columns, for the norm with weight g that reads `out` next;
+      of out^2 in parts, for the norm with weight g that reads `out` next;
     * `scale_in` = (sums `[m][parts]`, eps): `x` is such an xg, and the product's sums are multiplied
       by the row's 1 / sqrt(sum / k + eps) before the bias and the epilogue; with `swiglu`, `weight`
       is `interleave_gate_up(Wg, Wu)` and out = silu(gate) * up, bfloat16.
@@ -726,14 +730,15 @@ def linear_fused(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
             raise KernelError("linear_fused.norm_out: the product's own output must be float32")
         _need(out_g, "linear_fused.norm_out.g", torch.float32, (n,))
         _need(out_xg, "linear_fused.norm_out.xg", torch.bfloat16, (m, n))
-        _need(out_ssq, "linear_fused.norm_out.sums", torch.float32, (m, norm_sum_parts(n)))
+        _need(out_ssq, "linear_fused.norm_out.sums", torch.float32, (m, norm_sum_parts(n, m)))
     aligned = not (x.data_ptr() % 16 or weight.data_ptr() % 16 or k % 8)
     splits, per = _k_split(m, n, k, swiglu, aligned, tiled=tiled is not None)
     part = workspace("skinny", splits * m * n, x.device) if (splits > 1 or (swiglu and m > 16)) else None
     _need_tiled(tiled, "linear_fused.tiled", n, k)
     rc = _fn("gemm_bf16", "mf_gemm_bf16_skinny_fused")(
         _ptr(x), k, _ptr(weight), _ptr(tiled), k, _ptr(bias), _ptr(out), ldc, _ptr(part), m, n, k, splits, per, epi,
-        _ptr(in_ssq), in_parts, float(in_eps), _ptr(out_g), _ptr(out_xg), _ptr(out_ssq), _stream())
+        _ptr(in_ssq), in_parts, float(in_eps), _ptr(out_g), _ptr(out_xg), _ptr(out_ssq),
+        out_ssq.shape[1] if out_ssq is not None else 0, _stream())
     if rc == NOT_BUILT:
         return False
     _check(rc, f"gemm_bf16_skinny_fused{'(swiglu)' if swiglu else ''} {m}x{n}x{k}")

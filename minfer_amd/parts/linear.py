@@ -87,17 +87,19 @@ class Linear:
         """Runs the product with the next norm's input prepared beside it (bf16(out g) and the rows'
         partial sums of squares, left in `ctx.norm_ahead`) where the block has said which norm
         that is, the norm is of the RMS form and the product's kernels have a place for it (steps of
-        17 to 64 rows whose K is split over blocks).  False: nothing ran."""
+        17 to 64 rows whose K is split over blocks; steps of at most 16 rows in the one-kernel
+        forms).  False: nothing ran."""
         norm = getattr(ctx, "norm_next", None)
-        if norm is None or not 16 < x.shape[0] <= 64 or x.dtype != torch.bfloat16 or out.dtype != torch.float32:
+        if norm is None or not 0 < x.shape[0] <= 64 or x.dtype != torch.bfloat16 or out.dtype != torch.float32:
             return False
-        if tuning.NO_NORM_AHEAD:
+        if tuning.NO_NORM_AHEAD or x.device.type != "cuda":
             return False
         fold = norm.rms_scale()
         if fold is None or fold[0].numel() != self.out_features:
             return False
         xg = torch.empty(out.shape, dtype=torch.bfloat16, device=out.device)
-        sums = torch.empty((out.shape[0], ops.norm_sum_parts(self.out_features)), dtype=torch.float32, device=out.device)
+        sums = torch.empty((out.shape[0], ops.norm_sum_parts(self.out_features, out.shape[0])), dtype=torch.float32,
+                           device=out.device)
         if not ops.linear_fused(x, self.weight, self.bias, out, accumulate=accumulate, tiled=self.tiled,
                                 norm_out=(fold[0], xg, sums)):
             return False

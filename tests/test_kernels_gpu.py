@@ -796,45 +796,59 @@ def test_gemm_bf16_normed_declines(ops):
     assert torch.all(out == 7.0)
 
 
-# ------------------------------------------------------------------ the norm folded around the products of 17 to 64 rows
-@pytest.mark.parametrize("m,n,k", [(64, 3584, 3584), (20, 3584, 18944), (33, 5120, 5120), (17, 1000, 2048), (64, 3584 + 24, 3584)])
+# ------------------------------------------------------------------ the norm folded around the products of at most 64 rows
+@pytest.mark.parametrize("m,n,k", [(64, 3584, 3584), (20, 3584, 18944), (33, 5120, 5120), (17, 1000, 2048), (64, 3584 + 24, 3584),
+                                   (8, 3584, 3584), (16, 3584, 18944), (1, 3584, 18944), (5, 896, 4864), (13, 2048, 11008),
+                                   (8, 5120, 5120), (3, 1536, 1536)])
 def test_product_prepares_the_next_norm(ops, m, n, k):
     """A product that adds into the residual stream and leaves, for the norm that reads the stream
-    next, bf16(stream g) and the rows' sums of squares in runs of 256 columns: the stream itself is
-    what `linear` gives bit for bit, and what it leaves is what the stream's new rows say."""
+    next, bf16(stream g) and the rows' sums of squares in parts (runs of 256 columns from 17 rows on,
+    one part per workgroup of the one-kernel forms below that, the unused places zero): the stream
+    itself is what `linear` gives bit for bit, and what it leaves is what the stream's new rows say."""
     x, w, b = rnd((m, k), torch.bfloat16, 70), rnd((n, k), torch.bfloat16, 71, 0.05), rnd((n,), seed=72)
     g = (1.0 + rnd((n,), seed=73, scale=0.2)).to(DEV)
     base = rnd((m, n), seed=74, scale=3.0)
-    base[1, 7] = 50.0
+    base[m - 1, 7] = 50.0
     plain = base.to(DEV).clone()
     ops.linear(x.to(DEV), w.to(DEV), b.to(DEV), plain, accumulate=True)
     out = base.to(DEV).clone()
     xg = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
-    sums = torch.full((m, ops.norm_sum_parts(n)), float("nan"), device=DEV)
-    assert ops.linear_fused(x.to(DEV), w.to(DEV), b.to(DEV), out, accumulate=True, norm_out=(g, xg, sums))
+    sums = torch.full((m, ops.norm_sum_parts(n, m)), float("nan"), device=DEV)
+    tiled = ops.tile_weight(w.to(DEV)) if m <= 16 else None
+    assert ops.linear_fused(x.to(DEV), w.to(DEV), b.to(DEV), out, accumulate=True, norm_out=(g, xg, sums), tiled=tiled)
     assert torch.equal(out, plain)
     assert torch.equal(xg, (out * g).to(torch.bfloat16))
-    want = torch.nn.functional.pad(out.double() ** 2, (0, sums.shape[1] * 256 - n)).view(m, -1, 256).sum(-1)
-    close(sums, want.cpu(), 1e-6 * float(want.max()), 1e-5)
+    if m > 16:
+        want = torch.nn.functional.pad(out.double() ** 2, (0, sums.shape[1] * 256 - n)).view(m, -1, 256).sum(-1)
+        close(sums, want.cpu(), 1e-6 * float(want.max()), 1e-5)
+    else:
+        assert torch.isfinite(sums).all() and (sums >= 0).all()
+        want = (out.double() ** 2).sum(-1)
+        close(sums.double().sum(-1), want.cpu(), 1e-6 * float(want.max()), 1e-5)
     # twice the same bits
     xg2, sums2, out2 = torch.empty_like(xg), torch.empty_like(sums), base.to(DEV).clone()
-    assert ops.linear_fused(x.to(DEV), w.to(DEV), b.to(DEV), out2, accumulate=True, norm_out=(g, xg2, sums2))
+    assert ops.linear_fused(x.to(DEV), w.to(DEV), b.to(DEV), out2, accumulate=True, norm_out=(g, xg2, sums2), tiled=tiled)
     assert torch.equal(xg, xg2) and torch.equal(sums, sums2) and torch.equal(out, out2)
 
 
 @pytest.mark.parametrize("m,n,k,swiglu", [(64, 4608, 3584, False), (20, 37888, 3584, True), (40, 152064, 3584, False),
-                                          (33, 7168, 5120, False), (17, 1000, 2048, False), (64, 2200, 2048, True)])
+                                          (33, 7168, 5120, False), (17, 1000, 2048, False), (64, 2200, 2048, True),
+                                          (8, 4608, 3584, False), (16, 37888, 3584, True), (1, 152064, 3584, False),
+                                          (5, 1152, 896, False), (7, 9728, 896, True), (12, 7168, 5120, False),
+                                          (3, 22016, 2048, True)])
 def test_product_takes_a_prepared_norm(ops, m, n, k, swiglu):
     """The product behind the norm: its activations are bf16(x g), its sums are multiplied by each
     row's 1 / sqrt(sum of the partial sums / k + eps).  Against the formula in float64 with that one
     rounding, and against norm-then-product as the two kernels do it (the same size of error)."""
     h = rnd((m, k), seed=80, scale=3.0)
-    h[2, 11] = 45.0
+    h[min(2, m - 1), 11] = 45.0
     gw = 1.0 + rnd((k,), seed=81, scale=0.2)
     eps = 1e-5
     xg = (h * gw).to(torch.bfloat16).to(DEV)
     parts = ops.norm_sum_parts(k)
     sums = torch.nn.functional.pad(h.double() ** 2, (0, parts * 256 - k)).view(m, parts, 256).sum(-1).float().to(DEV)
+    if m <= 16:         # as a one-kernel product leaves them: a part per workgroup, zeros behind the last
+        sums = torch.nn.functional.pad(sums, (0, ops.norm_sum_parts(k, m) - parts))
     if swiglu:
         nf = n // 2
         wg, wu = rnd((nf, k), torch.bfloat16, 82, 0.05), rnd((nf, k), torch.bfloat16, 83, 0.05)
@@ -864,12 +878,13 @@ def test_product_takes_a_prepared_norm(ops, m, n, k, swiglu):
 
 
 def test_fused_norm_declines_where_no_kernel_has_a_place_for_it(ops):
-    """At most 16 rows in one kernel, or a K that is not split: nothing is written, the caller is told."""
-    for m, n, k in ((8, 3584, 3584), (20, 300, 200), (64, 64, 256)):
+    """A K that is not split at 17 rows and more, a shape of few rows that the register-resident
+    kernel does not take: nothing is written, the caller is told."""
+    for m, n, k in ((8, 300, 200), (20, 300, 200), (64, 64, 256)):
         x, w = rnd((m, k), torch.bfloat16, 90).to(DEV), rnd((n, k), torch.bfloat16, 91).to(DEV)
         out = torch.full((m, n), 7.0, device=DEV)
         xg = torch.full((m, n), 3.0, dtype=torch.bfloat16, device=DEV)
-        sums = torch.full((m, ops.norm_sum_parts(n)), 5.0, device=DEV)
+        sums = torch.full((m, ops.norm_sum_parts(n, m)), 5.0, device=DEV)
         g = torch.ones(n, device=DEV)
         assert not ops.linear_fused(x, w, None, out, accumulate=True, norm_out=(g, xg, sums))
         s_in = torch.ones((m, ops.norm_sum_parts(k)), device=DEV)

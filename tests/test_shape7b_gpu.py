@@ -111,7 +111,8 @@ def test_batch_of_forty_through_four_layers(folder4):
     """Forty short requests through four layers: steps of 17 to 64 rows, where the norms are folded
     around the products (the product that adds into the stream prepares the next norm's input, the
     product behind the norm applies the rows' factors), from one layer to the next and into the
-    final norm; then the batch thins out into the steps of at most 16 rows."""
+    final norm; then the batch thins out into the steps of at most 16 rows, where the one-kernel
+    products do the same between them (the reading product then takes its activations in bfloat16)."""
     from minfer_amd import Engine, load_model
     from minfer_amd.kernels import ops
     plain = PlainQwen2.from_folder(folder4, dtype=np.float64)
@@ -129,7 +130,8 @@ def test_batch_of_forty_through_four_layers(folder4):
     finally:
         ops.linear_fused = real
     took = [c for c in calls if c[2]]
-    assert any(c[1] for c in took) and any(not c[1] for c in took), "both sides of the fold ran"
+    for rows in (lambda m: m > 16, lambda m: m <= 16):        # the K-split kernels' fold, and the one-kernel forms'
+        assert any(c[1] for c in took if rows(c[0])) and any(not c[1] for c in took if rows(c[0])), "both sides of the fold ran"
     print(f"worst abs err {worst:.3e}; {len(took)} of {len(calls)} fused calls ran")
 
 
