@@ -670,6 +670,14 @@ def linear_normed(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, row_id
 NORM_SUM_RUN = 256       # columns a partial sum of squares covers (a block of the kernel that adds a K split's parts)
 
 
+# Steps of at most 16 rows prepare the next norm in a product's epilogue only for rows of this many
+# values: measured at batch 8 (a decode step with it against without), width 896: 10 % slower (the
+# reading product waits for the rows' sums, a trip to memory, where the whole kernel is 7 us), 1536
+# and 2048: 0.5 % slower, 3584: 0.7 % faster (2.4 % at batch 1), 5120: 4.5 % faster; from 5121 on
+# the register-resident product has no form that reads bfloat16 activations.
+NORM_AHEAD_16_WIDTHS = (3072, 5120)
+
+
 def norm_sum_parts(n: int, m: int = 64) -> int:
     """Partial sums of squares a row of `n` values comes with from a product of `m` rows (see
     `linear_fused`): one per run of 256 columns from 17 rows on (the kernel that adds the parts of a K

@@ -94,6 +94,9 @@ class Linear:
             return False
         if tuning.NO_NORM_AHEAD or x.device.type != "cuda":
             return False
+        lo, hi = ops.NORM_AHEAD_16_WIDTHS
+        if x.shape[0] <= 16 and not lo <= self.out_features <= hi:
+            return False
         fold = norm.rms_scale()
         if fold is None or fold[0].numel() != self.out_features:
             return False
