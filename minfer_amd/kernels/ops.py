@@ -682,7 +682,8 @@ def norm_sum_parts(n: int, m: int = 64) -> int:
     """Partial sums of squares a row of `n` values comes with from a product of `m` rows (see
     `linear_fused`): one per run of 256 columns from 17 rows on (the kernel that adds the parts of a K
     split writes them), one per workgroup of the product's one kernel for at most 16 rows."""
-    return cu_count() if m <= 16 else (n + NORM_SUM_RUN - 1) // NORM_SUM_RUN
+    runs = (n + NORM_SUM_RUN - 1) // NORM_SUM_RUN
+    return max(cu_count(), runs) if m <= 16 else runs
 
 
 def linear_fused(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
